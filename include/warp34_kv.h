@@ -1,0 +1,216 @@
+/*
+ * warp34_kv.h -- C ABI of the MI355X (gfx950) KV-cache hot path.
+ *
+ * This is the drop-in boundary: the descriptor structs, enum values, symbol names,
+ * argument lists and the int error convention are those of the reference's kernel
+ * crate for this path, so warp34-host binds to libwarp34_kernels built from this
+ * repository without source changes:
+ *
+ *   reference C header : crates/warp34-kernels/csrc/warp34_cuda.h:20-44   (enums)
+ *                        crates/warp34-kernels/csrc/warp34_cuda.h:50-101  (structs)
+ *                        crates/warp34-kernels/csrc/warp34_cuda.h:142-164 (runtime shims)
+ *                        crates/warp34-kernels/csrc/warp34_cuda.h:353-373 (KV write + attention)
+ *   reference Rust view: crates/warp34-kernels/src/ffi.rs:6-90,701-760
+ *
+ * Conventions (all entry points):
+ *   - return 0 on success; a positive value is a hipError_t; nothing is synchronised
+ *     inside a call, all work is enqueued on ex->stream and is stream-capturable;
+ *   - the caller owns every buffer; the library allocates nothing.  Temporary space
+ *     comes only from ex->scratch_ptr / ex->scratch_size.  When the scratch is null,
+ *     misaligned (16 B) or too small the attention calls run a single-pass kernel and
+ *     do not touch it;
+ *   - every index array in warp34_attention_batch is a DEVICE pointer; the scalar
+ *     fields max_q_len / max_seq_len / max_blocks_per_req are host-known upper bounds
+ *     used only for launch geometry -- results do not depend on them;
+ *   - masked tokens / requests (valid_token_mask[tok]==0, valid_req_mask[req]==0,
+ *     write slot < 0) write nothing and leave the output row untouched.
+ */
+#ifndef WARP34_KV_H
+#define WARP34_KV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* warp34_cuda.h:20-24 */
+enum {
+    WARP34_KV_NAMESPACE_TARGET_FULL_ATTN = 0,
+    WARP34_KV_NAMESPACE_MTP_FULL_ATTN    = 1,
+    WARP34_KV_NAMESPACE_DFLASH_DRAFT_CTX = 2,
+};
+
+/* warp34_cuda.h:26-32 */
+enum {
+    WARP34_KV_FORMAT_FP16     = 0, /* 2 B / element                                   */
+    WARP34_KV_FORMAT_BF16     = 1, /* 2 B / element                                   */
+    WARP34_KV_FORMAT_TQ4      = 2, /* 66 B per 128 elements: fp16 scale + 64 B nibbles */
+    WARP34_KV_FORMAT_Q8_0     = 3, /* 68 B per 64 elements  (not built yet)           */
+    WARP34_KV_FORMAT_FP8_E4M3 = 4, /* 264 B per 256 elements (not built yet)          */
+};
+
+/* warp34_cuda.h:34-37 */
+enum {
+    WARP34_KV_TRANSFORM_IDENTITY          = 0,
+    WARP34_KV_TRANSFORM_RADEMACHER_WHT256 = 1,
+};
+
+/* warp34_cuda.h:39-44 */
+enum {
+    WARP34_ATTN_MASK_CAUSAL           = 0,
+    WARP34_ATTN_MASK_SYMMETRIC_WINDOW = 1, /* legacy name */
+    WARP34_ATTN_MASK_NONCAUSAL_WINDOW = 1,
+};
+
+/* warp34_cuda.h:50-57 -- 32 bytes */
+typedef struct {
+    uintptr_t stream;       /* hipStream_t */
+    uint64_t  scratch_ptr;  /* device workspace, may be 0 */
+    size_t    scratch_size; /* bytes */
+    uint64_t  flags;
+} warp34_exec;
+
+/* warp34_cuda.h:59-80 -- 104 bytes */
+typedef struct {
+    uint64_t k_base;
+    uint64_t v_base;
+    uint64_t k_page_stride_bytes;
+    uint64_t k_head_stride_bytes;
+    uint64_t k_token_stride_bytes;
+    uint64_t v_page_stride_bytes;
+    uint64_t v_head_stride_bytes;
+    uint64_t v_token_stride_bytes;
+    int32_t  namespace_id;
+    int32_t  layer_id;
+    int32_t  local_kv_heads;
+    int32_t  head_dim;
+    int32_t  block_size;
+    int32_t  k_format;
+    int32_t  v_format;
+    int32_t  k_transform;
+    int32_t  v_transform;
+    int32_t  reserved;
+} warp34_kv_layer_layout;
+
+/* warp34_cuda.h:82-101 -- 96 bytes */
+typedef struct {
+    const int32_t* query_start_loc;     /* [num_reqs + 1] */
+    const int32_t* context_lens_before; /* [num_reqs] or NULL (= seq_lens_after - q_len) */
+    const int32_t* seq_lens_after;      /* [num_reqs] */
+    const int32_t* block_tables;        /* [num_reqs, max_blocks_per_req] physical page ids */
+    const int32_t* write_slot_mapping;  /* [total_tokens] page*block_size + offset, <0 = skip */
+    const uint8_t* valid_token_mask;    /* [total_tokens] or NULL */
+    const uint8_t* valid_req_mask;      /* [num_reqs] or NULL */
+    int32_t        num_reqs;
+    int32_t        total_tokens;
+    int32_t        max_blocks_per_req;
+    int32_t        max_q_len;
+    int32_t        max_seq_len;
+    int32_t        mask_mode;
+    int32_t        sliding_window;
+    float          sm_scale;
+    int32_t        reserved;
+} warp34_attention_batch;
+
+#if defined(__cplusplus)
+static_assert(sizeof(warp34_exec) == 32, "warp34_exec ABI size");
+static_assert(sizeof(warp34_kv_layer_layout) == 104, "warp34_kv_layer_layout ABI size");
+static_assert(sizeof(warp34_attention_batch) == 96, "warp34_attention_batch ABI size");
+#else
+_Static_assert(sizeof(warp34_exec) == 32, "warp34_exec ABI size");
+_Static_assert(sizeof(warp34_kv_layer_layout) == 104, "warp34_kv_layer_layout ABI size");
+_Static_assert(sizeof(warp34_attention_batch) == 96, "warp34_attention_batch ABI size");
+#endif
+
+/* ------------------------------------------------------------------------------------
+ * Quantize-on-append (replaces op_kv_cache.cu:325-368,828-858).
+ *
+ * k_in / v_in: [total_tokens, row_stride] fp16 elements, head h of token t at
+ * t*row_stride + h*head_dim.  Row strides are in ELEMENTS and must be
+ * >= local_kv_heads*head_dim.  Destination row:
+ *   base + (slot / block_size)*page_stride + head*head_stride + (slot % block_size)*token_stride.
+ * Formats built: FP16, BF16 (converted from fp16), TQ4 (head_dim 256 + WHT256 transform).
+ * TQ4 rows are bit-exact with the declared-numerics CPU restatement of
+ * op_kv_cache.cu:152-218.
+ * ------------------------------------------------------------------------------------ */
+int warp34_kv_cache_write(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
+                          const warp34_attention_batch* batch,
+                          const void* k_in, const void* v_in);               /* warp34_cuda.h:353-355 */
+int warp34_kv_cache_write_strided(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
+                                  const warp34_attention_batch* batch,
+                                  const void* k_in, const void* v_in,
+                                  int k_row_stride, int v_row_stride);       /* warp34_cuda.h:356-359 */
+
+/* bf16 source rows (replaces op_kv_cache.cu:798-824,1172-1190).  The reference accepts
+ * only BF16-format identity layouts here; this library additionally accepts TQ4+WHT256
+ * layouts at head_dim 256 (bf16 -> fp32 is exact, the encode is the same arithmetic). */
+int warp34_kv_cache_write_bf16(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
+                               const warp34_attention_batch* batch,
+                               const void* k_in, const void* v_in);          /* warp34_cuda.h:362-363 */
+int warp34_kv_cache_write_strided_bf16(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
+                                       const warp34_attention_batch* batch,
+                                       const void* k_in, const void* v_in,
+                                       int row_stride_elems);                /* warp34_cuda.h:364-365 */
+
+/* ------------------------------------------------------------------------------------
+ * Paged GQA attention (replaces op_paged_attn.cu:1266-1448 and op_kv_cache.cu:1192-1241).
+ *
+ * q_in / attn_out: [total_tokens, num_q_heads, head_dim] contiguous, fp16 for _f16 and
+ * bf16 for _bf16.  kv_head = q_head / (num_q_heads / local_kv_heads).  Visible keys of
+ * token t of request r: [min_kv, max_kv] with
+ *   max_kv = (mask_mode == NONCAUSAL_WINDOW ? seq_after-1 : ctx_before + q_off), clamped to seq_after-1
+ *   min_kv = sliding_window > 0 ? max(0, ctx_before + q_off - sliding_window + 1) : 0
+ * Output = softmax(sm_scale * q.K^T) V in fp32 accumulation; an empty key range gives zeros.
+ * _f16 accepts FP16 and TQ4+WHT256 layouts; _bf16 accepts BF16 (reference) and,
+ * additionally, TQ4+WHT256 layouts.  head_dim must be 256 and block_size a multiple of 16.
+ * ------------------------------------------------------------------------------------ */
+int warp34_paged_attention_f16(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
+                               const warp34_attention_batch* batch,
+                               const void* q_in, void* attn_out, int num_q_heads);  /* warp34_cuda.h:369-372 */
+int warp34_paged_attention_bf16(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
+                                const warp34_attention_batch* batch,
+                                const void* q_in, void* attn_out, int num_q_heads); /* warp34_cuda.h:366-367 */
+
+/* Test-only kernel selector (op_paged_attn.cu:1451-1519): 0 = split-K decode/verify kernel
+ * run as a single pass, 1 / 2 = the multi-row MFMA tile kernel.  All selections compute
+ * the same function. */
+int warp34_paged_attention_f16_force_kernel_for_test(
+    const warp34_exec* ex, const warp34_kv_layer_layout* layout,
+    const warp34_attention_batch* batch,
+    const void* q_in, void* attn_out, int num_q_heads, int use_64q);
+
+/* Bytes of scratch the attention entry points can make use of for a batch of this shape
+ * (split-K partials).  No counterpart in the reference, whose engine simply guarantees
+ * >= 8 MiB (op_paged_attn.cu:1301-1304); provided so a host can size ex->scratch. */
+size_t warp34_paged_attention_scratch_bytes(int total_tokens, int num_q_heads, int max_seq_len);
+
+/* ------------------------------------------------------------------------------------
+ * Runtime shims a standalone harness needs (replace op_init.cu; warp34_cuda.h:135,142-164).
+ * ------------------------------------------------------------------------------------ */
+const char* warp34_cuda_error_string(int code);
+int warp34_get_device_count(int* out_count);
+int warp34_set_device(int device_id);
+int warp34_device_synchronize(void);
+int warp34_get_mem_info(size_t* out_free, size_t* out_total);
+int warp34_malloc(void** out_ptr, size_t bytes);
+int warp34_free(void* ptr);
+int warp34_memcpy_h2d_async(void* dst, const void* src, size_t bytes, uintptr_t stream);
+int warp34_memcpy_d2h_async(void* dst, const void* src, size_t bytes, uintptr_t stream);
+int warp34_memcpy_d2d_async(void* dst, const void* src, size_t bytes, uintptr_t stream);
+int warp34_memset_async(void* dst, int value, size_t bytes, uintptr_t stream);
+int warp34_stream_create(uintptr_t* out_stream);
+int warp34_stream_destroy(uintptr_t stream);
+int warp34_stream_synchronize(uintptr_t stream);
+int warp34_event_create(uintptr_t* out_event, int enable_timing);
+int warp34_event_destroy(uintptr_t event);
+int warp34_event_record(uintptr_t event, uintptr_t stream);
+int warp34_stream_wait_event(uintptr_t stream, uintptr_t event);
+int warp34_event_synchronize(uintptr_t event);
+int warp34_event_elapsed_ms(float* out_ms, uintptr_t start_event, uintptr_t end_event);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WARP34_KV_H */

@@ -1,0 +1,655 @@
+/*
+ * tq4_oracle.c -- CPU restatement of the reference's TQ4 quantize-on-append, paged
+ * layout addressing and paged GQA attention.  TEST INFRASTRUCTURE ONLY (see tq4_oracle.h
+ * for the declared numerics and for what pins each function).
+ *
+ * Build: gcc -O2 -std=c99 -ffp-contract=off -fno-fast-math -fPIC -shared -pthread
+ */
+#define _GNU_SOURCE
+#include "tq4_oracle.h"
+
+#include <math.h>
+#include <pthread.h>
+#include <stdlib.h>
+#include <string.h>
+#include <unistd.h>
+
+/* ---- tables: csrc/tq/tq4_codebook.cuh:46-101 (numeric literals are the contract) ---- */
+static const float kCentroids[16] = {
+    -1.694104124e-1f, -1.285881878e-1f, -1.006979993e-1f, -7.824930800e-2f,
+    -5.873210384e-2f, -4.094919437e-2f, -2.420087619e-2f, -8.008373692e-3f,
+    8.008373692e-3f,  2.420087619e-2f,  4.094919437e-2f,  5.873210384e-2f,
+    7.824930800e-2f,  1.006979993e-1f,  1.285881878e-1f,  1.694104124e-1f,
+};
+static const float kBoundaries[15] = {
+    -1.489993001e-1f, -1.146430936e-1f, -8.947365365e-2f, -6.849070592e-2f,
+    -4.984064910e-2f, -3.257503528e-2f, -1.610462494e-2f, 0.000000000e0f,
+    1.610462494e-2f,  3.257503528e-2f,  4.984064910e-2f,  6.849070592e-2f,
+    8.947365365e-2f,  1.146430936e-1f,  1.489993001e-1f,
+};
+/* Seed-42 Rademacher diagonal, bit i set <=> sign[i] = -1 (little-endian 64-bit words). */
+static const uint64_t kSignMask[4] = {
+    0x4897475229e1d357ull, 0xf1297e2aeebc0de4ull, 0xe2eb25d0ba639274ull, 0x36b5bda1fde0ee14ull,
+};
+static float g_signs[256];
+static pthread_once_t g_once = PTHREAD_ONCE_INIT;
+static void init_tables(void) {
+    for (int i = 0; i < 256; ++i)
+        g_signs[i] = ((kSignMask[i >> 6] >> (i & 63)) & 1ull) ? -1.0f : 1.0f;
+}
+const float* tq4o_centroids256(void) { return kCentroids; }
+const float* tq4o_boundaries256(void) { return kBoundaries; }
+const float* tq4o_signs256(void) {
+    pthread_once(&g_once, init_tables);
+    return g_signs;
+}
+
+/* ---- 16-bit float conversions, round to nearest even ---- */
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+float tq4o_f16_to_f32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1Fu;
+    uint32_t man = h & 0x3FFu;
+    if (exp == 0) {
+        if (man == 0) return u2f(sign);
+        /* subnormal: value = man * 2^-24 */
+        float v = (float)man * 5.9604644775390625e-8f;
+        return sign ? -v : v;
+    }
+    if (exp == 31) return u2f(sign | 0x7F800000u | (man << 13));
+    return u2f(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+uint16_t tq4o_f32_to_f16(float f) {
+    uint32_t x = f2u(f);
+    uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+    uint32_t ax = x & 0x7FFFFFFFu;
+    if (ax >= 0x7F800000u) /* inf / nan */
+        return (uint16_t)(sign | 0x7C00u | ((ax > 0x7F800000u) ? 0x200u : 0u));
+    if (ax >= 0x477FF000u) /* >= 65520 rounds to inf */
+        return (uint16_t)(sign | 0x7C00u);
+    if (ax < 0x38800000u) { /* below the smallest normal half: subnormal or zero */
+        if (ax < 0x33000000u) return sign; /* < 2^-25 rounds to zero (2^-25 itself ties to even = 0) */
+        uint32_t e = ax >> 23;                       /* biased fp32 exponent, 102..112 */
+        uint32_t m = (ax & 0x7FFFFFu) | 0x800000u;   /* 24-bit significand */
+        uint32_t shift = 126u - e;                   /* 14..24: result = m >> shift in units of 2^-24 */
+        uint32_t q = m >> shift;
+        uint32_t rem = m & ((1u << shift) - 1u);
+        uint32_t half = 1u << (shift - 1u);
+        if (rem > half || (rem == half && (q & 1u))) q++;
+        return (uint16_t)(sign | q);
+    }
+    uint32_t e = (ax >> 23) - 112u;
+    uint32_t m = ax & 0x7FFFFFu;
+    uint32_t q = (e << 10) | (m >> 13);
+    uint32_t rem = m & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (q & 1u))) q++;
+    return (uint16_t)(sign | q);
+}
+
+float tq4o_bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+
+uint16_t tq4o_f32_to_bf16(float f) {
+    uint32_t x = f2u(f);
+    if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((x >> 16) | 0x40u);
+    uint32_t lsb = (x >> 16) & 1u;
+    x += 0x7FFFu + lsb;
+    return (uint16_t)(x >> 16);
+}
+
+static inline float load16(const uint16_t* p, int dtype) {
+    return dtype == TQ4O_DT_BF16 ? tq4o_bf16_to_f32(*p) : tq4o_f16_to_f32(*p);
+}
+
+/* ---- WHT-256: csrc/tq/tq4_kv_common.cuh:75-107.
+ * Butterfly stages over index bits 0..7 in that order; the element with the bit clear
+ * becomes a+b, the one with the bit set a-b (a = bit-clear element); the last stage
+ * multiplies both results by 1/16. ---- */
+void tq4o_wht256(float* x) {
+    for (int h = 1; h < 256; h <<= 1) {
+        for (int i = 0; i < 256; ++i) {
+            if (i & h) continue;
+            float a = x[i], b = x[i | h];
+            if (h == 128) {
+                x[i] = (a + b) * 0.0625f;
+                x[i | h] = (a - b) * 0.0625f;
+            } else {
+                x[i] = a + b;
+                x[i | h] = a - b;
+            }
+        }
+    }
+}
+
+/* 32-lane xor-butterfly sum, csrc/tq/tq4_kv_common.cuh:54-60 */
+static float warp_sum32(const float* lane_vals) {
+    float cur[32], nxt[32];
+    memcpy(cur, lane_vals, sizeof(cur));
+    for (int off = 16; off > 0; off >>= 1) {
+        for (int l = 0; l < 32; ++l) nxt[l] = cur[l] + cur[l ^ off];
+        memcpy(cur, nxt, sizeof(cur));
+    }
+    return cur[0];
+}
+
+/* ---- TQ4 encode: op_kv_cache.cu:152-218.  Element i lives in lane i%32, register i/32. ---- */
+void tq4o_encode_row(const float* x, uint8_t* dst) {
+    const float* sg = tq4o_signs256();
+    float y[256];
+    for (int i = 0; i < 256; ++i) y[i] = x[i] * sg[i]; /* :163-167 */
+    tq4o_wht256(y);                                    /* :168 */
+
+    float tmp[32];
+    float s_sq[2] = {0.0f, 0.0f};
+    for (int j = 0; j < 4; ++j) { /* :170-175 */
+        for (int l = 0; l < 32; ++l) tmp[l] = y[l + 32 * j] * y[l + 32 * j];
+        s_sq[0] += warp_sum32(tmp);
+        for (int l = 0; l < 32; ++l) tmp[l] = y[l + 32 * (j + 4)] * y[l + 32 * (j + 4)];
+        s_sq[1] += warp_sum32(tmp);
+    }
+    float inv_norm[2];
+    for (int h = 0; h < 2; ++h) { /* :176-179 */
+        float rs = (float)(1.0 / sqrt((double)s_sq[h]));
+        inv_norm[h] = (s_sq[h] > 1e-20f) ? (0.7071067811865475f * rs) : 0.0f;
+    }
+
+    uint8_t code[256];
+    float vc_dot[2] = {0.0f, 0.0f}, c_sq[2] = {0.0f, 0.0f};
+    for (int j = 0; j < 8; ++j) { /* :184-209 */
+        float vc[32], cc[32];
+        for (int l = 0; l < 32; ++l) {
+            const int i = l + 32 * j;
+            const float rv = y[i] * inv_norm[j >> 2];
+            int q = 0;
+            for (int t = 0; t < 15; ++t) q += (rv > kBoundaries[t]) ? 1 : 0;
+            code[i] = (uint8_t)q;
+            const float c = kCentroids[q];
+            vc[l] = y[i] * c;
+            cc[l] = c * c;
+        }
+        vc_dot[j >> 2] += warp_sum32(vc);
+        c_sq[j >> 2] += warp_sum32(cc);
+    }
+    for (int h = 0; h < 2; ++h) { /* :193-198 pack, :210-215 scale */
+        uint8_t* blk = dst + 66 * h;
+        const float d = (c_sq[h] > 1e-10f) ? (vc_dot[h] / c_sq[h]) : 0.0f;
+        const uint16_t dh = tq4o_f32_to_f16(d);
+        blk[0] = (uint8_t)(dh & 0xFF);
+        blk[1] = (uint8_t)(dh >> 8);
+        for (int m = 0; m < 64; ++m)
+            blk[2 + m] = (uint8_t)(code[128 * h + 2 * m] | (code[128 * h + 2 * m + 1] << 4));
+    }
+}
+
+/* ---- TQ4 dequant: op_kv_cache.cu:298-306 ---- */
+void tq4o_dequant_row(const uint8_t* src, float* y) {
+    for (int col = 0; col < 256; ++col) {
+        const int sb = col >> 7, idx = col & 127;
+        const uint8_t* blk = src + 66 * sb;
+        const float d = tq4o_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        const uint8_t packed = blk[2 + (idx >> 1)];
+        const uint8_t nib = (idx & 1) ? (uint8_t)(packed >> 4) : (uint8_t)(packed & 0x0F);
+        y[col] = d * kCentroids[nib];
+    }
+}
+
+void tq4o_unrotate_row(const float* y, float* x) {
+    const float* sg = tq4o_signs256();
+    float t[256];
+    memcpy(t, y, sizeof(t));
+    tq4o_wht256(t);
+    for (int i = 0; i < 256; ++i) x[i] = t[i] * sg[i];
+}
+
+/* ---- request lookup shared by write and attention: op_kv_cache.cu:385-398 ---- */
+static int find_req(const tq4o_batch* B, int tok, int* q_start, int* q_end) {
+    for (int r = 0; r < B->num_reqs; ++r) {
+        const int lo = B->query_start_loc[r], hi = B->query_start_loc[r + 1];
+        if (tok >= lo && tok < hi) {
+            *q_start = lo;
+            *q_end = hi;
+            return r;
+        }
+    }
+    return -1;
+}
+
+static int write_row(uint8_t* dst, int format, int transform, const uint16_t* src, int head_dim,
+                     int in_dtype) {
+    if (format == TQ4O_FMT_FP16 || format == TQ4O_FMT_BF16) { /* op_kv_cache.cu:18-31 */
+        uint16_t* d16 = (uint16_t*)dst;
+        for (int c = 0; c < head_dim; ++c) {
+            const int same = (format == TQ4O_FMT_FP16 && in_dtype == TQ4O_DT_F16) ||
+                             (format == TQ4O_FMT_BF16 && in_dtype == TQ4O_DT_BF16);
+            if (same) {
+                d16[c] = src[c];
+            } else {
+                const float f = load16(src + c, in_dtype);
+                d16[c] = format == TQ4O_FMT_BF16 ? tq4o_f32_to_bf16(f) : tq4o_f32_to_f16(f);
+            }
+        }
+        return 0;
+    }
+    if (format == TQ4O_FMT_TQ4 && transform == TQ4O_XF_WHT256 && head_dim == 256) {
+        float x[256];
+        for (int c = 0; c < 256; ++c) x[c] = load16(src + c, in_dtype);
+        tq4o_encode_row(x, dst);
+        return 0;
+    }
+    return -1;
+}
+
+/* ---- paged append: op_kv_cache.cu:325-368 ---- */
+int tq4o_kv_cache_write(const tq4o_layout* L, const tq4o_batch* B, const uint16_t* k_in,
+                        const uint16_t* v_in, int k_row_stride, int v_row_stride, int in_dtype) {
+    for (int tok = 0; tok < B->total_tokens; ++tok) {
+        if (B->valid_token_mask && B->valid_token_mask[tok] == 0) continue;
+        if (B->valid_req_mask && B->query_start_loc && B->num_reqs > 0) {
+            int a, b;
+            const int r = find_req(B, tok, &a, &b);
+            if (r < 0 || B->valid_req_mask[r] == 0) continue;
+        }
+        const int32_t slot = B->write_slot_mapping[tok];
+        if (slot < 0) continue;
+        const int page = slot / L->block_size, off = slot % L->block_size;
+        for (int h = 0; h < L->local_kv_heads; ++h) {
+            uint8_t* kd = L->k_base + (size_t)page * L->k_page_stride + (size_t)h * L->k_head_stride +
+                          (size_t)off * L->k_token_stride;
+            uint8_t* vd = L->v_base + (size_t)page * L->v_page_stride + (size_t)h * L->v_head_stride +
+                          (size_t)off * L->v_token_stride;
+            const uint16_t* ks = k_in + (size_t)tok * k_row_stride + (size_t)h * L->head_dim;
+            const uint16_t* vs = v_in + (size_t)tok * v_row_stride + (size_t)h * L->head_dim;
+            if (write_row(kd, L->k_format, L->k_transform, ks, L->head_dim, in_dtype)) return -1;
+            if (write_row(vd, L->v_format, L->v_transform, vs, L->head_dim, in_dtype)) return -1;
+        }
+    }
+    return 0;
+}
+
+/* read one stored row as fp32 (op_kv_cache.cu:288-306) */
+static void read_row(const uint8_t* row, int format, int head_dim, float* y) {
+    if (format == TQ4O_FMT_TQ4) {
+        tq4o_dequant_row(row, y);
+        return;
+    }
+    const uint16_t* p = (const uint16_t*)row;
+    for (int c = 0; c < head_dim; ++c)
+        y[c] = format == TQ4O_FMT_BF16 ? tq4o_bf16_to_f32(p[c]) : tq4o_f16_to_f32(p[c]);
+}
+
+/* Visible key range of one query token: op_kv_cache.cu:406-424.  Returns 0 when the row
+ * is skipped (masked / no owning request). */
+static int row_range(const tq4o_batch* B, int tok, int* req, int* min_kv, int* max_kv) {
+    if (B->valid_token_mask && B->valid_token_mask[tok] == 0) return 0;
+    int q_start = 0, q_end = 0;
+    const int r = find_req(B, tok, &q_start, &q_end);
+    if (r < 0) return 0;
+    if (B->valid_req_mask && B->valid_req_mask[r] == 0) return 0;
+    const int q_off = tok - q_start;
+    const int ctx_before = B->context_lens_before ? B->context_lens_before[r]
+                                                  : (B->seq_lens_after[r] - (q_end - q_start));
+    const int seq_after = B->seq_lens_after[r];
+    int mx = (B->mask_mode == 1) ? (seq_after - 1) : (ctx_before + q_off);
+    if (mx >= seq_after) mx = seq_after - 1;
+    int mn = 0;
+    if (B->sliding_window > 0) {
+        const int ws = ctx_before + q_off - B->sliding_window + 1;
+        if (ws > mn) mn = ws;
+    }
+    *req = r;
+    *min_kv = mn;
+    *max_kv = mx;
+    return 1;
+}
+
+static inline const uint8_t* kv_row_ptr(const uint8_t* base, uint64_t ps, uint64_t hs, uint64_t ts,
+                                        const tq4o_batch* B, int req, int kv_head, int pos, int bs) {
+    const int32_t page = B->block_tables[(size_t)req * B->max_blocks_per_req + pos / bs];
+    return base + (size_t)page * ps + (size_t)kv_head * hs + (size_t)(pos % bs) * ts;
+}
+
+/* Partial softmax state of `g` query heads of one kv head over keys [lo, hi]:
+ * acc[g][head_dim] un-normalised, m[g] running max, l[g] sum of exp(score - m).
+ * fp64 throughout (declared oracle numerics). */
+static void attend_range(const tq4o_layout* L, const tq4o_batch* B, int req, int kv_head,
+                         const float* qrows /* [g][hd], already rotated */, int g, int lo, int hi,
+                         double* acc, double* m, double* l) {
+    const int hd = L->head_dim;
+    const int n = hi - lo + 1;
+    float kv[256];
+    double* sc = (double*)malloc((size_t)g * (size_t)(n > 0 ? n : 1) * sizeof(double));
+    for (int a = 0; a < g; ++a) {
+        m[a] = -INFINITY;
+        l[a] = 0.0;
+        for (int c = 0; c < hd; ++c) acc[(size_t)a * hd + c] = 0.0;
+    }
+    for (int pos = lo; pos <= hi; ++pos) {
+        read_row(kv_row_ptr(L->k_base, L->k_page_stride, L->k_head_stride, L->k_token_stride, B, req,
+                            kv_head, pos, L->block_size),
+                 L->k_format, hd, kv);
+        for (int a = 0; a < g; ++a) {
+            const float* q = qrows + (size_t)a * hd;
+            double dot = 0.0;
+            for (int c = 0; c < hd; ++c) dot += (double)q[c] * (double)kv[c];
+            const double s = dot * (double)B->sm_scale;
+            sc[(size_t)a * n + (pos - lo)] = s;
+            if (s > m[a]) m[a] = s;
+        }
+    }
+    for (int a = 0; a < g; ++a)
+        for (int i = 0; i < n; ++i) {
+            const double p = exp(sc[(size_t)a * n + i] - m[a]);
+            sc[(size_t)a * n + i] = p;
+            l[a] += p;
+        }
+    for (int pos = lo; pos <= hi; ++pos) {
+        read_row(kv_row_ptr(L->v_base, L->v_page_stride, L->v_head_stride, L->v_token_stride, B, req,
+                            kv_head, pos, L->block_size),
+                 L->v_format, hd, kv);
+        for (int a = 0; a < g; ++a) {
+            const double p = sc[(size_t)a * n + (pos - lo)];
+            double* ac = acc + (size_t)a * hd;
+            for (int c = 0; c < hd; ++c) ac[c] += p * (double)kv[c];
+        }
+    }
+    free(sc);
+}
+
+/* load + optionally rotate the query rows of one (token, kv head): op_kv_cache.cu:435-451 */
+static void load_q(const tq4o_layout* L, const uint16_t* q, int q_dtype, int tok, int num_q_heads,
+                   int q_head0, int g, float* qrows) {
+    const int hd = L->head_dim;
+    const float* sg = tq4o_signs256();
+    for (int a = 0; a < g; ++a) {
+        const uint16_t* src = q + ((size_t)tok * num_q_heads + q_head0 + a) * hd;
+        float* dst = qrows + (size_t)a * hd;
+        for (int c = 0; c < hd; ++c) dst[c] = load16(src + c, q_dtype);
+        if (hd == 256 && L->k_transform == TQ4O_XF_WHT256) {
+            for (int c = 0; c < 256; ++c) dst[c] *= sg[c];
+            tq4o_wht256(dst);
+        }
+    }
+}
+
+/* finalise one row: normalise, un-rotate (op_kv_cache.cu:762-790) */
+static void store_out(const tq4o_layout* L, const double* acc, double l, float* out_row) {
+    const int hd = L->head_dim;
+    float t[256];
+    const double inv = l > 0.0 ? 1.0 / l : 0.0;
+    for (int c = 0; c < hd; ++c) t[c] = (float)(acc[c] * inv);
+    if (hd == 256 && L->v_transform == TQ4O_XF_WHT256)
+        tq4o_unrotate_row(t, out_row);
+    else
+        memcpy(out_row, t, (size_t)hd * sizeof(float));
+}
+
+/* merge chunk states in chunk order (fp64) */
+static void merge_state(double* acc, double* m, double* l, const double* acc2, double m2, double l2,
+                        int hd) {
+    if (l2 <= 0.0) return;
+    if (*l <= 0.0) {
+        memcpy(acc, acc2, (size_t)hd * sizeof(double));
+        *m = m2;
+        *l = l2;
+        return;
+    }
+    const double mt = *m > m2 ? *m : m2;
+    const double w1 = exp(*m - mt), w2 = exp(m2 - mt);
+    for (int c = 0; c < hd; ++c) acc[c] = acc[c] * w1 + acc2[c] * w2;
+    *l = *l * w1 + l2 * w2;
+    *m = mt;
+}
+
+#define ORACLE_CHUNK 2048 /* keys per work item; fixed so results do not depend on threads */
+
+typedef struct {
+    const tq4o_layout* L;
+    const tq4o_batch* B;
+    const uint16_t* q;
+    int q_dtype, num_q_heads, g;
+    /* work items */
+    int n_items;
+    int* it_tok;
+    int* it_kvh;
+    int* it_req;
+    int* it_lo;
+    int* it_hi;
+    double* it_acc; /* [n_items][g][hd] */
+    double* it_m;   /* [n_items][g] */
+    double* it_l;
+    int next;
+    pthread_mutex_t mu;
+} attn_job;
+
+static void* attn_worker(void* arg) {
+    attn_job* J = (attn_job*)arg;
+    const int hd = J->L->head_dim;
+    float* qrows = (float*)malloc((size_t)J->g * hd * sizeof(float));
+    for (;;) {
+        pthread_mutex_lock(&J->mu);
+        const int it = J->next++;
+        pthread_mutex_unlock(&J->mu);
+        if (it >= J->n_items) break;
+        load_q(J->L, J->q, J->q_dtype, J->it_tok[it], J->num_q_heads, J->it_kvh[it] * J->g, J->g, qrows);
+        attend_range(J->L, J->B, J->it_req[it], J->it_kvh[it], qrows, J->g, J->it_lo[it], J->it_hi[it],
+                     J->it_acc + (size_t)it * J->g * hd, J->it_m + (size_t)it * J->g,
+                     J->it_l + (size_t)it * J->g);
+    }
+    free(qrows);
+    return NULL;
+}
+
+int tq4o_paged_attention(const tq4o_layout* L, const tq4o_batch* B, const uint16_t* q, int q_dtype,
+                         float* out, int num_q_heads, int n_threads) {
+    if (L->local_kv_heads <= 0 || num_q_heads % L->local_kv_heads) return -1;
+    if (L->head_dim > 256) return -1;
+    const int hd = L->head_dim, g = num_q_heads / L->local_kv_heads;
+    attn_job J;
+    memset(&J, 0, sizeof(J));
+    J.L = L; J.B = B; J.q = q; J.q_dtype = q_dtype; J.num_q_heads = num_q_heads; J.g = g;
+    pthread_mutex_init(&J.mu, NULL);
+    /* enumerate items */
+    size_t cap = 0;
+    for (int pass = 0; pass < 2; ++pass) {
+        int n = 0;
+        for (int tok = 0; tok < B->total_tokens; ++tok) {
+            int req, lo, hi;
+            if (!row_range(B, tok, &req, &lo, &hi)) continue;
+            for (int h = 0; h < L->local_kv_heads; ++h) {
+                int c0 = lo;
+                do {
+                    int c1 = c0 + ORACLE_CHUNK - 1;
+                    if (c1 > hi) c1 = hi;
+                    if (pass) {
+                        J.it_tok[n] = tok; J.it_kvh[n] = h; J.it_req[n] = req;
+                        J.it_lo[n] = c0; J.it_hi[n] = c1;
+                    }
+                    ++n;
+                    c0 = c1 + 1;
+                } while (c0 <= hi);
+            }
+        }
+        if (!pass) {
+            cap = (size_t)(n > 0 ? n : 1);
+            J.n_items = n;
+            J.it_tok = (int*)malloc(cap * sizeof(int));
+            J.it_kvh = (int*)malloc(cap * sizeof(int));
+            J.it_req = (int*)malloc(cap * sizeof(int));
+            J.it_lo = (int*)malloc(cap * sizeof(int));
+            J.it_hi = (int*)malloc(cap * sizeof(int));
+            J.it_acc = (double*)malloc(cap * g * hd * sizeof(double));
+            J.it_m = (double*)malloc(cap * g * sizeof(double));
+            J.it_l = (double*)malloc(cap * g * sizeof(double));
+        }
+    }
+    if (n_threads < 1) n_threads = 1;
+    if (n_threads > 256) n_threads = 256;
+    if (n_threads == 1) {
+        attn_worker(&J);
+    } else {
+        pthread_t th[256];
+        for (int t = 0; t < n_threads; ++t) pthread_create(&th[t], NULL, attn_worker, &J);
+        for (int t = 0; t < n_threads; ++t) pthread_join(th[t], NULL);
+    }
+    /* merge the chunk states of every (token, kv head) in chunk order and store */
+    double* acc = (double*)malloc((size_t)hd * sizeof(double));
+    int it = 0;
+    while (it < J.n_items) {
+        const int tok = J.it_tok[it], h = J.it_kvh[it];
+        int end = it;
+        while (end < J.n_items && J.it_tok[end] == tok && J.it_kvh[end] == h) ++end;
+        for (int a = 0; a < g; ++a) {
+            double m = -INFINITY, l = 0.0;
+            for (int c = 0; c < hd; ++c) acc[c] = 0.0;
+            for (int k = it; k < end; ++k)
+                merge_state(acc, &m, &l, J.it_acc + ((size_t)k * g + a) * hd, J.it_m[(size_t)k * g + a],
+                            J.it_l[(size_t)k * g + a], hd);
+            store_out(L, acc, l, out + ((size_t)tok * num_q_heads + (size_t)h * g + a) * hd);
+        }
+        it = end;
+    }
+    free(acc);
+    free(J.it_tok); free(J.it_kvh); free(J.it_req); free(J.it_lo); free(J.it_hi);
+    free(J.it_acc); free(J.it_m); free(J.it_l);
+    pthread_mutex_destroy(&J.mu);
+    return 0;
+}
+
+/* ---- split-KV: op_paged_attn.cu:323-341 (page partition), :544-558 (fp32 partials),
+ * :1132-1218 (merge in fp32: m_tot, w = exp(m_s - m_tot), sum acc*w / sum l*w) ---- */
+int tq4o_paged_attention_split(const tq4o_layout* L, const tq4o_batch* B, const uint16_t* q,
+                               int q_dtype, float* out, int num_q_heads, int n_splits) {
+    if (L->local_kv_heads <= 0 || num_q_heads % L->local_kv_heads) return -1;
+    if (n_splits < 1) n_splits = 1;
+    const int hd = L->head_dim, g = num_q_heads / L->local_kv_heads, bs = L->block_size;
+    float* qrows = (float*)malloc((size_t)g * hd * sizeof(float));
+    double* acc = (double*)malloc((size_t)g * hd * sizeof(double));
+    double* m = (double*)malloc((size_t)g * sizeof(double));
+    double* l = (double*)malloc((size_t)g * sizeof(double));
+    float* p_acc = (float*)malloc((size_t)n_splits * g * hd * sizeof(float));
+    float* p_m = (float*)malloc((size_t)n_splits * g * sizeof(float));
+    float* p_l = (float*)malloc((size_t)n_splits * g * sizeof(float));
+    for (int tok = 0; tok < B->total_tokens; ++tok) {
+        int req, lo, hi;
+        if (!row_range(B, tok, &req, &lo, &hi)) continue;
+        const int first_page = lo / bs;
+        const int total_pages = hi >= lo ? hi / bs - first_page + 1 : 0;
+        const int pps = (total_pages + n_splits - 1) / n_splits > 0 ? (total_pages + n_splits - 1) / n_splits : 1;
+        for (int h = 0; h < L->local_kv_heads; ++h) {
+            load_q(L, q, q_dtype, tok, num_q_heads, h * g, g, qrows);
+            int active = 0;
+            for (int s = 0; s < n_splits; ++s) {
+                const int p0 = first_page + s * pps, p1 = p0 + pps;
+                int klo = p0 * bs, khi = p1 * bs - 1;
+                if (klo < lo) klo = lo;
+                if (khi > hi) khi = hi;
+                if (klo > khi) break;
+                attend_range(L, B, req, h, qrows, g, klo, khi, acc, m, l);
+                for (int a = 0; a < g; ++a) {
+                    for (int c = 0; c < hd; ++c)
+                        p_acc[((size_t)s * g + a) * hd + c] = (float)acc[(size_t)a * hd + c];
+                    p_m[(size_t)s * g + a] = (float)m[a];
+                    p_l[(size_t)s * g + a] = (float)l[a];
+                }
+                ++active;
+            }
+            for (int a = 0; a < g; ++a) {
+                float m_tot = -INFINITY;
+                for (int s = 0; s < active; ++s)
+                    if (p_l[(size_t)s * g + a] > 0.0f && p_m[(size_t)s * g + a] > m_tot)
+                        m_tot = p_m[(size_t)s * g + a];
+                float l_tot = 0.0f;
+                float o[256];
+                for (int c = 0; c < hd; ++c) o[c] = 0.0f;
+                for (int s = 0; s < active; ++s) {
+                    const float ls = p_l[(size_t)s * g + a];
+                    if (!(ls > 0.0f)) continue;
+                    const float w = expf(p_m[(size_t)s * g + a] - m_tot);
+                    l_tot += ls * w;
+                    for (int c = 0; c < hd; ++c) o[c] += p_acc[((size_t)s * g + a) * hd + c] * w;
+                }
+                const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+                for (int c = 0; c < hd; ++c) o[c] *= inv;
+                float* dst = out + ((size_t)tok * num_q_heads + (size_t)h * g + a) * hd;
+                if (hd == 256 && L->v_transform == TQ4O_XF_WHT256)
+                    tq4o_unrotate_row(o, dst);
+                else
+                    memcpy(dst, o, (size_t)hd * sizeof(float));
+            }
+        }
+    }
+    free(qrows); free(acc); free(m); free(l); free(p_acc); free(p_m); free(p_l);
+    return 0;
+}
+
+/* ---- deterministic synthetic inputs ---- */
+uint64_t tq4o_splitmix64(uint64_t* s) {
+    uint64_t z = (*s += 0x9E3779B97F4A7C15ull);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+static void normal_pair(uint64_t* s, double* z0, double* z1) {
+    const double u1 = ((double)(tq4o_splitmix64(s) >> 11) + 1.0) * 0x1.0p-53; /* (0,1] */
+    const double u2 = (double)(tq4o_splitmix64(s) >> 11) * 0x1.0p-53;         /* [0,1) */
+    const double r = sqrt(-2.0 * log(u1));
+    const double a = 6.283185307179586476925 * u2;
+    *z0 = r * cos(a);
+    *z1 = r * sin(a);
+}
+
+static inline uint16_t store16(float f, int dtype) {
+    return dtype == TQ4O_DT_BF16 ? tq4o_f32_to_bf16(f) : tq4o_f32_to_f16(f);
+}
+
+void tq4o_fill_normal(uint16_t* dst, size_t n, uint64_t seed, int dtype) {
+    uint64_t s = seed;
+    for (size_t i = 0; i < n; i += 2) {
+        double a, b;
+        normal_pair(&s, &a, &b);
+        dst[i] = store16((float)a, dtype);
+        if (i + 1 < n) dst[i + 1] = store16((float)b, dtype);
+    }
+}
+
+void tq4o_permutation(int32_t* dst, int n, uint64_t seed) {
+    uint64_t s = seed ^ 0xA5A5A5A5DEADBEEFull;
+    for (int i = 0; i < n; ++i) dst[i] = i;
+    for (int i = n - 1; i > 0; --i) { /* Fisher-Yates */
+        const int j = (int)(tq4o_splitmix64(&s) % (uint64_t)(i + 1));
+        const int32_t t = dst[i];
+        dst[i] = dst[j];
+        dst[j] = t;
+    }
+}
+
+void tq4o_fill_kv_rows(uint16_t* dst, size_t rows, int kv_heads, int head_dim, uint64_t seed,
+                       int dtype, int n_outliers) {
+    /* outlier channels per kv head: first n_outliers of a seeded permutation of 0..head_dim-1 */
+    float* gain = (float*)malloc((size_t)kv_heads * head_dim * sizeof(float));
+    int32_t* perm = (int32_t*)malloc((size_t)head_dim * sizeof(int32_t));
+    for (int h = 0; h < kv_heads; ++h) {
+        for (int c = 0; c < head_dim; ++c) gain[(size_t)h * head_dim + c] = 1.0f;
+        tq4o_permutation(perm, head_dim, seed * 1315423911ull + (uint64_t)h + 17u);
+        for (int k = 0; k < n_outliers && k < head_dim; ++k) gain[(size_t)h * head_dim + perm[k]] = 20.0f;
+    }
+    uint64_t s = seed;
+    const size_t per_row = (size_t)kv_heads * head_dim;
+    const size_t n = rows * per_row;
+    for (size_t i = 0; i < n; i += 2) {
+        double a, b;
+        normal_pair(&s, &a, &b);
+        dst[i] = store16((float)a * gain[i % per_row], dtype);
+        if (i + 1 < n) dst[i + 1] = store16((float)b * gain[(i + 1) % per_row], dtype);
+    }
+    free(gain);
+    free(perm);
+}
+
+int tq4o_hw_threads(void) {
+    long n = sysconf(_SC_NPROCESSORS_ONLN);
+    return n > 0 ? (int)n : 1;
+}

@@ -1,0 +1,131 @@
+/*
+ * tq4_oracle.h -- CPU restatement of the reference's KV-cache hot path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Nothing in the product library links, loads or calls this
+ * code: it exists so that tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg
+ * can check (and time) the HIP path against the reference's algorithm.
+ *
+ * The reference has no CPU implementation of this path and cannot be compiled here
+ * (CUDA kernels + a Rust host), so there is no oracle/_ref build; every function below
+ * restates the reference source it cites, with the numerics the CUDA source leaves to
+ * nvcc's -use_fast_math fixed as follows (declared oracle numerics):
+ *   - fp32 arithmetic in source order, no FMA contraction (build with -ffp-contract=off);
+ *   - 32-lane warp sums as the xor butterfly with offsets 16,8,4,2,1
+ *     (csrc/tq/tq4_kv_common.cuh:54-60);
+ *   - rsqrtf(x)  := (float)(1.0 / sqrt((double)x));
+ *   - a / b      := IEEE-754 fp32 division, round to nearest even;
+ *   - float -> fp16 / bf16 conversions round to nearest even;
+ *   - attention: fp32 dequantisation (scale * centroid), fp64 dot products, softmax and
+ *     accumulation (the tolerance of the parity tests covers the fp32/fp16 differences of
+ *     the kernels).
+ *
+ * Pins (what each function is checked against, see tests/test_oracle_*.py):
+ *   tables            reference literals (tests/golden/tq4_tables.json) + Lloyd-Max fixed
+ *                     point of the Beta(256) coordinate density by numeric integration
+ *   tq4o_wht256       Sylvester Hadamard matrix / 16, exact on integer inputs; involution
+ *   tq4o_encode_row   independent fp64 nearest-centroid + least-squares restatement,
+ *                     zero-row special case, layout pins (132 B stride, nibble order)
+ *                     -- exact code/scale BYTES for general inputs are pinned by no
+ *                     reference-held vector (none exists): "parity unpinned" beyond that
+ *   tq4o_attention    closed forms (Q=K=0 -> running mean of V, single key -> that V row),
+ *                     brute-force fp64 softmax over independently dequantised rows
+ *   tq4o_split_merge  equality with the single-pass result
+ */
+#ifndef TQ4_ORACLE_H
+#define TQ4_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { TQ4O_FMT_FP16 = 0, TQ4O_FMT_BF16 = 1, TQ4O_FMT_TQ4 = 2 };
+enum { TQ4O_XF_IDENTITY = 0, TQ4O_XF_WHT256 = 1 };
+enum { TQ4O_DT_F16 = 0, TQ4O_DT_BF16 = 1 };
+
+/* Host-pointer mirror of warp34_kv_layer_layout (csrc/warp34_cuda.h:59-80). */
+typedef struct {
+    uint8_t* k_base;
+    uint8_t* v_base;
+    uint64_t k_page_stride, k_head_stride, k_token_stride;
+    uint64_t v_page_stride, v_head_stride, v_token_stride;
+    int32_t  local_kv_heads, head_dim, block_size;
+    int32_t  k_format, v_format, k_transform, v_transform;
+} tq4o_layout;
+
+/* Host-pointer mirror of warp34_attention_batch (csrc/warp34_cuda.h:82-101). */
+typedef struct {
+    const int32_t* query_start_loc;
+    const int32_t* context_lens_before;
+    const int32_t* seq_lens_after;
+    const int32_t* block_tables;
+    const int32_t* write_slot_mapping;
+    const uint8_t* valid_token_mask;
+    const uint8_t* valid_req_mask;
+    int32_t num_reqs, total_tokens, max_blocks_per_req;
+    int32_t mask_mode, sliding_window;
+    float   sm_scale;
+} tq4o_batch;
+
+/* --- tables (csrc/tq/tq4_codebook.cuh:46-101) --- */
+const float* tq4o_centroids256(void);  /* [16] */
+const float* tq4o_boundaries256(void); /* [15] */
+const float* tq4o_signs256(void);      /* [256] */
+
+/* --- scalar conversions (crates/warp34-host/src/cuda/half.rs:10-95 semantics) --- */
+float    tq4o_f16_to_f32(uint16_t h);
+uint16_t tq4o_f32_to_f16(float f);
+float    tq4o_bf16_to_f32(uint16_t h);
+uint16_t tq4o_f32_to_bf16(float f);
+
+/* --- csrc/tq/tq4_kv_common.cuh:75-107 : in-place 256-point Walsh-Hadamard, scaled 1/16 --- */
+void tq4o_wht256(float* x);
+
+/* --- op_kv_cache.cu:152-218 : quantize one 256-wide row (fp32 values of the fp16/bf16
+ * source) into 132 bytes --- */
+void tq4o_encode_row(const float* x, uint8_t* dst132);
+
+/* --- op_kv_cache.cu:298-306 : dequantise one 132-byte row into the ROTATED domain --- */
+void tq4o_dequant_row(const uint8_t* src132, float* y);
+
+/* un-rotate: x = sign * WHT(y)  (op_kv_cache.cu:775-781) */
+void tq4o_unrotate_row(const float* y, float* x);
+
+/* --- op_kv_cache.cu:325-368, 798-824 : paged append.  k_in/v_in are 16-bit rows of dtype
+ * in_dtype with strides in elements.  Returns 0, or -1 for an unsupported layout. --- */
+int tq4o_kv_cache_write(const tq4o_layout* L, const tq4o_batch* B,
+                        const uint16_t* k_in, const uint16_t* v_in,
+                        int k_row_stride, int v_row_stride, int in_dtype);
+
+/* --- op_kv_cache.cu:373-457,619-792 : paged GQA attention, one (token, q_head) row at a
+ * time.  q is 16-bit of dtype q_dtype; out is fp32 [total_tokens, num_q_heads, head_dim];
+ * rows that the reference leaves untouched are left untouched here too.
+ * n_threads > 1 spreads rows over pthreads (results do not depend on it). --- */
+int tq4o_paged_attention(const tq4o_layout* L, const tq4o_batch* B,
+                         const uint16_t* q, int q_dtype, float* out, int num_q_heads,
+                         int n_threads);
+
+/* Same, but the key range of every row is cut into n_splits contiguous page ranges whose
+ * partial (acc, m, l) states are merged as op_paged_attn.cu:1132-1218 does. */
+int tq4o_paged_attention_split(const tq4o_layout* L, const tq4o_batch* B,
+                               const uint16_t* q, int q_dtype, float* out, int num_q_heads,
+                               int n_splits);
+
+/* --- deterministic synthetic inputs: SplitMix64 -> Box-Muller (fp64) -> RNE bf16/fp16 --- */
+uint64_t tq4o_splitmix64(uint64_t* state);
+/* fills n values ~ N(0,1) rounded to dtype; channels listed in outlier_cols (period
+ * head_dim within every row of row_elems) are multiplied by 20 before rounding */
+void tq4o_fill_normal(uint16_t* dst, size_t n, uint64_t seed, int dtype);
+void tq4o_fill_kv_rows(uint16_t* dst, size_t rows, int kv_heads, int head_dim,
+                       uint64_t seed, int dtype, int n_outliers);
+void tq4o_permutation(int32_t* dst, int n, uint64_t seed);
+
+/* number of hardware threads the timed baseline may use */
+int tq4o_hw_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
