@@ -1,0 +1,146 @@
+"""GPU parity: paged GQA decode / verify attention through the C ABI vs the CPU oracle.
+
+Tolerance (BASELINE): |got - want| <= 2e-3 + 1e-2 |want| against the fp64-accumulating oracle.
+Invariants follow the reference's GPU tests: page-permutation 0-ULP
+(tests/backbone_and_collectives.rs:455-572), split vs single pass < 2e-3 and graph-bucket
+bound independence (tests/tq4_vision_and_moe.rs:1355-1663), masked rows untouched
+(cuda/tests.rs sentinel 0x5500), scratch canaries (tests/paged_fa2.rs:171-200).
+"""
+import numpy as np
+import pytest
+
+import oracle
+from cases import make_case
+from oracle import DT_BF16, DT_F16, FMT_TQ4
+
+pytestmark = pytest.mark.gpu
+
+SCRATCH = 16 << 20
+
+
+def _dev_pool(pool):
+    import gpu_harness as G
+
+    d = G.DevPool(pool)
+    d.upload()
+    return d
+
+
+def _check(fmt, dtype, block_size, seq_lens, q_lens, seed, scratch=SCRATCH, q_heads=8, kv_heads=2,
+           mask_mode=0, window=0, ctx_null=False, **kw):
+    import gpu_harness as G
+
+    pool, bt, k, v, q, aq, ctx = make_case(fmt, block_size, seq_lens, q_lens, seed, dtype, kv_heads=kv_heads,
+                                           q_heads=q_heads)
+    hb = oracle.HostBatch(aq, seq_lens, bt, context_lens_before=None if ctx_null else ctx, mask_mode=mask_mode,
+                          sliding_window=window)
+    want = oracle.paged_attention(pool, hb, q, dtype, q_heads, n_threads=4)
+    dpool = _dev_pool(pool)
+    rc, got, _ = G.dev_attention(dpool, hb, q, dtype, q_heads, scratch_bytes=scratch, **kw)
+    assert rc == 0
+    err = G.assert_close(got, dtype, want, what="fmt=%d bs=%d seq=%s q=%s" % (fmt, block_size, seq_lens, q_lens))
+    return got, want, err
+
+
+@pytest.mark.parametrize("dtype", [DT_BF16, DT_F16])
+@pytest.mark.parametrize("block_size", [16, 64])
+def test_tq4_decode_small_batch(dtype, block_size):
+    _check(FMT_TQ4, dtype, block_size, [70, 33, 129, 1, 32], [1, 1, 1, 1, 1], 11)
+
+
+@pytest.mark.parametrize("scratch", [0, SCRATCH])
+def test_tq4_decode_gqa8_long(scratch):
+    """16 q heads / 2 kv heads (GQA 8), one sequence of 5000 tokens, with and without scratch."""
+    _check(FMT_TQ4, DT_BF16, 64, [5000], [1], 21, scratch=scratch, q_heads=16)
+
+
+def test_tq4_decode_split_vs_single_pass():
+    import gpu_harness as G
+
+    pool, bt, k, v, q, aq, ctx = make_case(FMT_TQ4, 64, [20000, 777], [1, 1], 31, DT_BF16, q_heads=16)
+    hb = oracle.HostBatch(aq, [20000, 777], bt, context_lens_before=ctx)
+    dpool = _dev_pool(pool)
+    rc0, single, _ = G.dev_attention(dpool, hb, q, DT_BF16, 16, scratch_bytes=0)
+    rc1, split, ws = G.dev_attention(dpool, hb, q, DT_BF16, 16, scratch_bytes=SCRATCH)
+    assert rc0 == 0 and rc1 == 0
+    # split vs single pass (tests/tq4_vision_and_moe.rs:1652-1660: < 2e-3 on unit-scale data);
+    # both are bf16 here, so allow the same row-scaled bound as against the oracle
+    G.assert_close(split, DT_BF16, oracle.bf16_bits_to_f32(single), what="split vs single")
+    want = oracle.paged_attention(pool, hb, q, DT_BF16, 16, n_threads=8)
+    G.assert_close(split, DT_BF16, want, what="split")
+    G.assert_close(single, DT_BF16, want, what="single")
+    # a scratch that is too small or misaligned must be left untouched (single pass instead)
+    rc2, small, ws2 = G.dev_attention(dpool, hb, q, DT_BF16, 16, scratch_bytes=4096)
+    assert rc2 == 0 and bool((ws2 == 0x5A).all())
+    assert small.tobytes() == single.tobytes()
+
+
+@pytest.mark.parametrize("q_lens", [[4, 4], [2, 3], [16]])
+def test_tq4_verify_multi_token_causal(q_lens):
+    seq = [300 + 7 * i for i in range(len(q_lens))]
+    _check(FMT_TQ4, DT_BF16, 64, seq, q_lens, 41, q_heads=16)
+    _check(FMT_TQ4, DT_F16, 16, seq, q_lens, 42, q_heads=8, scratch=0)
+
+
+@pytest.mark.parametrize("mask_mode,window", [(0, 40), (1, 0), (1, 100), (0, 5)])
+def test_tq4_windows(mask_mode, window):
+    _check(FMT_TQ4, DT_BF16, 16, [333, 90], [3, 2], 51, mask_mode=mask_mode, window=window, ctx_null=True)
+
+
+def test_page_permutation_and_bounds_do_not_change_bits():
+    import gpu_harness as G
+
+    outs = []
+    for perm_seed in (1, 2):
+        pool, bt, k, v, q, aq, ctx = make_case(FMT_TQ4, 16, [1500, 200], [1, 1], 61, DT_F16, perm_seed=perm_seed)
+        hb = oracle.HostBatch(aq, [1500, 200], bt, context_lens_before=ctx)
+        dpool = _dev_pool(pool)
+        for bound in (None, 4096):
+            rc, out, _ = G.dev_attention(dpool, hb, q, DT_F16, 8, scratch_bytes=SCRATCH, max_seq_len=bound)
+            assert rc == 0
+            outs.append(out)
+    for o in outs[1:]:
+        assert o.tobytes() == outs[0].tobytes()
+
+
+def test_masked_rows_are_untouched():
+    import gpu_harness as G
+
+    seq_lens, q_lens = [40, 24, 300], [2, 3, 1]
+    pool, bt, k, v, q, aq, ctx = make_case(FMT_TQ4, 64, seq_lens, q_lens, 71, DT_BF16)
+    tmask = np.array([1, 0, 1, 1, 1, 1], dtype=np.uint8)
+    rmask = np.array([1, 0, 1], dtype=np.uint8)
+    hb = oracle.HostBatch(aq, seq_lens, bt, context_lens_before=ctx, valid_token_mask=tmask, valid_req_mask=rmask)
+    want = oracle.paged_attention(pool, hb, q, DT_BF16, 8)
+    dpool = _dev_pool(pool)
+    for scratch in (0, SCRATCH):
+        rc, got, _ = G.dev_attention(dpool, hb, q, DT_BF16, 8, scratch_bytes=scratch, sentinel=0x5500)
+        assert rc == 0
+        for tok in (1, 2, 3, 4):
+            assert (got[tok] == 0x5500).all()
+        for tok in (0, 5):
+            G.assert_close(got[tok], DT_BF16, want[tok], what="tok %d" % tok)
+
+
+def test_empty_key_range_gives_zeros():
+    """A sliding window that ends before the first key -> zeros (op_kv_cache.cu:939-946)."""
+    import gpu_harness as G
+
+    pool, bt, k, v, q, aq, ctx = make_case(FMT_TQ4, 16, [50], [1], 81, DT_BF16)
+    hb = oracle.HostBatch(aq, [10], bt, context_lens_before=[60], sliding_window=4)  # window [57, 60], seq 10
+    dpool = _dev_pool(pool)
+    rc, got, _ = G.dev_attention(dpool, hb, q, DT_BF16, 8, scratch_bytes=SCRATCH)
+    assert rc == 0 and not oracle.bf16_bits_to_f32(got).any()  # +-0 everywhere
+
+
+def test_force_kernel_selector_agrees():
+    import gpu_harness as G
+
+    pool, bt, k, v, q, aq, ctx = make_case(FMT_TQ4, 16, [260], [8], 91, DT_F16)
+    hb = oracle.HostBatch(aq, [260], bt, context_lens_before=ctx)
+    want = oracle.paged_attention(pool, hb, q, DT_F16, 8)
+    dpool = _dev_pool(pool)
+    for sel in (0, 1, 2):
+        rc, got, _ = G.dev_attention(dpool, hb, q, DT_F16, 8, force_kernel=sel)
+        assert rc == 0
+        G.assert_close(got, DT_F16, want, what="selector %d" % sel)

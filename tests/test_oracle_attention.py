@@ -15,6 +15,7 @@ import pytest
 from scipy.linalg import hadamard
 
 import oracle
+from cases import make_case
 from oracle import DT_BF16, DT_F16, FMT_BF16, FMT_FP16, FMT_TQ4, XF_IDENTITY, XF_WHT256
 
 H = hadamard(256).astype(np.float64)
@@ -50,38 +51,6 @@ def brute(qf, K, V, lo, hi, scale):
     sc = (K[lo:hi + 1] @ qf) * scale
     p = np.exp(sc - sc.max())
     return (p[:, None] * V[lo:hi + 1]).sum(0) / p.sum()
-
-
-def make_case(fmt, block_size, seq_lens, q_lens, seed, dtype, kv_heads=2, q_heads=8, perm_seed=5,
-              extra_pages=3):
-    """Append seq_len tokens per request through the oracle's write, return everything."""
-    xf = XF_WHT256 if fmt == FMT_TQ4 else XF_IDENTITY
-    pages_per = [(s + block_size - 1) // block_size for s in seq_lens]
-    num_pages = sum(pages_per) + extra_pages
-    perm = oracle.permutation(num_pages, perm_seed)
-    pool = oracle.HostPool(num_pages, kv_heads, 256, block_size, fmt, xf)
-    mb = max(pages_per)
-    bt = np.zeros((len(seq_lens), mb), dtype=np.int32)
-    at = 0
-    slots, qsl = [], [0]
-    for r, s in enumerate(seq_lens):
-        bt[r, :pages_per[r]] = perm[at:at + pages_per[r]]
-        at += pages_per[r]
-        slots.append(oracle.slot_mapping(bt[r], 0, s, block_size))
-        qsl.append(qsl[-1] + s)
-    total = qsl[-1]
-    k = oracle.fill_kv_rows(total, kv_heads, 256, seed, dtype, 3)
-    v = oracle.fill_kv_rows(total, kv_heads, 256, seed + 1, dtype, 3)
-    wb = oracle.HostBatch(qsl, seq_lens, bt, context_lens_before=[0] * len(seq_lens),
-                          write_slot_mapping=np.concatenate(slots))
-    oracle.kv_cache_write(pool, wb, k, v, dtype)
-    # attention batch: last q_len tokens of each request are the queries
-    aq = [0]
-    for ql in q_lens:
-        aq.append(aq[-1] + ql)
-    q = oracle.fill_normal(aq[-1] * q_heads * 256, seed + 2, dtype).reshape(aq[-1], q_heads, 256)
-    ctx = [s - ql for s, ql in zip(seq_lens, q_lens)]
-    return pool, bt, k, v, q, aq, ctx
 
 
 @pytest.mark.parametrize("fmt,dtype", [(FMT_TQ4, DT_BF16), (FMT_TQ4, DT_F16), (FMT_FP16, DT_F16), (FMT_BF16, DT_BF16)])

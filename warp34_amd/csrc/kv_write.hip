@@ -1,0 +1,284 @@
+// Quantize-on-append for gfx950: writes one (token, kv head) K row and V row per wave64
+// into the paged slabs described by warp34_kv_layer_layout.
+//
+// Replaces the reference's kv_cache_write_kernel / write_kv_row (op_kv_cache.cu:10-368) and
+// kv_cache_write_bf16_kernel (op_kv_cache.cu:798-824) behind the same entry points
+// (op_kv_cache.cu:828-858,1172-1190).
+//
+// Mapping: lanes 0-31 of a wave encode the K row, lanes 32-63 the V row, so the reference's
+// 32-lane reduction tree (tq4_kv_common.cuh:54-60) is reproduced with xor shuffles that stay
+// inside one half of the wave.  Element i of a row lives in lane i%32, register i/32, as in
+// op_kv_cache.cu:164-167.
+//
+// Numerics of the TQ4 encode (bit-exact contract with the CPU restatement): fp32 in source
+// order with FMA contraction disabled for this file (-ffp-contract=off), rsqrt(x) computed
+// as (float)(1.0/sqrt((double)x)), IEEE fp32 division, round-to-nearest-even fp16 scale.
+#include "kv_common.h"
+
+namespace w34 {
+
+// 32-lane xor butterfly sum, offsets 16,8,4,2,1 (tq4_kv_common.cuh:54-60).
+__device__ __forceinline__ float half_wave_sum(float v) {
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 8, 64);
+    v += __shfl_xor(v, 4, 64);
+    v += __shfl_xor(v, 2, 64);
+    v += __shfl_xor(v, 1, 64);
+    return v;
+}
+
+// 256-point Walsh-Hadamard over 32 lanes x 8 registers (tq4_kv_common.cuh:75-107):
+// stages over index bits 0..4 cross lanes, bits 5..7 stay in registers; the last stage
+// carries the 1/16 scale.
+__device__ __forceinline__ void wht256_half_wave(float (&v)[8], int l32) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        float val = v[j];
+#pragma unroll
+        for (int h = 1; h < 32; h <<= 1) {
+            const float o = __shfl_xor(val, h, 64);
+            val = (l32 & h) ? (o - val) : (val + o);
+        }
+        v[j] = val;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j += 2) {
+        const float a = v[j], b = v[j + 1];
+        v[j] = a + b;
+        v[j + 1] = a - b;
+    }
+#pragma unroll
+    for (int g = 0; g < 8; g += 4) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const float a = v[g + i], b = v[g + i + 2];
+            v[g + i] = a + b;
+            v[g + i + 2] = a - b;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float a = v[i], b = v[i + 4];
+        v[i] = (a + b) * 0.0625f;
+        v[i + 4] = (a - b) * 0.0625f;
+    }
+}
+
+// TQ4 encode of one 256-wide row held as v[j] = x[l32 + 32 j] (op_kv_cache.cu:152-218).
+__device__ __forceinline__ void tq4_encode_row(float (&v)[8], int l32, uint8_t* dst) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = apply_sign(v[j], l32 + 32 * j);
+    wht256_half_wave(v, l32);
+
+    float s_sq0 = 0.0f, s_sq1 = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        s_sq0 += half_wave_sum(v[j] * v[j]);
+        s_sq1 += half_wave_sum(v[j + 4] * v[j + 4]);
+    }
+    const float rs0 = (float)(1.0 / sqrt((double)s_sq0));
+    const float rs1 = (float)(1.0 / sqrt((double)s_sq1));
+    const float inv_norm0 = (s_sq0 > 1e-20f) ? (0.7071067811865475f * rs0) : 0.0f;
+    const float inv_norm1 = (s_sq1 > 1e-20f) ? (0.7071067811865475f * rs1) : 0.0f;
+
+    float vc_dot0 = 0.0f, c_sq0 = 0.0f, vc_dot1 = 0.0f, c_sq1 = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float raw_v = v[j];
+        const float rv = raw_v * ((j < 4) ? inv_norm0 : inv_norm1);
+        int q = 0;
+#pragma unroll
+        for (int i = 0; i < 15; ++i) q += (rv > kBoundaries[i]) ? 1 : 0;
+        // byte m of a 64-byte block holds elements 2m (low nibble) and 2m+1 (high nibble);
+        // elements l32 and l32^1 of register j are neighbours.
+        const int partner = __shfl_xor(q, 1, 64);
+        if ((l32 & 1) == 0) {
+            dst[66 * (j >> 2) + 2 + (((j & 3) * 32 + l32) >> 1)] = (uint8_t)(q | (partner << 4));
+        }
+        const float c = kCentroids[q];
+        const float vc = half_wave_sum(raw_v * c);
+        const float cc = half_wave_sum(c * c);
+        if (j < 4) {
+            vc_dot0 += vc;
+            c_sq0 += cc;
+        } else {
+            vc_dot1 += vc;
+            c_sq1 += cc;
+        }
+    }
+    if (l32 == 0) {
+        const float d0 = (c_sq0 > 1e-10f) ? (vc_dot0 / c_sq0) : 0.0f;
+        const float d1 = (c_sq1 > 1e-10f) ? (vc_dot1 / c_sq1) : 0.0f;
+        *reinterpret_cast<uint16_t*>(dst) = F16::from_f32(d0);
+        *reinterpret_cast<uint16_t*>(dst + 66) = F16::from_f32(d1);
+    }
+}
+
+// One wave per (token, kv head); lanes 0-31 write K, lanes 32-63 write V.
+template <typename TIn>
+__global__ __launch_bounds__(256) void kv_append_kernel(warp34_kv_layer_layout L,
+                                                        warp34_attention_batch B,
+                                                        const uint16_t* __restrict__ k_in,
+                                                        const uint16_t* __restrict__ v_in,
+                                                        int k_row_stride, int v_row_stride,
+                                                        int check_req_mask) {
+    const int wave = (int)(threadIdx.x >> 6);
+    const int item = (int)blockIdx.x * 4 + wave;
+    const int tok = item / L.local_kv_heads;
+    const int head = item - tok * L.local_kv_heads;
+    if (tok >= B.total_tokens) return;
+    if (B.valid_token_mask != nullptr && B.valid_token_mask[tok] == 0) return;
+    if (check_req_mask) {
+        int a, b;
+        const int r = find_request(B, tok, a, b);
+        if (r < 0 || (B.valid_req_mask != nullptr && B.valid_req_mask[r] == 0)) return;
+    }
+    const int32_t slot = B.write_slot_mapping[tok];
+    if (slot < 0) return;
+    const int page = slot / L.block_size;
+    const int off = slot - page * L.block_size;
+
+    const int lane = lane_id();
+    const int is_v = lane >> 5;
+    const int l32 = lane & 31;
+    const int format = is_v ? L.v_format : L.k_format;
+    uint8_t* dst = reinterpret_cast<uint8_t*>((uintptr_t)(is_v ? L.v_base : L.k_base)) +
+                   (size_t)page * (is_v ? L.v_page_stride_bytes : L.k_page_stride_bytes) +
+                   (size_t)head * (is_v ? L.v_head_stride_bytes : L.k_head_stride_bytes) +
+                   (size_t)off * (is_v ? L.v_token_stride_bytes : L.k_token_stride_bytes);
+    const uint16_t* src = (is_v ? v_in : k_in) +
+                          (size_t)tok * (size_t)(is_v ? v_row_stride : k_row_stride) +
+                          (size_t)head * (size_t)L.head_dim;
+
+    if (format == WARP34_KV_FORMAT_TQ4) {
+        // host side guarantees head_dim == 256 and the WHT256 transform for TQ4
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = TIn::to_f32(src[l32 + 32 * j]);
+        tq4_encode_row(v, l32, dst);
+        return;
+    }
+    // 16-bit storage formats: plain copy when the storage type is the source type,
+    // otherwise convert through fp32 (op_kv_cache.cu:18-31).
+    uint16_t* d16 = reinterpret_cast<uint16_t*>(dst);
+    const bool same = (format == TIn::kStorageFormat);
+    for (int c = l32; c < L.head_dim; c += 32) {
+        const uint16_t b = src[c];
+        if (same) {
+            d16[c] = b;
+        } else {
+            const float f = TIn::to_f32(b);
+            d16[c] = (format == WARP34_KV_FORMAT_BF16) ? BF16::from_f32(f) : F16::from_f32(f);
+        }
+    }
+}
+
+static bool format_supported_for_write(int format, int transform, int head_dim) {
+    if (format == WARP34_KV_FORMAT_FP16 || format == WARP34_KV_FORMAT_BF16) {
+        return transform == WARP34_KV_TRANSFORM_IDENTITY;
+    }
+    if (format == WARP34_KV_FORMAT_TQ4) {
+        return head_dim == 256 && transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256;
+    }
+    return false;
+}
+
+template <typename TIn>
+static int launch_append(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
+                         const warp34_attention_batch* batch, const void* k_in, const void* v_in,
+                         int k_row_stride, int v_row_stride) {
+    const long long items = (long long)batch->total_tokens * layout->local_kv_heads;
+    const unsigned grid = (unsigned)((items + 3) / 4);
+    const int check_req = (batch->valid_req_mask != nullptr && batch->query_start_loc != nullptr &&
+                           batch->num_reqs > 0)
+                              ? 1
+                              : 0;
+    hipLaunchKernelGGL((kv_append_kernel<TIn>), dim3(grid), dim3(256), 0, (hipStream_t)ex->stream,
+                       *layout, *batch, (const uint16_t*)k_in, (const uint16_t*)v_in, k_row_stride,
+                       v_row_stride, check_req);
+    return (int)hipGetLastError();
+}
+
+}  // namespace w34
+
+using namespace w34;
+
+// op_kv_cache.cu:828-850
+extern "C" int warp34_kv_cache_write_strided(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
+                                             const warp34_attention_batch* batch, const void* k_in,
+                                             const void* v_in, int k_row_stride, int v_row_stride) {
+    if (ex == nullptr || layout == nullptr || batch == nullptr || k_in == nullptr || v_in == nullptr) {
+        return (int)hipErrorInvalidValue;
+    }
+    if (layout->k_format == WARP34_KV_FORMAT_FP8_E4M3 || layout->v_format == WARP34_KV_FORMAT_FP8_E4M3) {
+        if (layout->head_dim != 256) return (int)hipErrorInvalidValue;
+        return (int)hipErrorNotSupported;
+    }
+    if (batch->total_tokens <= 0 || layout->local_kv_heads <= 0) return 0;
+    const int min_stride = layout->local_kv_heads * layout->head_dim;
+    if (k_row_stride < min_stride || v_row_stride < min_stride) return (int)hipErrorInvalidValue;
+    if (batch->write_slot_mapping == nullptr || layout->block_size <= 0 || layout->k_base == 0 ||
+        layout->v_base == 0) {
+        return (int)hipErrorInvalidValue;
+    }
+    if (!format_supported_for_write(layout->k_format, layout->k_transform, layout->head_dim) ||
+        !format_supported_for_write(layout->v_format, layout->v_transform, layout->head_dim)) {
+        return (int)hipErrorNotSupported;
+    }
+    return launch_append<F16>(ex, layout, batch, k_in, v_in, k_row_stride, v_row_stride);
+}
+
+// op_kv_cache.cu:852-858
+extern "C" int warp34_kv_cache_write(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
+                                     const warp34_attention_batch* batch, const void* k_in,
+                                     const void* v_in) {
+    if (layout == nullptr) return (int)hipErrorInvalidValue;
+    const int stride = layout->local_kv_heads * layout->head_dim;
+    return warp34_kv_cache_write_strided(ex, layout, batch, k_in, v_in, stride, stride);
+}
+
+// Layouts the bf16 entry points accept: the reference's BF16 identity layout
+// (op_kv_cache.cu:860-865) plus TQ4 + WHT256 at head_dim 256.
+static bool valid_bf16_entry_layout(const warp34_kv_layer_layout* l) {
+    if (!l || l->local_kv_heads <= 0 || l->block_size <= 0 || l->head_dim <= 0 || l->head_dim > 256 ||
+        !l->k_base || !l->v_base) {
+        return false;
+    }
+    const bool bf16 = l->k_format == WARP34_KV_FORMAT_BF16 && l->v_format == WARP34_KV_FORMAT_BF16 &&
+                      l->k_transform == WARP34_KV_TRANSFORM_IDENTITY &&
+                      l->v_transform == WARP34_KV_TRANSFORM_IDENTITY;
+    const bool tq4 = l->head_dim == 256 && l->k_format == WARP34_KV_FORMAT_TQ4 &&
+                     l->v_format == WARP34_KV_FORMAT_TQ4 &&
+                     l->k_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 &&
+                     l->v_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256;
+    return bf16 || tq4;
+}
+
+// op_kv_cache.cu:1172-1183
+extern "C" int warp34_kv_cache_write_strided_bf16(const warp34_exec* ex,
+                                                  const warp34_kv_layer_layout* layout,
+                                                  const warp34_attention_batch* batch, const void* k,
+                                                  const void* v, int row_stride_elems) {
+    if (!ex || !valid_bf16_entry_layout(layout) || !batch || !k || !v ||
+        row_stride_elems < layout->local_kv_heads * layout->head_dim || batch->total_tokens < 0 ||
+        batch->num_reqs <= 0 || !batch->query_start_loc || !batch->write_slot_mapping) {
+        return (int)hipErrorInvalidValue;
+    }
+    if (!batch->total_tokens) return 0;
+    // the reference's bf16 writer always resolves the owning request (op_kv_cache.cu:803-807)
+    const long long items = (long long)batch->total_tokens * layout->local_kv_heads;
+    const unsigned grid = (unsigned)((items + 3) / 4);
+    hipLaunchKernelGGL((kv_append_kernel<BF16>), dim3(grid), dim3(256), 0, (hipStream_t)ex->stream,
+                       *layout, *batch, (const uint16_t*)k, (const uint16_t*)v, row_stride_elems,
+                       row_stride_elems, 1);
+    return (int)hipGetLastError();
+}
+
+// op_kv_cache.cu:1185-1190
+extern "C" int warp34_kv_cache_write_bf16(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
+                                          const warp34_attention_batch* batch, const void* k,
+                                          const void* v) {
+    if (!valid_bf16_entry_layout(layout)) return (int)hipErrorInvalidValue;
+    return warp34_kv_cache_write_strided_bf16(ex, layout, batch, k, v,
+                                              layout->local_kv_heads * layout->head_dim);
+}
