@@ -1,0 +1,250 @@
+#!/usr/bin/env python3
+"""Headline benchmark: paged TQ4 decode attention at 128K context on one MI355X.
+
+One "step" = one full-attention layer's decode attention for the workload
+(`warp34_paged_attention_bf16` over TQ4 pages, through the C ABI).  The KV pools of
+several layers are allocated and the steps cycle through them, as a decode step of the model
+would, so that the working set (layers x 69.2 MB) exceeds the 256 MB last-level cache and
+the figure is an HBM figure.  K/V are synthetic bf16 N(0,1) with 1 % outlier channels (x20),
+TQ4-encoded by the library's own quantize-on-append kernel into 64-token pages whose
+physical order is a random permutation.
+
+Prints ONE JSON line (see README / DESIGN for the fields).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+KV_HEADS, Q_HEADS, HEAD_DIM, BLOCK = 2, 16, 256, 64
+ROW_BYTES = 132
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="tq4_decode_b1_ctx131072",
+                    choices=["tq4_decode_b1_ctx131072", "tq4_decode_b32_ctx1k_64k"])
+    ap.add_argument("--layers", type=int, default=0, help="KV pools to cycle through (0 = auto, > 256 MB total)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-ctx", type=int, default=32768, help="context length of the CPU-oracle sample")
+    return ap.parse_args()
+
+
+def build_workload(name, seed=0):
+    rng = np.random.default_rng(seed)
+    if name == "tq4_decode_b1_ctx131072":
+        ctx = np.array([131072], dtype=np.int64)
+    else:
+        ctx = rng.integers(1024, 65537, size=32).astype(np.int64)
+    return ctx
+
+
+class Layer:
+    """One layer's TQ4 pool on the device, filled through the append kernel."""
+
+    def __init__(self, torch, lib, ffi, ctx, pool_pages, seed):
+        dev = "cuda:0"
+        self.tok, self.head = ROW_BYTES, BLOCK * ROW_BYTES
+        self.page = KV_HEADS * self.head
+        self.k = torch.zeros(pool_pages * self.page, dtype=torch.uint8, device=dev)
+        self.v = torch.zeros(pool_pages * self.page, dtype=torch.uint8, device=dev)
+        self.layout = ffi.Warp34KvLayerLayout(
+            self.k.data_ptr(), self.v.data_ptr(), self.page, self.head, self.tok, self.page, self.head, self.tok,
+            0, seed, KV_HEADS, HEAD_DIM, BLOCK, ffi.WARP34_KV_FORMAT_TQ4, ffi.WARP34_KV_FORMAT_TQ4,
+            ffi.WARP34_KV_TRANSFORM_RADEMACHER_WHT256, ffi.WARP34_KV_TRANSFORM_RADEMACHER_WHT256, 0)
+        g = torch.Generator(device=dev)
+        g.manual_seed(1000 + seed)
+        pages_per = [(int(c) + BLOCK - 1) // BLOCK for c in ctx]
+        perm = torch.randperm(pool_pages, generator=g, device=dev).to(torch.int32)
+        mb = max(pages_per)
+        bt = torch.zeros((len(ctx), mb), dtype=torch.int32, device=dev)
+        at = 0
+        for r, n in enumerate(pages_per):
+            bt[r, :n] = perm[at:at + n]
+            at += n
+        self.block_tables = bt
+        self.max_blocks = mb
+        # outlier channels: 3 of 256 per kv head scaled x20
+        gain = torch.ones((KV_HEADS, HEAD_DIM), device=dev)
+        for h in range(KV_HEADS):
+            idx = torch.randperm(HEAD_DIM, generator=g, device=dev)[:3]
+            gain[h, idx] = 20.0
+        stream = torch.cuda.current_stream().cuda_stream
+        ex = ffi.Warp34Exec(stream, 0, 0, 0)
+        chunk = 8192
+        for r, c in enumerate(ctx):
+            c = int(c)
+            for t0 in range(0, c, chunk):
+                n = min(chunk, c - t0)
+                kk = (torch.randn((n, KV_HEADS, HEAD_DIM), generator=g, device=dev) * gain).to(torch.bfloat16)
+                vv = (torch.randn((n, KV_HEADS, HEAD_DIM), generator=g, device=dev) * gain).to(torch.bfloat16)
+                pos = torch.arange(t0, t0 + n, device=dev)
+                slots = (bt[r, (pos // BLOCK)].to(torch.int64) * BLOCK + pos % BLOCK).to(torch.int32)
+                qsl = torch.tensor([0, n], dtype=torch.int32, device=dev)
+                seq = torch.tensor([t0 + n], dtype=torch.int32, device=dev)
+                b = ffi.Warp34AttentionBatch(qsl.data_ptr(), None, seq.data_ptr(), bt[r].data_ptr(), slots.data_ptr(),
+                                             None, None, 1, n, mb, n, t0 + n, 0, 0, 0.0625, 0)
+                rc = lib.warp34_kv_cache_write_bf16(C.byref(ex), C.byref(self.layout), C.byref(b),
+                                                    C.c_void_p(kk.data_ptr()), C.c_void_p(vv.data_ptr()))
+                if rc:
+                    raise RuntimeError("warp34_kv_cache_write_bf16 rc=%d" % rc)
+                torch.cuda.synchronize()
+
+
+def cpu_baseline(ctx_len, threads):
+    """The CPU oracle (port of the reference's scalar path) timed on this host: one decode
+    attention layer at ctx_len tokens, all hardware threads."""
+    import oracle
+
+    n_pages = (ctx_len + BLOCK - 1) // BLOCK
+    pool = oracle.HostPool(n_pages, KV_HEADS, HEAD_DIM, BLOCK, oracle.FMT_TQ4, oracle.XF_WHT256)
+    # encode a small set of rows and tile them: the attention cost does not depend on values
+    rows = 256
+    k = oracle.fill_kv_rows(rows, KV_HEADS, HEAD_DIM, 1, oracle.DT_BF16, 3)
+    v = oracle.fill_kv_rows(rows, KV_HEADS, HEAD_DIM, 2, oracle.DT_BF16, 3)
+    small = oracle.HostPool(rows // BLOCK, KV_HEADS, HEAD_DIM, BLOCK, oracle.FMT_TQ4, oracle.XF_WHT256)
+    bt_s = np.arange(rows // BLOCK, dtype=np.int32).reshape(1, -1)
+    wb = oracle.HostBatch([0, rows], [rows], bt_s, context_lens_before=[0],
+                          write_slot_mapping=oracle.slot_mapping(bt_s[0], 0, rows, BLOCK))
+    t0 = time.perf_counter()
+    oracle.kv_cache_write(small, wb, k, v, oracle.DT_BF16)
+    t_append = time.perf_counter() - t0
+    reps = (pool.k.size + small.k.size - 1) // small.k.size
+    pool.k[:] = np.tile(small.k, reps)[:pool.k.size]
+    pool.v[:] = np.tile(small.v, reps)[:pool.v.size]
+    bt = oracle.permutation(n_pages, 3).reshape(1, -1)
+    q = oracle.fill_normal(Q_HEADS * HEAD_DIM, 4, oracle.DT_BF16).reshape(1, Q_HEADS, HEAD_DIM)
+    hb = oracle.HostBatch([0, 1], [ctx_len], bt, context_lens_before=[ctx_len - 1])
+    t0 = time.perf_counter()
+    oracle.paged_attention(pool, hb, q, oracle.DT_BF16, Q_HEADS, n_threads=threads)
+    dt = time.perf_counter() - t0
+    kv_bytes = ctx_len * KV_HEADS * 2 * ROW_BYTES
+    return {
+        "value": round(kv_bytes / dt / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": "CPU oracle (oracle/tq4_oracle.c), 1 layer decode attention, ctx %d tokens, %d pthreads: "
+                  "%.1f ms/layer; append of %d rows single-thread: %.0f rows/s"
+                  % (ctx_len, threads, dt * 1e3, rows * KV_HEADS * 2, rows * KV_HEADS * 2 / t_append),
+        "us_per_layer": round(dt * 1e6, 1),
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU only (this build has no multi-GPU path); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from warp34_amd import ffi
+
+    if not torch.cuda.is_available():
+        print("no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    lib = ffi.load()
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    ctx = build_workload(args.workload)
+    total_tokens_kv = int(ctx.sum())
+    kv_bytes = total_tokens_kv * KV_HEADS * 2 * ROW_BYTES  # algorithmic bytes per step (K + V rows)
+    pool_pages = sum((int(c) + BLOCK - 1) // BLOCK for c in ctx) + 16
+    layer_bytes = 2 * pool_pages * KV_HEADS * BLOCK * ROW_BYTES
+    n_layers = args.layers or max(2, -(-(640 << 20) // layer_bytes))
+    layers = [Layer(torch, lib, ffi, ctx, pool_pages, s) for s in range(n_layers)]
+
+    R = len(ctx)
+    g = torch.Generator(device=dev)
+    g.manual_seed(7)
+    q = torch.randn((R, Q_HEADS, HEAD_DIM), generator=g, device=dev).to(torch.bfloat16)
+    out = torch.zeros_like(q)
+    qsl = torch.arange(0, R + 1, dtype=torch.int32, device=dev)
+    seq = torch.tensor(ctx, dtype=torch.int32, device=dev)
+    ctxb = seq - 1
+    scratch_bytes = 32 << 20
+    scratch = torch.zeros(scratch_bytes, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    ex = ffi.Warp34Exec(stream, scratch.data_ptr(), scratch_bytes, 0)
+    batches = []
+    for L in layers:
+        batches.append(ffi.Warp34AttentionBatch(
+            qsl.data_ptr(), ctxb.data_ptr(), seq.data_ptr(), L.block_tables.data_ptr(), None, None, None,
+            R, R, L.max_blocks, 1, int(ctx.max()), 0, 0, 1.0 / 16.0, 0))
+
+    def step(i):
+        L = layers[i % n_layers]
+        rc = lib.warp34_paged_attention_bf16(C.byref(ex), C.byref(L.layout), C.byref(batches[i % n_layers]),
+                                             C.c_void_p(q.data_ptr()), C.c_void_p(out.data_ptr()), Q_HEADS)
+        if rc:
+            raise RuntimeError("warp34_paged_attention_bf16 rc=%d" % rc)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t_wall0 = time.perf_counter()
+    e0.record()
+    for i in range(args.steps):
+        step(i)
+    e1.record()
+    torch.cuda.synchronize()
+    t_wall = time.perf_counter() - t_wall0
+    ms_per_step = e0.elapsed_time(e1) / args.steps
+    assert torch.isfinite(out.float()).all()
+
+    gbs = kv_bytes / (ms_per_step * 1e-3) / 1e9
+    result = {
+        "metric": "paged TQ4 decode attn: us/layer + achieved HBM GB/s (% peak) at 128K ctx",
+        "value": round(gbs, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "us_per_layer": round(ms_per_step * 1e3, 3),
+        "pct_of_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16 MFMA operands (TQ4 codes -> fp16 centroids), f32 accumulate, bf16 Q/out",
+        "data": "synthetic",
+        "config": {
+            "workload": args.workload,
+            "requests": R,
+            "context_tokens_total": total_tokens_kv,
+            "q_heads": Q_HEADS, "kv_heads": KV_HEADS, "head_dim": HEAD_DIM, "page_tokens": BLOCK,
+            "kv_format": "tq4+wht256", "kv_pools_cycled": n_layers,
+            "kv_bytes_per_step": kv_bytes,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(gbs, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(gbs / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "kernel": "paged_attn_tq4_kernel (+ split_merge_kernel, both inside the timed launch)",
+            "avg_launch_us": round(ms_per_step * 1e3, 3),
+            "host_wall_us_per_step": round(t_wall / args.steps * 1e6, 2),
+        },
+    }
+    if not args.no_cpu_baseline:
+        import oracle
+
+        result["cpu_baseline"] = cpu_baseline(args.cpu_ctx, min(oracle.hw_threads(), 16))
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
