@@ -35,6 +35,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="tq4_decode_b1_ctx131072",
                     choices=["tq4_decode_b1_ctx131072", "tq4_decode_b32_ctx1k_64k"])
+    ap.add_argument("--ctx", type=int, default=0, help="override: one request with this context length")
     ap.add_argument("--layers", type=int, default=0, help="KV pools to cycle through (0 = auto, > 256 MB total)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-ctx", type=int, default=32768, help="context length of the CPU-oracle sample")
@@ -156,6 +157,9 @@ def main():
     dev = "cuda:0"
     torch.cuda.set_device(0)
     ctx = build_workload(args.workload)
+    if args.ctx:
+        ctx = np.array([args.ctx], dtype=np.int64)
+        args.workload = "tq4_decode_b1_ctx%d" % args.ctx
     total_tokens_kv = int(ctx.sum())
     kv_bytes = total_tokens_kv * KV_HEADS * 2 * ROW_BYTES  # algorithmic bytes per step (K + V rows)
     pool_pages = sum((int(c) + BLOCK - 1) // BLOCK for c in ctx) + 16

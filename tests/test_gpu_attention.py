@@ -1,6 +1,7 @@
 """GPU parity: paged GQA decode / verify attention through the C ABI vs the CPU oracle.
 
-Tolerance (BASELINE): |got - want| <= 2e-3 + 1e-2 |want| against the fp64-accumulating oracle.
+Tolerance (BASELINE): |got - want| <= 2e-3 * scale + 1e-2 |want| against the fp64-accumulating oracle,
+scale = magnitude of the V channel being averaged (1 on unit-scale data, see gpu_harness.assert_close).
 Invariants follow the reference's GPU tests: page-permutation 0-ULP
 (tests/backbone_and_collectives.rs:455-572), split vs single pass < 2e-3 and graph-bucket
 bound independence (tests/tq4_vision_and_moe.rs:1355-1663), masked rows untouched
@@ -38,7 +39,8 @@ def _check(fmt, dtype, block_size, seq_lens, q_lens, seed, scratch=SCRATCH, q_he
     dpool = _dev_pool(pool)
     rc, got, _ = G.dev_attention(dpool, hb, q, dtype, q_heads, scratch_bytes=scratch, **kw)
     assert rc == 0
-    err = G.assert_close(got, dtype, want, what="fmt=%d bs=%d seq=%s q=%s" % (fmt, block_size, seq_lens, q_lens))
+    err = G.assert_close(got, dtype, want, what="fmt=%d bs=%d seq=%s q=%s" % (fmt, block_size, seq_lens, q_lens),
+                         scale=G.channel_scale(v, dtype, hb, q_heads))
     return got, want, err
 
 

@@ -9,32 +9,37 @@
 //   tile  = up to TT consecutive query tokens of one request x the q heads of one kv head
 //           (16*NT MFMA columns; decode: 1 token x 8 heads -> 8 of 16 columns used)
 //   chunk = contiguous range of 32-token "units" of the tile's visible keys; one workgroup
-//           (4 waves) per (chunk, kv head, tile).  The number of chunks of a tile depends only
+//           (8 waves) per (chunk, kv head, tile).  The number of chunks of a tile depends only
 //           on the tile's own key range and on a host cap derived from total_tokens and the
 //           scratch size -- never on max_seq_len, max_blocks_per_req, physical page numbers or
 //           local_kv_heads -- so outputs are bit-identical under page permutation, graph-bucket
 //           bounds and head sharding (tests/tq4_vision_and_moe.rs:1089-1663).
 //   unit  = 32 consecutive tokens handled by ONE wave start to finish: the wave copies the
-//           raw K and V rows of the unit into its private LDS area (flat, coalesced 16-byte
-//           loads; next unit prefetched into registers), forms S^T = K Q'^T with MFMA, does the
-//           online softmax in registers and accumulates O^T += V^T P^T with MFMA.  Waves never
-//           synchronise inside the key loop; their (m, l, O) states are merged once at the end.
+//           raw K and V rows of the unit into its private LDS area (coalesced 16-byte loads
+//           from a wave-uniform base, next unit prefetched into registers), forms
+//           S^T = K Q'^T with MFMA, does the online softmax in registers and accumulates
+//           O^T += V^T P^T with MFMA.  Waves never synchronise inside the key loop; their
+//           (m, l, O) states are merged once at the end.
 //
 // TQ4 specifics (row = [fp16 d0][64 B nibbles][fp16 d1][64 B nibbles], 132 B, 33 dwords):
 //   * dequantisation is a 256-entry LDS table indexed by a code BYTE that returns the two
-//     centroids as packed fp16; the table is replicated once per LDS bank so random indices
-//     never conflict;
+//     centroids as packed fp16.  The table is replicated once per lane (entry stride 256 B) so
+//     that random indices never conflict and the address is a single v_perm_b32:
+//     addr = (byte << 8) | (lane << 2);
 //   * the per-128 scales are not applied per element: K scales multiply the two half-row
 //     partial scores, V scales are folded into the probabilities (two P matrices);
-//   * the first half of a row starts at byte 2, so aligned dwords straddle code words.  The
-//     K path treats the row as 33 aligned dwords and zeroes the query for the 8 nibble slots
-//     that hold scale bytes; the V path builds dword column 0 as [codes 0-3 | codes 124-127]
-//     from dwords 0 and 16, every other column is an aligned dword;
+//   * LDS reads must be dword aligned (misaligned ds_read_b32 is ~15x slower on this part)
+//     but the first half of a row starts at byte 2.  The K path therefore treats the row as 33
+//     aligned dwords and zeroes the query for the 8 nibble slots that hold scale bytes; the V
+//     path builds dword column 0 as [codes 0-3 | codes 124-127] from dwords 0 and 16, every
+//     other column is an aligned dword;
 //   * attention runs in the rotated domain: Q' = WHT(sign*q) once per tile, the output is
 //     un-rotated once at the end (op_kv_cache.cu:443-451,763-783).
 //
 // MFMA use: v_mfma_f32_16x16x32_f16.  A = K rows (QK) or V^T (PV) so that every lane owns one
 // query column: softmax state and the O rescale are per-lane scalars.
+#include <type_traits>
+
 #include "kv_common.h"
 
 namespace w34 {
@@ -45,17 +50,43 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 typedef float f2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 
-constexpr int kWaves = 4;            // waves per workgroup
-constexpr int kUnit = 32;            // tokens per wave iteration
-constexpr int kLutBytes = 256 * 128; // 256 entries x 32 bank replicas x 4 B
-constexpr int kStageTq4 = 2 * kUnit * kTq4RowBytes;  // K + V raw rows of one unit: 8448 B
+// waves per workgroup: 8 for one N tile (<= 256 VGPRs each), 4 for two N tiles (the second
+// tile's accumulators and operands need the full 512-register budget)
+__host__ __device__ constexpr int waves_for(int nt) { return nt == 1 ? 8 : 4; }
+constexpr int kUnit = 32;             // tokens per wave iteration
+constexpr int kLutBytes = 256 * 256;  // 256 entries x 64 lane replicas x 4 B
+constexpr int kRunBytes = 16 * kTq4RowBytes;  // 16 rows = 2112 B = 132 16-byte pieces
+constexpr int kStageTq4 = 4 * kRunBytes;      // K rows 0-31 then V rows 0-31: 8448 B
+__host__ __device__ constexpr int merge_floats_for(int nt) {
+    return waves_for(nt) * (nt * 16 * 258 + 8) + (waves_for(nt) + 1) * nt * 16 * 2;
+}
+__host__ __device__ constexpr int smem_bytes_for(int nt) {
+    const int loop_bytes = kLutBytes + waves_for(nt) * kStageTq4;
+    const int merge_bytes = merge_floats_for(nt) * 4;
+    return (loop_bytes > merge_bytes ? loop_bytes : merge_bytes) + 256;
+}
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kNegBig = -1.0e30f;  // "minus infinity" that stays finite under subtraction
-// The table holds fp16(kLutGain * centroid); the gain is folded back into the fp32 row scales.
-// 1.908032 minimises the worst fp16 rounding error of the eight centroid magnitudes
-// (9.4e-5 relative instead of 3.7e-4), which is what limits the accuracy of the scores.
+// The table holds fp16(kLutGain * centroid); the gain is divided out of the query (K side)
+// and of the final normalisation (V side).  1.908032 minimises the worst fp16 rounding error
+// of the eight centroid magnitudes (9.4e-5 relative instead of 3.7e-4), which is what limits
+// the accuracy of the scores.
 constexpr float kLutGain = 1.908032f;
 constexpr float kLutInvGain = 1.0f / kLutGain;
+
+#ifdef W34_TRACE
+__device__ unsigned long long g_trace[64 * 64];
+#define W34_TP(slot)                                                                   \
+    do {                                                                               \
+        if (lane == 0 && (blockIdx.x == 0 || blockIdx.x == 77) && blockIdx.y == 0) {  \
+            g_trace[((blockIdx.x ? 8 : 0) + wave) * 64 + (slot)] = __builtin_readcyclecounter(); \
+            if ((slot) == 0) g_trace[((blockIdx.x ? 8 : 0) + wave) * 64 + 63] = wall_clock64(); \
+            if ((slot) == 40) g_trace[((blockIdx.x ? 8 : 0) + wave) * 64 + 62] = wall_clock64(); \
+        }                                                                              \
+    } while (0)
+#else
+#define W34_TP(slot) do {} while (0)
+#endif
 
 struct AttnParams {
     warp34_kv_layer_layout L;
@@ -76,11 +107,11 @@ struct AttnParams {
 
 // token of k-slot (s, b, i) inside a unit: spreads the four 4-row groups of an MFMA over LDS
 // banks so that neither the K-row reads nor the V-column reads conflict.
-__device__ __forceinline__ int unit_token(int s, int b, int i) {
+__device__ __forceinline__ constexpr int unit_token(int s, int b, int i) {
     return 16 * (b & 1) + 8 * s + 4 * (b >> 1) + i;
 }
 
-// chunk geometry of a tile, identical in the attention and the merge kernel
+// chunk geometry of a tile
 struct ChunkGeom {
     int u_first, n_units, upc, n_chunks;
 };
@@ -124,53 +155,110 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
     h2 h = __builtin_convertvector(f, h2);
     return __builtin_bit_cast(uint32_t, h);
 }
+__device__ __forceinline__ float half_lo_to_f32(uint32_t w) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xFFFFu));
+}
+__device__ __forceinline__ float half_hi_to_f32(uint32_t w) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+}
+// max / sum over the four 16-lane rows of a wave, result in every lane (pure VALU on gfx950)
+__device__ __forceinline__ float max_over_rows(float x) {
+    auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_over_rows(float x) {
+    auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 
-__device__ __forceinline__ float half_bits_to_f32(uint32_t b) {
-    return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
+// Table lookup: the dequantisation table sits at LDS address 0 (it is the start of the dynamic
+// LDS block and the kernel has no static LDS), so the v_perm_b32 result IS the address.
+typedef __attribute__((address_space(3))) const uint32_t lds_cu32;
+typedef __attribute__((address_space(1))) const u4 global_cu4;
+__device__ __forceinline__ uint32_t lut_read(uint32_t code_word, uint32_t lut_lane, uint32_t sel) {
+    const uint32_t addr = __builtin_amdgcn_perm(code_word, lut_lane, sel);
+    return *reinterpret_cast<lds_cu32*>((uintptr_t)addr);
 }
 
 // element index (0..255) of nibble i of aligned dword D of a TQ4 row, -1 for scale nibbles
-__device__ __forceinline__ int tq4_dword_elem(int D, int i) {
+__device__ __forceinline__ constexpr int tq4_dword_elem(int D, int i) {
     if (D == 0) return i >= 4 ? i - 4 : -1;
     if (D < 16) return 8 * D - 4 + i;
     if (D == 16) return i < 4 ? 124 + i : -1;
     return 128 + 8 * (D - 17) + i;
 }
-// dword read by lane k-block bk for QK MFMA m of half h (h=0: m 0..4, h=1: m 0..3)
-__device__ __forceinline__ int tq4_qk_dword(int h, int m, int bk) {
+// dword read by k-block bk for QK MFMA m of half h (h=0: m 0..4, h=1: m 0..3).  The k-blocks of
+// lanes 0-31 (bk 0,1) sit 8 dwords apart, which keeps the 32 simultaneous reads on 32 banks.
+__device__ __forceinline__ constexpr int tq4_qk_dword(int h, int m, int bk) {
     const int base = 8 * (bk & 1) + 4 * (bk >> 1);
     if (h == 0) return m < 4 ? base + m : 16;
     return 17 + base + m;
 }
 // element index of V^T row r, nibble j, half h (PV MFMA output row -> head dimension)
-__device__ __forceinline__ int tq4_pv_elem(int h, int j, int r) {
+__device__ __forceinline__ constexpr int tq4_pv_elem(int h, int j, int r) {
     if (h == 1) return 128 + 8 * r + j;
     if (r == 0) return j < 4 ? j : 120 + j;
     return 8 * r - 4 + j;
 }
 
 template <typename TQ, int NT>
-__global__ __launch_bounds__(256, (NT == 1 ? 2 : 1)) void paged_attn_tq4_kernel(const AttnParams P) {
+__global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(const AttnParams P) {
+    constexpr int kWaves = waves_for(NT);
     extern __shared__ __align__(16) uint8_t smem[];
-    uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
     uint8_t* stage_all = smem + kLutBytes;  // kWaves * kStageTq4 bytes, reused by prologue/epilogue
+    // lut_read() addresses the table absolutely
+    if ((uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem != 0u) __builtin_trap();
 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int n = lane & 15;  // MFMA column = query row of this lane
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15;  // MFMA column = query row of this lane; also A-operand row
     const int b = lane >> 4;  // MFMA k-block / output row group
     const warp34_kv_layer_layout& L = P.L;
     const warp34_attention_batch& B = P.B;
 
-    // ---- tile identification ------------------------------------------------------------
+    // ---- tile identification (wave-uniform, scalar loads) -------------------------------------
     const int tok0 = (int)blockIdx.z;
     const int kv_sub = (int)blockIdx.y;
     const int kv_head = kv_sub / P.q_subgroups;
     const int q_head_base = kv_head * P.gqa + (kv_sub % P.q_subgroups) * P.q_group;
     const int chunk = (int)blockIdx.x;
 
+    W34_TP(0);
     if (tok0 >= B.total_tokens) return;
+
+    // Work that depends on nothing goes first so that it overlaps the request lookup below:
+    // the raw query rows of this wave's columns (validity is decided later) and the table.
+    constexpr int kColsPerWave = (16 * NT + kWaves - 1) / kWaves;
+    uint2 q_raw[kColsPerWave];
+#pragma unroll
+    for (int c = 0; c < kColsPerWave; ++c) {
+        const int col = wave + c * kWaves;
+        const int t = col / P.q_group;
+        const int a = col - t * P.q_group;
+        q_raw[c] = uint2{0u, 0u};
+        if (col < 16 * NT && tok0 + t < B.total_tokens) {
+            const uint16_t* qrow =
+                P.q + ((size_t)(tok0 + t) * P.num_q_heads + (size_t)(q_head_base + a)) * kHeadDim;
+            q_raw[c] = *reinterpret_cast<const uint2*>(qrow + 4 * lane);
+        }
+    }
+    {
+        // entry e = (gain*centroid[e & 15], gain*centroid[e >> 4]) as packed fp16, 64 copies
+        constexpr int kThreadsPerEntry = kWaves * 64 / 256;      // 2 or 1
+        constexpr int kBytesPerThread = 256 / kThreadsPerEntry;  // 128 or 256
+        const int e = tid / kThreadsPerEntry;
+        const uint32_t v = pack_h2(kLutGain * kCentroids[e & 15], kLutGain * kCentroids[e >> 4]);
+        u4 vv = {v, v, v, v};
+        u4* dst = reinterpret_cast<u4*>(smem + e * 256 + (tid % kThreadsPerEntry) * kBytesPerThread);
+#pragma unroll
+        for (int k = 0; k < kBytesPerThread / 16; ++k) dst[k] = vv;
+    }
+
     int rq_start = 0, rq_end = 0;
     const int req = find_request(B, tok0, rq_start, rq_end);
     if (req < 0) return;
@@ -178,89 +266,198 @@ __global__ __launch_bounds__(256, (NT == 1 ? 2 : 1)) void paged_attn_tq4_kernel(
     if (((tok0 - rq_start) % P.tok_tile) != 0) return;  // not a tile leader
     int tile_tokens = rq_end - tok0;
     if (tile_tokens > P.tok_tile) tile_tokens = P.tok_tile;
+    // every token of the tile belongs to request `req`: its ranges follow from two scalars
+    // (op_kv_cache.cu:406-424)
+    const int seq_after = B.seq_lens_after[req];
+    const int ctx_before =
+        B.context_lens_before != nullptr ? B.context_lens_before[req] : seq_after - (rq_end - rq_start);
 
     // per-lane column info (one column per N tile)
-    int col_lo[NT], col_hi[NT], col_tok[NT], col_qh[NT];
+    int col_lo[NT], col_hi[NT];
     bool col_ok[NT];
-    int u_lo = 0x7fffffff, u_hi = -1;
+    int u_lo = 0x7fffffff, u_hi = -1;  // union of the visible ranges
+    int i_lo = 0, i_hi = 0x7fffffff;   // intersection of the visible ranges
+    uint32_t ok_mask[NT];              // bit c: column nt*16+c is live (wave-uniform)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         const int col = nt * 16 + n;
         const int t = col / P.q_group;
-        const int a = col - t * P.q_group;
-        col_tok[nt] = tok0 + t;
-        col_qh[nt] = q_head_base + a;
-        col_ok[nt] = false;
-        col_lo[nt] = 0;
-        col_hi[nt] = -1;
-        if (t < tile_tokens) {
-            const RowRange rr = row_range(B, tok0 + t);
-            if (rr.req >= 0) {
-                col_ok[nt] = true;
-                col_lo[nt] = rr.min_kv;
-                col_hi[nt] = rr.max_kv;
+        const int tok = tok0 + t;
+        bool ok = t < tile_tokens;
+        if (ok && B.valid_token_mask != nullptr) ok = B.valid_token_mask[tok] != 0;
+        const int q_off = tok - rq_start;
+        int mx = (B.mask_mode == WARP34_ATTN_MASK_NONCAUSAL_WINDOW) ? seq_after - 1 : ctx_before + q_off;
+        if (mx >= seq_after) mx = seq_after - 1;
+        int mn = 0;
+        if (B.sliding_window > 0) mn = max(0, ctx_before + q_off - B.sliding_window + 1);
+        col_ok[nt] = ok;
+        col_lo[nt] = ok ? mn : 0;
+        col_hi[nt] = ok ? mx : -1;
+        if (ok) {
+            i_lo = max(i_lo, mn);
+            i_hi = min(i_hi, mx);
+            if (mn <= mx) {
+                u_lo = min(u_lo, mn);
+                u_hi = max(u_hi, mx);
             }
         }
-        if (col_ok[nt] && col_lo[nt] <= col_hi[nt]) {
-            u_lo = min(u_lo, col_lo[nt]);
-            u_hi = max(u_hi, col_hi[nt]);
-        }
+        ok_mask[nt] = (uint32_t)(__ballot(ok) & 0xFFFFull);
     }
-    // union over the 16 columns (lanes sharing b hold the same columns)
 #pragma unroll
     for (int off = 1; off < 16; off <<= 1) {
         u_lo = min(u_lo, __shfl_xor(u_lo, off, 64));
         u_hi = max(u_hi, __shfl_xor(u_hi, off, 64));
+        i_lo = max(i_lo, __shfl_xor(i_lo, off, 64));
+        i_hi = min(i_hi, __shfl_xor(i_hi, off, 64));
     }
-    bool any_ok = false;
+    {
+        uint32_t any = 0;
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) any_ok |= col_ok[nt];
-    if (__ballot(any_ok) == 0ull) return;  // whole tile masked: outputs untouched
+        for (int nt = 0; nt < NT; ++nt) any |= ok_mask[nt];
+        if (any == 0u) return;  // whole tile masked: outputs untouched
+    }
     if (u_hi < 0) u_lo = 0;
+    u_lo = __builtin_amdgcn_readfirstlane(u_lo);
+    u_hi = __builtin_amdgcn_readfirstlane(u_hi);
+    i_lo = __builtin_amdgcn_readfirstlane(i_lo);
+    i_hi = __builtin_amdgcn_readfirstlane(i_hi);
 
     const ChunkGeom g = chunk_geom(u_lo, u_hi, P.max_chunks, P.min_upc);
     if (chunk >= g.n_chunks) return;
     const int cu_first = g.u_first + chunk * g.upc;
     int cu_end = cu_first + g.upc;
     if (cu_end > g.u_first + g.n_units) cu_end = g.u_first + g.n_units;
+    W34_TP(1);
 
-    // ---- prologue: LUT, rotated queries ---------------------------------------------------
-    {
-        // thread t builds entry t: (centroid[t & 15], centroid[t >> 4]) as packed fp16
-        const uint32_t e = pack_h2(kLutGain * kCentroids[tid & 15], kLutGain * kCentroids[tid >> 4]);
-        u4 v = {e, e, e, e};
-        u4* dst = reinterpret_cast<u4*>(lut + tid * 32);
+    // ---- staging machinery ----------------------------------------------------------------------
+    const int32_t* req_blocks = B.block_tables + (size_t)req * B.max_blocks_per_req;
+    const uint8_t* k_base = reinterpret_cast<const uint8_t*>((uintptr_t)L.k_base) +
+                            (size_t)kv_head * L.k_head_stride_bytes;
+    const uint8_t* v_base = reinterpret_cast<const uint8_t*>((uintptr_t)L.v_base) +
+                            (size_t)kv_head * L.v_head_stride_bytes;
+    uint8_t* stage = stage_all + wave * kStageTq4;  // [K rows 0..31][V rows 0..31], 132 B each
+
+    // A unit is four contiguous runs of 16 rows (2112 B = 132 16-byte pieces): K rows 0-15,
+    // K rows 16-31, V rows 0-15, V rows 16-31.  Pieces 0-127 of every run are two full-wave
+    // loads from a wave-uniform base; the four tails (pieces 128-131) share one load.
+    // The physical page ids of a unit are fetched (scalar loads) one iteration before its data.
+    u4 pf[9];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) dst[k] = v;
+    for (int i = 0; i < 9; ++i) pf[i] = u4{0u, 0u, 0u, 0u};
+    auto lookup_pages = [&](int unit, int32_t (&pg)[2], int (&in_page)[2]) {
+#pragma unroll
+        for (int gidx = 0; gidx < 2; ++gidx) {
+            const int pos = unit * kUnit + 16 * gidx;
+            const int page_slot = pos / L.block_size;
+            in_page[gidx] = pos - page_slot * L.block_size;
+            // a run is fetched only when it overlaps the visible key range and its block
+            // table entry exists; everything else keeps stale (finite-by-construction) bytes
+            const bool live = unit < cu_end && pos <= u_hi && pos + 15 >= u_lo && page_slot < B.max_blocks_per_req;
+            pg[gidx] = live ? req_blocks[page_slot] : -1;
+        }
+    };
+    auto issue_loads = [&](const int32_t (&pg)[2], const int (&in_page)[2]) {
+        const uint8_t* run_ptr[4];
+#pragma unroll
+        for (int gidx = 0; gidx < 2; ++gidx) {
+            const bool live = pg[gidx] >= 0;
+            run_ptr[gidx] = live ? k_base + (size_t)pg[gidx] * L.k_page_stride_bytes +
+                                       (size_t)in_page[gidx] * L.k_token_stride_bytes
+                                 : nullptr;
+            run_ptr[2 + gidx] = live ? v_base + (size_t)pg[gidx] * L.v_page_stride_bytes +
+                                           (size_t)in_page[gidx] * L.v_token_stride_bytes
+                                     : nullptr;
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            if (run_ptr[r] != nullptr) {  // wave-uniform
+                pf[2 * r] = *(global_cu4*)(run_ptr[r] + 16 * lane);
+                pf[2 * r + 1] = *(global_cu4*)(run_ptr[r] + 1024 + 16 * lane);
+            }
+        }
+        {
+            const int r = lane >> 2;
+            const uint8_t* base = r == 0 ? run_ptr[0] : r == 1 ? run_ptr[1] : r == 2 ? run_ptr[2] : run_ptr[3];
+            if (lane < 16 && base != nullptr) pf[8] = *(global_cu4*)(base + 2048 + 16 * (lane & 3));
+        }
+    };
+    auto commit_loads = [&]() {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            *reinterpret_cast<u4*>(stage + r * kRunBytes + 16 * lane) = pf[2 * r];
+            *reinterpret_cast<u4*>(stage + r * kRunBytes + 1024 + 16 * lane) = pf[2 * r + 1];
+        }
+        if (lane < 16) *reinterpret_cast<u4*>(stage + (lane >> 2) * kRunBytes + 2048 + 16 * (lane & 3)) = pf[8];
+    };
+
+    // first unit's data goes in flight before the prologue work, the second unit's page ids too
+    int unit = cu_first + wave;
+    int32_t pg_next[2];
+    int inpage_next[2];
+    {
+        int32_t pg0[2];
+        int inpage0[2];
+        lookup_pages(unit, pg0, inpage0);
+        lookup_pages(unit + kWaves, pg_next, inpage_next);
+        issue_loads(pg0, inpage0);
     }
-    // rotated, fp16 query rows in LDS: [16*NT][264] halves (aliases the staging area)
+
+    // ---- prologue: rotated queries -------------------------------------------------------------
+    // The rotated fp16 queries are staged in the (still unused) staging area as [16*NT][264]
+    // halves.  All the constant factors of the scores (softmax scale, log2 e, 1 / table gain)
+    // go into Q'.
     constexpr int kQStride = 264;
     _Float16* qlds = reinterpret_cast<_Float16*>(stage_all);
-    for (int col = wave; col < 16 * NT; col += kWaves) {
-        const int t = col / P.q_group;
-        const int a = col - t * P.q_group;
-        float v[4] = {0.f, 0.f, 0.f, 0.f};
-        bool ok = false;
-        if (t < tile_tokens) {
-            const RowRange rr = row_range(B, tok0 + t);
-            ok = rr.req >= 0;
-        }
-        if (ok) {
-            const uint16_t* qrow =
-                P.q + ((size_t)(tok0 + t) * P.num_q_heads + (size_t)(q_head_base + a)) * kHeadDim;
-            const uint2 raw = *reinterpret_cast<const uint2*>(qrow + 4 * lane);
-            v[0] = TQ::to_f32((uint16_t)(raw.x & 0xFFFFu));
-            v[1] = TQ::to_f32((uint16_t)(raw.x >> 16));
-            v[2] = TQ::to_f32((uint16_t)(raw.y & 0xFFFFu));
-            v[3] = TQ::to_f32((uint16_t)(raw.y >> 16));
+    const float q_scale = B.sm_scale * kLog2e * kLutInvGain;
+    {
+        float v[kColsPerWave][4];
+        bool okc[kColsPerWave];
 #pragma unroll
-            for (int k = 0; k < 4; ++k) v[k] = apply_sign(v[k], 4 * lane + k);
-            wht256_wave(v, lane);
+        for (int c = 0; c < kColsPerWave; ++c) {
+            const int col = wave + c * kWaves;
+            okc[c] = col < 16 * NT && ((ok_mask[(col >> 4) & (NT - 1)] >> (col & 15)) & 1u);
+            v[c][0] = TQ::to_f32((uint16_t)(q_raw[c].x & 0xFFFFu));
+            v[c][1] = TQ::to_f32((uint16_t)(q_raw[c].x >> 16));
+            v[c][2] = TQ::to_f32((uint16_t)(q_raw[c].y & 0xFFFFu));
+            v[c][3] = TQ::to_f32((uint16_t)(q_raw[c].y >> 16));
+#pragma unroll
+            for (int k = 0; k < 4; ++k) v[c][k] = okc[c] ? apply_sign(v[c][k], 4 * lane + k) : 0.f;
         }
-        uint2 packed;
-        packed.x = pack_h2(v[0], v[1]);
-        packed.y = pack_h2(v[2], v[3]);
-        *reinterpret_cast<uint2*>(qlds + col * kQStride + 4 * lane) = packed;
+        bool any_col = false;
+#pragma unroll
+        for (int c = 0; c < kColsPerWave; ++c) any_col |= okc[c];
+        if (any_col) {  // wave-uniform; the columns of a wave are transformed together
+#pragma unroll
+            for (int c = 0; c < kColsPerWave; ++c) {
+                const float a0 = v[c][0] + v[c][1], a1 = v[c][0] - v[c][1];
+                const float a2 = v[c][2] + v[c][3], a3 = v[c][2] - v[c][3];
+                v[c][0] = a0 + a2;
+                v[c][1] = a1 + a3;
+                v[c][2] = a0 - a2;
+                v[c][3] = a1 - a3;
+            }
+#pragma unroll
+            for (int h = 1; h < 64; h <<= 1) {
+#pragma unroll
+                for (int c = 0; c < kColsPerWave; ++c) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const float o = __shfl_xor(v[c][k], h, 64);
+                        v[c][k] = (lane & h) ? (o - v[c][k]) : (v[c][k] + o);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < kColsPerWave; ++c) {
+            const int col = wave + c * kWaves;
+            if (col < 16 * NT) {
+                uint2 packed;
+                packed.x = pack_h2(v[c][0] * (0.0625f * q_scale), v[c][1] * (0.0625f * q_scale));
+                packed.y = pack_h2(v[c][2] * (0.0625f * q_scale), v[c][3] * (0.0625f * q_scale));
+                *reinterpret_cast<uint2*>(qlds + col * kQStride + 4 * lane) = packed;
+            }
+        }
     }
     __syncthreads();
 
@@ -283,12 +480,11 @@ __global__ __launch_bounds__(256, (NT == 1 ? 2 : 1)) void paged_attn_tq4_kernel(
             bq[nt][mf] = x;
         }
     }
-    __syncthreads();  // qlds is dead, the staging area may be overwritten
+    __syncthreads();  // qlds is dead, the staging area may be overwritten; the table is complete
+    W34_TP(2);
 
     // ---- per-wave state -----------------------------------------------------------------------
-    uint8_t* stage = stage_all + wave * kStageTq4;  // [K rows 0..31][V rows 0..31], 132 B each
-    const uint32_t lut_lane = (uint32_t)(lane & 31);
-    const float score_scale = B.sm_scale * kLog2e * kLutInvGain;
+    const uint32_t lut_lane = (uint32_t)lane << 2;  // byte 0 of every table address
 
     f4 o_acc[NT][2][8];
     float m_run[NT], l_run[NT];
@@ -302,115 +498,91 @@ __global__ __launch_bounds__(256, (NT == 1 ? 2 : 1)) void paged_attn_tq4_kernel(
             for (int j = 0; j < 8; ++j) o_acc[nt][h][j] = f4{0.f, 0.f, 0.f, 0.f};
     }
 
-    const int32_t* req_blocks = B.block_tables + (size_t)req * B.max_blocks_per_req;
-    const uint8_t* k_base = reinterpret_cast<const uint8_t*>((uintptr_t)L.k_base) +
-                            (size_t)kv_head * L.k_head_stride_bytes;
-    const uint8_t* v_base = reinterpret_cast<const uint8_t*>((uintptr_t)L.v_base) +
-                            (size_t)kv_head * L.v_head_stride_bytes;
-
-    // Staging copy: the unit is 4 contiguous runs of 16 rows (2112 B = 132 16-byte pieces):
-    // K rows 0-15, K rows 16-31, V rows 0-15, V rows 16-31.  Piece c = lane + 64 i of the
-    // 528 pieces belongs to run c / 132.
-    constexpr int kPieces = 9;  // ceil(528 / 64)
-    u4 pf[kPieces];
-    auto issue_loads = [&](int unit) {
-        const int t0 = unit * kUnit;
-        const uint8_t* run_ptr[4];
-#pragma unroll
-        for (int gidx = 0; gidx < 2; ++gidx) {
-            const int pos = t0 + 16 * gidx;
-            const int page_slot = pos / L.block_size;
-            const int in_page = pos - page_slot * L.block_size;
-            // a run is fetched only when it overlaps the visible key range and its block
-            // table entry exists; everything else keeps stale (finite-by-construction) bytes
-            bool live = pos <= u_hi && pos + 15 >= u_lo && page_slot < B.max_blocks_per_req;
-            const int32_t page = live ? req_blocks[page_slot] : -1;
-            live = live && page >= 0;
-            run_ptr[gidx] = live ? k_base + (size_t)page * L.k_page_stride_bytes +
-                                       (size_t)in_page * L.k_token_stride_bytes
-                                 : nullptr;
-            run_ptr[2 + gidx] = live ? v_base + (size_t)page * L.v_page_stride_bytes +
-                                           (size_t)in_page * L.v_token_stride_bytes
-                                     : nullptr;
-        }
-#pragma unroll
-        for (int i = 0; i < kPieces; ++i) {
-            const int c = lane + 64 * i;
-            const int run = c / 132;
-            const int idx = c - run * 132;
-            const uint8_t* base = run == 0 ? run_ptr[0] : run == 1 ? run_ptr[1] : run == 2 ? run_ptr[2] : run_ptr[3];
-            u4 v = {0u, 0u, 0u, 0u};
-            if (c < 528 && base != nullptr) v = *reinterpret_cast<const u4*>(base + 16 * idx);
-            pf[i] = v;
-        }
-    };
-    auto commit_loads = [&]() {
-#pragma unroll
-        for (int i = 0; i < kPieces; ++i) {
-            const int c = lane + 64 * i;
-            if (c < 528) *reinterpret_cast<u4*>(stage + 16 * c) = pf[i];
-        }
-    };
-
-    int unit = cu_first + wave;
-    if (unit < cu_end) issue_loads(unit);
-
-    for (; unit < cu_end; unit += kWaves) {
-        commit_loads();
-        if (unit + kWaves < cu_end) issue_loads(unit + kWaves);
-        const int t0 = unit * kUnit;
+#ifdef W34_TRACE
+    int trace_it = 0;
+#endif
+    // one 32-token unit.  MASKED = false (wave-uniform) is the interior case: every token of the
+    // unit is visible to every live column, so the compares / selects are branched over.
+    auto process_unit = [&](int t0, const bool MASKED) {
         const uint8_t* k_rows = stage;
-        const uint8_t* v_rows = stage + kUnit * kTq4RowBytes;
+        const uint8_t* v_rows = stage + 2 * kRunBytes;
 
         // ---- S^T = K Q'^T for the two 16-key sub-tiles ------------------------------------
+        // Phase structure (few, large LDS batches so that one s_waitcnt covers many reads):
+        // all raw K dwords and K scales -> per sub-tile 36 table reads -> 9 MFMAs.
         float sc[NT][8];
-        {
+        uint32_t kw[2][9], ks0[2][4], ks16[2][4];
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                const int arow = unit_token(s, n >> 2, n & 3);  // A row n of sub-tile s
-                const uint32_t* row32 = reinterpret_cast<const uint32_t*>(k_rows + arow * kTq4RowBytes);
-                f4 s_acc[NT][2];
+        for (int s = 0; s < 2; ++s) {
+            const int arow = unit_token(s, n >> 2, n & 3);  // A row n of sub-tile s
+            const uint32_t* row32 = reinterpret_cast<const uint32_t*>(k_rows + arow * kTq4RowBytes);
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    s_acc[nt][0] = f4{0.f, 0.f, 0.f, 0.f};
-                    s_acc[nt][1] = f4{0.f, 0.f, 0.f, 0.f};
-                }
+            for (int mf = 0; mf < 9; ++mf) kw[s][mf] = row32[tq4_qk_dword(mf < 5 ? 0 : 1, mf < 5 ? mf : mf - 5, b)];
 #pragma unroll
-                for (int mf = 0; mf < 9; ++mf) {
-                    const int h = mf < 5 ? 0 : 1;
-                    const int m = mf < 5 ? mf : mf - 5;
-                    const uint32_t w = row32[tq4_qk_dword(h, m, b)];
-                    u4 a;
-                    a[0] = lut[((w & 0xFFu) << 5) + lut_lane];
-                    a[1] = lut[(((w >> 8) & 0xFFu) << 5) + lut_lane];
-                    a[2] = lut[(((w >> 16) & 0xFFu) << 5) + lut_lane];
-                    a[3] = lut[((w >> 24) << 5) + lut_lane];
-                    const h8 av = __builtin_bit_cast(h8, a);
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t* r32 =
+                    reinterpret_cast<const uint32_t*>(k_rows + unit_token(s, b, i) * kTq4RowBytes);
+                ks0[s][i] = r32[0];
+                ks16[s][i] = r32[16];
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#ifdef W34_TRACE
+        if (trace_it < 8) W34_TP(4 + 4 * trace_it + 1);
+#endif
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            u4 a[9];
+#pragma unroll
+            for (int mf = 0; mf < 9; ++mf) {
+                const uint32_t w = kw[s][mf];
+                a[mf][0] = lut_read(w, lut_lane, 0x0c0c0400u);
+                a[mf][1] = lut_read(w, lut_lane, 0x0c0c0500u);
+                a[mf][2] = lut_read(w, lut_lane, 0x0c0c0600u);
+                a[mf][3] = lut_read(w, lut_lane, 0x0c0c0700u);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            f4 s_acc[NT][2];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                s_acc[nt][0] = f4{0.f, 0.f, 0.f, 0.f};
+                s_acc[nt][1] = f4{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int m = 0; m < 5; ++m) {
+                // alternate the two half-row accumulators so consecutive MFMAs are independent
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    if (h == 1 && m == 4) continue;
+                    const int mf = h == 0 ? m : 5 + m;
+                    const h8 av = __builtin_bit_cast(h8, a[mf]);
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt) {
                         s_acc[nt][h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bq[nt][mf], s_acc[nt][h], 0, 0, 0);
                     }
                 }
-                // rows 4b+i of the result are tokens unit_token(s, b, i); apply the K scales
+            }
+            // rows 4b+i of the result are tokens unit_token(s, b, i); apply the K scales
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int trow = unit_token(s, b, i);
-                    const uint16_t* r16 = reinterpret_cast<const uint16_t*>(k_rows + trow * kTq4RowBytes);
-                    const float d0 = half_bits_to_f32(r16[0]) * score_scale;
-                    const float d1 = half_bits_to_f32(r16[33]) * score_scale;
-                    const int pos = t0 + trow;
+            for (int i = 0; i < 4; ++i) {
+                const int trow = unit_token(s, b, i);
+                const float d0 = half_lo_to_f32(ks0[s][i]);
+                const float d1 = half_hi_to_f32(ks16[s][i]);
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) {
-                        const float v = d0 * s_acc[nt][0][i] + d1 * s_acc[nt][1][i];
+                for (int nt = 0; nt < NT; ++nt) {
+                    const float v = d0 * s_acc[nt][0][i] + d1 * s_acc[nt][1][i];
+                    if (MASKED) {
+                        const int pos = t0 + trow;
                         const bool vis = col_ok[nt] && pos >= col_lo[nt] && pos <= col_hi[nt];
                         sc[nt][4 * s + i] = vis ? v : kNegBig;
+                    } else {
+                        sc[nt][4 * s + i] = v;
                     }
                 }
             }
         }
 
-        // ---- online softmax (log2 domain), per lane = per query column --------------------
-        // V scales of this lane's 8 tokens and the raw V dwords
+        // ---- raw V dwords of this lane's 8 tokens ------------------------------------------
         uint32_t vd0[8], vd16[8], vwr[8], vw1[8];
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
@@ -418,17 +590,17 @@ __global__ __launch_bounds__(256, (NT == 1 ? 2 : 1)) void paged_attn_tq4_kernel(
             const uint32_t* row32 = reinterpret_cast<const uint32_t*>(v_rows + trow * kTq4RowBytes);
             vd0[t] = row32[0];
             vd16[t] = row32[16];
-            vwr[t] = row32[n];       // n == 0 re-reads dword 0
+            vwr[t] = row32[n];  // n == 0 re-reads dword 0
             vw1[t] = row32[17 + n];
         }
+
+        // ---- online softmax (log2 domain), per lane = per query column --------------------
         uint32_t pb[NT][2][4];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-            float mx = sc[nt][0];
-#pragma unroll
-            for (int t = 1; t < 8; ++t) mx = fmaxf(mx, sc[nt][t]);
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            float mx = fmaxf(fmaxf(fmaxf(sc[nt][0], sc[nt][1]), fmaxf(sc[nt][2], sc[nt][3])),
+                             fmaxf(fmaxf(sc[nt][4], sc[nt][5]), fmaxf(sc[nt][6], sc[nt][7])));
+            mx = max_over_rows(mx);
             const float m_new = fmaxf(m_run[nt], mx);
             const float alpha = __builtin_amdgcn_exp2f(m_run[nt] - m_new);
             m_run[nt] = m_new;
@@ -436,7 +608,11 @@ __global__ __launch_bounds__(256, (NT == 1 ? 2 : 1)) void paged_attn_tq4_kernel(
             float psum = 0.f;
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
-                p[t] = sc[nt][t] > 0.5f * kNegBig ? __builtin_amdgcn_exp2f(sc[nt][t] - m_new) : 0.f;
+                if (MASKED) {
+                    p[t] = sc[nt][t] > 0.5f * kNegBig ? __builtin_amdgcn_exp2f(sc[nt][t] - m_new) : 0.f;
+                } else {
+                    p[t] = __builtin_amdgcn_exp2f(sc[nt][t] - m_new);
+                }
                 psum += p[t];
             }
             l_run[nt] = l_run[nt] * alpha + psum;
@@ -448,19 +624,27 @@ __global__ __launch_bounds__(256, (NT == 1 ? 2 : 1)) void paged_attn_tq4_kernel(
             }
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                const float d0a = half_bits_to_f32(vd0[2 * k] & 0xFFFFu) * kLutInvGain;
-                const float d0b = half_bits_to_f32(vd0[2 * k + 1] & 0xFFFFu) * kLutInvGain;
-                const float d1a = half_bits_to_f32(vd16[2 * k] >> 16) * kLutInvGain;
-                const float d1b = half_bits_to_f32(vd16[2 * k + 1] >> 16) * kLutInvGain;
-                // masked tokens have p == 0; select instead of multiply so that a garbage
-                // scale (rows beyond the sequence end) cannot inject NaN
-                pb[nt][0][k] = pack_h2(p[2 * k] > 0.f ? p[2 * k] * d0a : 0.f,
-                                       p[2 * k + 1] > 0.f ? p[2 * k + 1] * d0b : 0.f);
-                pb[nt][1][k] = pack_h2(p[2 * k] > 0.f ? p[2 * k] * d1a : 0.f,
-                                       p[2 * k + 1] > 0.f ? p[2 * k + 1] * d1b : 0.f);
+                const float d0a = half_lo_to_f32(vd0[2 * k]);
+                const float d0b = half_lo_to_f32(vd0[2 * k + 1]);
+                const float d1a = half_hi_to_f32(vd16[2 * k]);
+                const float d1b = half_hi_to_f32(vd16[2 * k + 1]);
+                if (MASKED) {
+                    // masked tokens have p == 0; select instead of multiply so that a garbage
+                    // scale (rows beyond the sequence end) cannot inject NaN
+                    pb[nt][0][k] = pack_h2(p[2 * k] > 0.f ? p[2 * k] * d0a : 0.f,
+                                           p[2 * k + 1] > 0.f ? p[2 * k + 1] * d0b : 0.f);
+                    pb[nt][1][k] = pack_h2(p[2 * k] > 0.f ? p[2 * k] * d1a : 0.f,
+                                           p[2 * k + 1] > 0.f ? p[2 * k + 1] * d1b : 0.f);
+                } else {
+                    pb[nt][0][k] = pack_h2(p[2 * k] * d0a, p[2 * k + 1] * d0b);
+                    pb[nt][1][k] = pack_h2(p[2 * k] * d1a, p[2 * k + 1] * d1b);
+                }
             }
         }
 
+#ifdef W34_TRACE
+        if (trace_it < 8) W34_TP(4 + 4 * trace_it + 2);
+#endif
         // ---- O^T += V^T P^T ------------------------------------------------------------------
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
@@ -481,16 +665,20 @@ __global__ __launch_bounds__(256, (NT == 1 ? 2 : 1)) void paged_attn_tq4_kernel(
                 lo[k] = (wa & 0x0F0F0F0Fu) | ((wb << 4) & 0xF0F0F0F0u);
                 hi[k] = ((wa >> 4) & 0x0F0F0F0Fu) | (wb & 0xF0F0F0F0u);
             }
+            u4 a[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                u4 a;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const uint32_t src = (j & 1) ? hi[k] : lo[k];
-                    const uint32_t byte = (src >> (8 * (j >> 1))) & 0xFFu;
-                    a[k] = lut[(byte << 5) + lut_lane];
+                    const uint32_t sel = 0x0c0c0400u + ((uint32_t)(j >> 1) << 8);
+                    a[j][k] = lut_read(src, lut_lane, sel);
                 }
-                const h8 av = __builtin_bit_cast(h8, a);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const h8 av = __builtin_bit_cast(h8, a[j]);
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
                     u4 pbv = {pb[nt][h][0], pb[nt][h][1], pb[nt][h][2], pb[nt][h][3]};
@@ -499,107 +687,115 @@ __global__ __launch_bounds__(256, (NT == 1 ? 2 : 1)) void paged_attn_tq4_kernel(
                 }
             }
         }
+    };
+
+
+    for (; unit < cu_end; unit += kWaves) {
+        commit_loads();
+#ifdef W34_TRACE
+        if (trace_it < 8) W34_TP(4 + 4 * trace_it);
+#endif
+        // next unit's data (page ids were fetched one iteration ago), next-next unit's page ids
+        issue_loads(pg_next, inpage_next);
+        lookup_pages(unit + 2 * kWaves, pg_next, inpage_next);
+        const int t0 = unit * kUnit;
+        process_unit(t0, !(t0 >= i_lo && t0 + kUnit - 1 <= i_hi));
+#ifdef W34_TRACE
+        if (trace_it < 8) W34_TP(4 + 4 * trace_it + 3);
+        ++trace_it;
+#endif
     }
+    W34_TP(36);
 
     // ---- combine the per-lane partial sums of l over the four k-block lanes of a column ------
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        l_run[nt] += __shfl_xor(l_run[nt], 16, 64);
-        l_run[nt] += __shfl_xor(l_run[nt], 32, 64);
-    }
+    for (int nt = 0; nt < NT; ++nt) l_run[nt] = sum_over_rows(l_run[nt]);
 
-    // ---- merge the waves' states through LDS (pairwise tree), result in wave 0 ----------------
-    __syncthreads();  // every wave is done with its staging area
-    // [2 senders][NT*16 cols][258] floats; overlays the LUT and the staging areas, both dead now
-    float* xbuf = reinterpret_cast<float*>(smem);
+    // ---- merge the waves' states through LDS ---------------------------------------------------
+    // Every wave publishes (m, l), rescales its O by 2^(m - m_tot) and stores it in its own
+    // region; then the waves split the columns and add the regions up in wave order.
+    // Region layout: element e of column c at dword c*258 + (e ^ ((e >> 5) & 1)): the lanes of a
+    // half-wave store (16 columns x 2 row groups that are 32 elements apart) hit 32 distinct
+    // banks.
+    __syncthreads();  // every wave is done with the table and with its staging area
     constexpr int kColStride = 258;
-#pragma unroll
-    for (int round = 0; round < 2; ++round) {
-        const int senders_lo = round == 0 ? 2 : 1;  // waves [senders_lo, 2*senders_lo) send
-        const int nsend = senders_lo;
-        if (wave >= senders_lo && wave < 2 * senders_lo) {
-            float* dst = xbuf + (size_t)(wave - senders_lo) * (NT * 16 * kColStride);
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                float* c = dst + (nt * 16 + n) * kColStride;
-#pragma unroll
-                for (int h = 0; h < 2; ++h)
-#pragma unroll
-                    for (int j = 0; j < 8; ++j)
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) c[tq4_pv_elem(h, j, 4 * b + i)] = o_acc[nt][h][j][i];
-                if (b == 0) {
-                    c[256] = m_run[nt];
-                    c[257] = l_run[nt];
-                }
-            }
-        }
-        __syncthreads();
-        if (wave < nsend) {
-            const float* src = xbuf + (size_t)wave * (NT * 16 * kColStride);
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const float* c = src + (nt * 16 + n) * kColStride;
-                const float m2 = c[256], l2 = c[257];
-                const float m_new = fmaxf(m_run[nt], m2);
-                const float w1 = __builtin_amdgcn_exp2f(m_run[nt] - m_new);
-                const float w2 = __builtin_amdgcn_exp2f(m2 - m_new);
-#pragma unroll
-                for (int h = 0; h < 2; ++h)
-#pragma unroll
-                    for (int j = 0; j < 8; ++j)
-#pragma unroll
-                        for (int i = 0; i < 4; ++i)
-                            o_acc[nt][h][j][i] = o_acc[nt][h][j][i] * w1 + c[tq4_pv_elem(h, j, 4 * b + i)] * w2;
-                l_run[nt] = l_run[nt] * w1 + l2 * w2;
-                m_run[nt] = m_new;
-            }
-        }
-        __syncthreads();
-    }
-
-    // ---- epilogue ----------------------------------------------------------------------------
-    // wave 0 publishes the tile state as [col][258] floats, then all waves either store the
-    // split partial or finish the rows (normalise, un-rotate, convert).
-    if (wave == 0) {
+    constexpr int kRegion = NT * 16 * kColStride + 8;
+    float* xbuf = reinterpret_cast<float*>(smem);
+    float* mlbuf = xbuf + kWaves * kRegion;  // [kWaves][NT*16][2]
+    static_assert(kWaves * kRegion + (kWaves + 1) * NT * 16 * 2 == merge_floats_for(NT), "merge layout");
+    static_assert(smem_bytes_for(NT) >= merge_floats_for(NT) * 4, "merge buffer must fit");
+    if (b == 0) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-            float* c = xbuf + (nt * 16 + n) * kColStride;
-#pragma unroll
-            for (int h = 0; h < 2; ++h)
-#pragma unroll
-                for (int j = 0; j < 8; ++j)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) c[tq4_pv_elem(h, j, 4 * b + i)] = o_acc[nt][h][j][i];
-            if (b == 0) {
-                c[256] = m_run[nt];
-                c[257] = l_run[nt];
-            }
+            mlbuf[(wave * NT * 16 + nt * 16 + n) * 2 + 0] = m_run[nt];
+            mlbuf[(wave * NT * 16 + nt * 16 + n) * 2 + 1] = l_run[nt];
         }
     }
     __syncthreads();
+    float m_tot[NT], l_tot[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        float mt = kNegBig;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) mt = fmaxf(mt, mlbuf[(w * NT * 16 + nt * 16 + n) * 2]);
+        float lt = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w)
+            lt += mlbuf[(w * NT * 16 + nt * 16 + n) * 2 + 1] *
+                  __builtin_amdgcn_exp2f(mlbuf[(w * NT * 16 + nt * 16 + n) * 2] - mt);
+        m_tot[nt] = mt;
+        l_tot[nt] = lt;
+        const float wgt = __builtin_amdgcn_exp2f(m_run[nt] - mt);
+        float* c = xbuf + wave * kRegion + (nt * 16 + n) * kColStride;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int e = tq4_pv_elem(h, j, 4 * b + i);
+                    c[e ^ ((e >> 5) & 1)] = o_acc[nt][h][j][i] * wgt;
+                }
+    }
+    // (m_tot, l_tot) of every column for the epilogue, read back by column below
+    float* mltot = mlbuf + kWaves * NT * 16 * 2;
+    if (wave == 0 && b == 0) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            mltot[(nt * 16 + n) * 2 + 0] = m_tot[nt];
+            mltot[(nt * 16 + n) * 2 + 1] = l_tot[nt];
+        }
+    }
+    __syncthreads();
+    W34_TP(37);
+
+    // ---- epilogue: per column, add the regions, then store the partial or finish the row -------
     for (int col = wave; col < 16 * NT; col += kWaves) {
         const int t = col / P.q_group;
         const int a = col - t * P.q_group;
-        if (t >= tile_tokens) continue;
-        const RowRange rr = row_range(B, tok0 + t);
-        if (rr.req < 0) continue;
+        if (!((ok_mask[col >> 4] >> (col & 15)) & 1u)) continue;
         const size_t row = (size_t)(tok0 + t) * P.num_q_heads + (size_t)(q_head_base + a);
-        const float* c = xbuf + col * kColStride;
-        float v[4];
+        float v[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int k = 0; k < 4; ++k) v[k] = c[4 * lane + k];
+        for (int w = 0; w < kWaves; ++w) {
+            const float* c = xbuf + w * kRegion + col * kColStride + 4 * lane;
+            const int f = (lane >> 3) & 1;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) v[k] += c[k ^ f];
+        }
+        const float m_col = mltot[col * 2 + 0];
+        const float l_col = mltot[col * 2 + 1];
         if (P.max_chunks > 1) {
+            // un-normalised, rotated, still carrying the table gain; the merge kernel finishes
             float* dst = P.part_acc + (row * P.max_chunks + chunk) * kHeadDim;
             *reinterpret_cast<f4*>(dst + 4 * lane) = f4{v[0], v[1], v[2], v[3]};
             if (lane == 0) {
-                P.part_ml[(row * P.max_chunks + chunk) * 2 + 0] = c[256];
-                P.part_ml[(row * P.max_chunks + chunk) * 2 + 1] = c[257];
+                P.part_ml[(row * P.max_chunks + chunk) * 2 + 0] = m_col;
+                P.part_ml[(row * P.max_chunks + chunk) * 2 + 1] = l_col;
                 if (chunk == 0) P.part_cnt[row] = g.n_chunks;
             }
         } else {
-            const float l = c[257];
-            const float inv = l > 0.f ? 1.0f / l : 0.f;
+            const float inv = l_col > 0.f ? kLutInvGain / l_col : 0.f;
 #pragma unroll
             for (int k = 0; k < 4; ++k) v[k] *= inv;
             wht256_wave(v, lane);
@@ -611,56 +807,86 @@ __global__ __launch_bounds__(256, (NT == 1 ? 2 : 1)) void paged_attn_tq4_kernel(
             *reinterpret_cast<uint2*>(P.out + row * kHeadDim + 4 * lane) = o;
         }
     }
+    W34_TP(40);
 }
 
-// Merge of the split-K partials of one (token, q head) row per wave
-// (op_paged_attn.cu:1132-1218): m_tot = max m_s, w_s = 2^(m_s - m_tot),
-// out = sum acc_s w_s / sum l_s w_s, then one inverse rotation.
+#ifdef W34_TRACE
+extern "C" int warp34_debug_read_trace(unsigned long long* dst) {
+    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_trace), sizeof(unsigned long long) * 64 * 64);
+}
+#endif
+
+// Merge of the split-K partials (op_paged_attn.cu:1132-1218): m_tot = max m_s,
+// w_s = 2^(m_s - m_tot), out = sum acc_s w_s / sum l_s w_s, then one inverse rotation.
+// One workgroup of 1024 threads per (token, q head) row: 16 groups of 64 threads stride the
+// chunks, each thread owns 4 of the 256 columns; the groups are summed through LDS.
+constexpr int kMergeGroups = 16;
 template <typename TQ>
-__global__ __launch_bounds__(256) void split_merge_kernel(const AttnParams P, int rotate) {
+__global__ __launch_bounds__(1024) void split_merge_kernel(const AttnParams P, float out_scale, int rotate) {
+    __shared__ f4 s_acc[kMergeGroups][64];
+    __shared__ float s_red[kMergeGroups];
     const int lane = (int)(threadIdx.x & 63);
-    const int wave = (int)(threadIdx.x >> 6);
-    const long long row = (long long)blockIdx.x * 4 + wave;
-    const long long rows = (long long)P.B.total_tokens * P.num_q_heads;
-    if (row >= rows) return;
+    const int grp = (int)(threadIdx.x >> 6);
+    const long long row = (long long)blockIdx.x;
     const int tok = (int)(row / P.num_q_heads);
     const RowRange rr = row_range(P.B, tok);
-    if (rr.req < 0) return;
+    if (rr.req < 0) return;  // masked row: output untouched (uniform for the block)
     const int n_chunks = P.part_cnt[row];
     const float* ml = P.part_ml + (size_t)row * P.max_chunks * 2;
     const float* acc = P.part_acc + (size_t)row * P.max_chunks * kHeadDim;
+
+    // pass 1: global maximum of m over chunks with l > 0
+    float m_loc = kNegBig;
+    for (int s = (int)threadIdx.x; s < n_chunks; s += 1024)
+        if (ml[2 * s + 1] > 0.f) m_loc = fmaxf(m_loc, ml[2 * s]);
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) m_loc = fmaxf(m_loc, __shfl_xor(m_loc, off, 64));
+    if (lane == 0) s_red[grp] = m_loc;
+    __syncthreads();
     float m_tot = kNegBig;
-    for (int s = 0; s < n_chunks; ++s)
-        if (ml[2 * s + 1] > 0.f) m_tot = fmaxf(m_tot, ml[2 * s]);
-    float v[4] = {0.f, 0.f, 0.f, 0.f};
-    float l_tot = 0.f;
-    for (int s = 0; s < n_chunks; ++s) {
+#pragma unroll
+    for (int k = 0; k < kMergeGroups; ++k) m_tot = fmaxf(m_tot, s_red[k]);
+    __syncthreads();
+
+    // pass 2: weighted sums
+    f4 v = {0.f, 0.f, 0.f, 0.f};
+    float l_part = 0.f;
+    for (int s = grp; s < n_chunks; s += kMergeGroups) {
         const float ls = ml[2 * s + 1];
         if (!(ls > 0.f)) continue;
         const float w = __builtin_amdgcn_exp2f(ml[2 * s] - m_tot);
-        l_tot += ls * w;
+        l_part += ls * w;
         const f4 a = *reinterpret_cast<const f4*>(acc + (size_t)s * kHeadDim + 4 * lane);
-#pragma unroll
-        for (int k = 0; k < 4; ++k) v[k] += a[k] * w;
+        v += a * w;
     }
-    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+    s_acc[grp][lane] = v;
+    if (lane == 0) s_red[grp] = l_part;
+    __syncthreads();
+    if (grp != 0) return;
+    float l_tot = 0.f;
+    f4 tot = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int k = 0; k < 4; ++k) v[k] *= inv;
+    for (int k = 0; k < kMergeGroups; ++k) {
+        tot += s_acc[k][lane];
+        l_tot += s_red[k];
+    }
+    const float inv = l_tot > 0.f ? out_scale / l_tot : 0.f;
+    float o[4] = {tot[0] * inv, tot[1] * inv, tot[2] * inv, tot[3] * inv};
     if (rotate) {
-        wht256_wave(v, lane);
+        wht256_wave(o, lane);
 #pragma unroll
-        for (int k = 0; k < 4; ++k) v[k] = apply_sign(v[k], 4 * lane + k);
+        for (int k = 0; k < 4; ++k) o[k] = apply_sign(o[k], 4 * lane + k);
     }
-    uint2 o;
-    o.x = (uint32_t)TQ::from_f32(v[0]) | ((uint32_t)TQ::from_f32(v[1]) << 16);
-    o.y = (uint32_t)TQ::from_f32(v[2]) | ((uint32_t)TQ::from_f32(v[3]) << 16);
-    *reinterpret_cast<uint2*>(P.out + (size_t)row * kHeadDim + 4 * lane) = o;
+    uint2 ob;
+    ob.x = (uint32_t)TQ::from_f32(o[0]) | ((uint32_t)TQ::from_f32(o[1]) << 16);
+    ob.y = (uint32_t)TQ::from_f32(o[2]) | ((uint32_t)TQ::from_f32(o[3]) << 16);
+    *reinterpret_cast<uint2*>(P.out + (size_t)row * kHeadDim + 4 * lane) = ob;
 }
 
 // ---- host side ---------------------------------------------------------------------------------
 constexpr int kMaxChunksCap = 256;
-constexpr int kMinUnitsPerChunk = 8;   // 256 tokens
-constexpr int kTargetWorkgroupsPerHead = 512;
+constexpr int kMinUnitsPerChunk = 16;  // 512 tokens: two units per wave
+constexpr int kTargetWorkgroupsPerHead = 128;
 
 static size_t partial_bytes(long long rows, int max_chunks) {
     return (size_t)rows * (size_t)max_chunks * (kHeadDim + 2) * sizeof(float) + (size_t)rows * sizeof(int);
@@ -745,23 +971,22 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     }
     const dim3 grid((unsigned)grid_x, (unsigned)(layout->local_kv_heads * P.q_subgroups),
                     (unsigned)batch->total_tokens);
-    const int lds = kLutBytes + kWaves * kStageTq4;
     hipStream_t stream = (hipStream_t)ex->stream;
     int rc;
     if (nt == 1) {
-        rc = ensure_dynamic_lds(paged_attn_tq4_kernel<TQ, 1>, lds);
+        rc = ensure_dynamic_lds(paged_attn_tq4_kernel<TQ, 1>, smem_bytes_for(1));
         if (rc) return rc;
-        hipLaunchKernelGGL((paged_attn_tq4_kernel<TQ, 1>), grid, dim3(256), lds, stream, P);
+        hipLaunchKernelGGL((paged_attn_tq4_kernel<TQ, 1>), grid, dim3(waves_for(1) * 64), smem_bytes_for(1), stream, P);
     } else {
-        rc = ensure_dynamic_lds(paged_attn_tq4_kernel<TQ, 2>, lds);
+        rc = ensure_dynamic_lds(paged_attn_tq4_kernel<TQ, 2>, smem_bytes_for(2));
         if (rc) return rc;
-        hipLaunchKernelGGL((paged_attn_tq4_kernel<TQ, 2>), grid, dim3(256), lds, stream, P);
+        hipLaunchKernelGGL((paged_attn_tq4_kernel<TQ, 2>), grid, dim3(waves_for(2) * 64), smem_bytes_for(2), stream, P);
     }
     rc = (int)hipGetLastError();
     if (rc) return rc;
     if (P.max_chunks > 1) {
-        hipLaunchKernelGGL((split_merge_kernel<TQ>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream,
-                           P, 1);
+        hipLaunchKernelGGL((split_merge_kernel<TQ>), dim3((unsigned)rows), dim3(1024), 0, stream, P,
+                           kLutInvGain, 1);
         rc = (int)hipGetLastError();
     }
     return rc;
@@ -781,7 +1006,6 @@ static bool tq4_geometry_ok(const warp34_kv_layer_layout* l, const void* q) {
            (l->v_page_stride_bytes & 15u) == 0 && (l->v_head_stride_bytes & 15u) == 0 &&
            (((uintptr_t)q) & 7u) == 0;
 }
-static_assert(kLutBytes + kWaves * kStageTq4 >= 2 * 2 * 16 * 258 * 4, "merge buffer must fit the LDS block");
 
 static int common_checks(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
                          const warp34_attention_batch* batch, const void* q, void* out, int num_q_heads) {
@@ -849,8 +1073,7 @@ extern "C" int warp34_paged_attention_f16_force_kernel_for_test(
 extern "C" size_t warp34_paged_attention_scratch_bytes(int total_tokens, int num_q_heads, int max_seq_len) {
     (void)max_seq_len;
     if (total_tokens <= 0 || num_q_heads <= 0) return 0;
-    int tiles = total_tokens;
-    int want = kTargetWorkgroupsPerHead / tiles;
+    int want = kTargetWorkgroupsPerHead / total_tokens;
     if (want > kMaxChunksCap) want = kMaxChunksCap;
     if (want < 2) want = 2;
     return partial_bytes((long long)total_tokens * num_q_heads, want);
