@@ -58,7 +58,7 @@ constexpr int kLutBytes = 256 * 256;  // 256 entries x 64 lane replicas x 4 B
 constexpr int kRunBytes = 16 * kTq4RowBytes;  // 16 rows = 2112 B = 132 16-byte pieces
 constexpr int kStageTq4 = 4 * kRunBytes;      // K rows 0-31 then V rows 0-31: 8448 B
 __host__ __device__ constexpr int merge_floats_for(int nt) {
-    return waves_for(nt) * (nt * 16 * 258 + 8) + (waves_for(nt) + 1) * nt * 16 * 2;
+    return waves_for(nt) * (nt * 16 * 260) + (waves_for(nt) + 1) * nt * 16 * 2;
 }
 __host__ __device__ constexpr int smem_bytes_for(int nt) {
     const int loop_bytes = kLutBytes + waves_for(nt) * kStageTq4;
@@ -129,6 +129,41 @@ __device__ __forceinline__ ChunkGeom chunk_geom(int u_lo, int u_hi, int max_chun
     return g;
 }
 
+// value of lane (lane ^ H) for every lane of a wave, built from DPP / lane-swap VALU ops
+// (no LDS round trip): quad permutes for 1 and 2, row shifts for 4, a row rotate for 8 and
+// the gfx950 row / half swaps for 16 and 32.
+template <int H>
+__device__ __forceinline__ float lane_xor(float x, int lane) {
+    const int xi = __float_as_int(x);
+    if constexpr (H == 1) {
+        return __int_as_float(__builtin_amdgcn_mov_dpp(xi, 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
+    } else if constexpr (H == 2) {
+        return __int_as_float(__builtin_amdgcn_mov_dpp(xi, 0x4E, 0xF, 0xF, true));  // quad_perm [2,3,0,1]
+    } else if constexpr (H == 4) {
+        // banks 0,2 (lanes 0-3, 8-11 of a row) take lane+4, banks 1,3 take lane-4
+        int r = __builtin_amdgcn_update_dpp(0, xi, 0x104, 0xF, 0x5, false);  // row_shl:4
+        r = __builtin_amdgcn_update_dpp(r, xi, 0x114, 0xF, 0xA, false);      // row_shr:4
+        return __int_as_float(r);
+    } else if constexpr (H == 8) {
+        return __int_as_float(__builtin_amdgcn_mov_dpp(xi, 0x128, 0xF, 0xF, true));  // row_ror:8
+    } else if constexpr (H == 16) {
+        const auto r = __builtin_amdgcn_permlane16_swap((uint32_t)xi, (uint32_t)xi, false, false);
+        return __uint_as_float((lane & 16) ? r[0] : r[1]);
+    } else {
+        const auto r = __builtin_amdgcn_permlane32_swap((uint32_t)xi, (uint32_t)xi, false, false);
+        return __uint_as_float((lane & 32) ? r[0] : r[1]);
+    }
+}
+
+template <int H>
+__device__ __forceinline__ void wht_stage(float (&v)[4], int lane) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float o = lane_xor<H>(v[k], lane);
+        v[k] = (lane & H) ? (o - v[k]) : (v[k] + o);
+    }
+}
+
 // 256-point WHT over one wave: element e = 4*lane + k, scaled by 1/16.
 __device__ __forceinline__ void wht256_wave(float (&v)[4], int lane) {
     {
@@ -138,16 +173,26 @@ __device__ __forceinline__ void wht256_wave(float (&v)[4], int lane) {
         v[2] = a0 - a2;
         v[3] = a1 - a3;
     }
-#pragma unroll
-    for (int h = 1; h < 64; h <<= 1) {
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const float o = __shfl_xor(v[k], h, 64);
-            v[k] = (lane & h) ? (o - v[k]) : (v[k] + o);
-        }
-    }
+    wht_stage<1>(v, lane);
+    wht_stage<2>(v, lane);
+    wht_stage<4>(v, lane);
+    wht_stage<8>(v, lane);
+    wht_stage<16>(v, lane);
+    wht_stage<32>(v, lane);
 #pragma unroll
     for (int k = 0; k < 4; ++k) v[k] *= 0.0625f;
+}
+
+// centroid k as an immediate select chain (no constant-memory load on the critical path)
+__device__ __forceinline__ float centroid_imm(int k) {
+    const float m = (k & 4) ? ((k & 2) ? ((k & 1) ? 1.694104124e-1f : 1.285881878e-1f)
+                                       : ((k & 1) ? 1.006979993e-1f : 7.824930800e-2f))
+                            : ((k & 2) ? ((k & 1) ? 5.873210384e-2f : 4.094919437e-2f)
+                                       : ((k & 1) ? 2.420087619e-2f : 8.008373692e-3f));
+    return m;  // magnitude of centroid 8 + k; centroid[7 - k] = -m
+}
+__device__ __forceinline__ float centroid_of_code(int code) {
+    return (code & 8) ? centroid_imm(code & 7) : -centroid_imm(7 - (code & 7));
 }
 
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
@@ -247,30 +292,72 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
             q_raw[c] = *reinterpret_cast<const uint2*>(qrow + 4 * lane);
         }
     }
+    // Request lookup in one memory round trip: lane l examines request base+l (the first
+    // matching request wins, as in the linear scan of op_kv_cache.cu:385-398) and carries that
+    // request's lengths, which are then broadcast with readlane.  Every token of the tile
+    // belongs to this request, so its key ranges follow from two scalars (op_kv_cache.cu:406-424).
+    bool req_hit = false;
+    int req = -1, rq_start = 0, rq_end = 0, seq_after = 0, ctx_before = 0;
+    for (int base = 0; base < B.num_reqs && !req_hit; base += 64) {
+        const int r = base + lane;
+        const bool inb = r < B.num_reqs;
+        const int lo = inb ? B.query_start_loc[r] : 0x7fffffff;
+        const int hi = inb ? B.query_start_loc[r + 1] : -0x7fffffff;
+        const int sa = inb ? B.seq_lens_after[r] : 0;
+        const int cb = (inb && B.context_lens_before != nullptr) ? B.context_lens_before[r] : 0;
+        const int rm = (inb && B.valid_req_mask != nullptr) ? (int)B.valid_req_mask[r] : 1;
+        const unsigned long long hits = __ballot(inb && tok0 >= lo && tok0 < hi);
+        if (hits != 0ull) {
+            const int src = __builtin_ctzll(hits);
+            req = base + src;
+            rq_start = __builtin_amdgcn_readlane(lo, src);
+            rq_end = __builtin_amdgcn_readlane(hi, src);
+            seq_after = __builtin_amdgcn_readlane(sa, src);
+            ctx_before = B.context_lens_before != nullptr ? __builtin_amdgcn_readlane(cb, src)
+                                                          : seq_after - (rq_end - rq_start);
+            req_hit = __builtin_amdgcn_readlane(rm, src) != 0;
+            if (!req_hit) break;  // masked request
+        }
+    }
+    // per-token validity of this lane's columns (independent of the request lookup)
+    bool tok_ok[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int tok = tok0 + (nt * 16 + n) / P.q_group;
+        tok_ok[nt] = tok < B.total_tokens &&
+                     (B.valid_token_mask == nullptr || B.valid_token_mask[min(tok, B.total_tokens - 1)] != 0);
+    }
     {
         // entry e = (gain*centroid[e & 15], gain*centroid[e >> 4]) as packed fp16, 64 copies
         constexpr int kThreadsPerEntry = kWaves * 64 / 256;      // 2 or 1
         constexpr int kBytesPerThread = 256 / kThreadsPerEntry;  // 128 or 256
         const int e = tid / kThreadsPerEntry;
-        const uint32_t v = pack_h2(kLutGain * kCentroids[e & 15], kLutGain * kCentroids[e >> 4]);
+        const uint32_t v = pack_h2(kLutGain * centroid_of_code(e & 15), kLutGain * centroid_of_code(e >> 4));
         u4 vv = {v, v, v, v};
         u4* dst = reinterpret_cast<u4*>(smem + e * 256 + (tid % kThreadsPerEntry) * kBytesPerThread);
 #pragma unroll
         for (int k = 0; k < kBytesPerThread / 16; ++k) dst[k] = vv;
     }
 
-    int rq_start = 0, rq_end = 0;
-    const int req = find_request(B, tok0, rq_start, rq_end);
-    if (req < 0) return;
-    if (B.valid_req_mask != nullptr && B.valid_req_mask[req] == 0) return;
+    // Rotate the query rows now (dead columns are zeroed when they are stored below): the
+    // request lookup and the first KV loads are then not held up behind this wave's VALU work.
+    float q_rot[kColsPerWave][4];
+#pragma unroll
+    for (int c = 0; c < kColsPerWave; ++c) {
+        q_rot[c][0] = TQ::to_f32((uint16_t)(q_raw[c].x & 0xFFFFu));
+        q_rot[c][1] = TQ::to_f32((uint16_t)(q_raw[c].x >> 16));
+        q_rot[c][2] = TQ::to_f32((uint16_t)(q_raw[c].y & 0xFFFFu));
+        q_rot[c][3] = TQ::to_f32((uint16_t)(q_raw[c].y >> 16));
+#pragma unroll
+        for (int k = 0; k < 4; ++k) q_rot[c][k] = apply_sign(q_rot[c][k], 4 * lane + k);
+        wht256_wave(q_rot[c], lane);
+    }
+
+    W34_TP(47);
+    if (!req_hit) return;  // no owning request (or masked request): outputs untouched
     if (((tok0 - rq_start) % P.tok_tile) != 0) return;  // not a tile leader
     int tile_tokens = rq_end - tok0;
     if (tile_tokens > P.tok_tile) tile_tokens = P.tok_tile;
-    // every token of the tile belongs to request `req`: its ranges follow from two scalars
-    // (op_kv_cache.cu:406-424)
-    const int seq_after = B.seq_lens_after[req];
-    const int ctx_before =
-        B.context_lens_before != nullptr ? B.context_lens_before[req] : seq_after - (rq_end - rq_start);
 
     // per-lane column info (one column per N tile)
     int col_lo[NT], col_hi[NT];
@@ -283,8 +370,7 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
         const int col = nt * 16 + n;
         const int t = col / P.q_group;
         const int tok = tok0 + t;
-        bool ok = t < tile_tokens;
-        if (ok && B.valid_token_mask != nullptr) ok = B.valid_token_mask[tok] != 0;
+        const bool ok = t < tile_tokens && tok_ok[nt];
         const int q_off = tok - rq_start;
         int mx = (B.mask_mode == WARP34_ATTN_MASK_NONCAUSAL_WINDOW) ? seq_after - 1 : ctx_before + q_off;
         if (mx >= seq_after) mx = seq_after - 1;
@@ -330,7 +416,6 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
     W34_TP(1);
 
     // ---- staging machinery ----------------------------------------------------------------------
-    const int32_t* req_blocks = B.block_tables + (size_t)req * B.max_blocks_per_req;
     const uint8_t* k_base = reinterpret_cast<const uint8_t*>((uintptr_t)L.k_base) +
                             (size_t)kv_head * L.k_head_stride_bytes;
     const uint8_t* v_base = reinterpret_cast<const uint8_t*>((uintptr_t)L.v_base) +
@@ -341,44 +426,50 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
     // K rows 16-31, V rows 0-15, V rows 16-31.  Pieces 0-127 of every run are two full-wave
     // loads from a wave-uniform base; the four tails (pieces 128-131) share one load.
     // The physical page ids of a unit are fetched (scalar loads) one iteration before its data.
+    // The physical page ids come from ONE vector load per 64 block-table slots: lane l holds
+    // the id of slot slot_base + l, a unit picks its two ids with readlane.  No scalar memory
+    // loads remain in the loop (they share the LDS wait counter and would serialise it).
     u4 pf[9];
-#pragma unroll
-    for (int i = 0; i < 9; ++i) pf[i] = u4{0u, 0u, 0u, 0u};
-    auto lookup_pages = [&](int unit, int32_t (&pg)[2], int (&in_page)[2]) {
+    const int32_t* req_blocks = B.block_tables + (size_t)req * B.max_blocks_per_req;
+    int slot_base = (cu_first * kUnit) / L.block_size;
+    int page_vec;
+    auto load_page_vec = [&]() {
+        const int slot = slot_base + lane;
+        page_vec = slot < B.max_blocks_per_req ? req_blocks[slot] : -1;
+    };
+    // Runs that do not overlap the visible key range, or whose block-table entry is missing,
+    // are read from page 0 of the slab instead: every row they deliver is masked, and any
+    // TQ4 bytes dequantise to finite values.  Keeping the loads unconditional lets the
+    // compiler count them statically (s_waitcnt vmcnt(N) instead of vmcnt(0)).
+    auto issue_loads = [&](int unit) {
+        const uint8_t* run_ptr[4];
 #pragma unroll
         for (int gidx = 0; gidx < 2; ++gidx) {
             const int pos = unit * kUnit + 16 * gidx;
             const int page_slot = pos / L.block_size;
-            in_page[gidx] = pos - page_slot * L.block_size;
-            // a run is fetched only when it overlaps the visible key range and its block
-            // table entry exists; everything else keeps stale (finite-by-construction) bytes
-            const bool live = unit < cu_end && pos <= u_hi && pos + 15 >= u_lo && page_slot < B.max_blocks_per_req;
-            pg[gidx] = live ? req_blocks[page_slot] : -1;
-        }
-    };
-    auto issue_loads = [&](const int32_t (&pg)[2], const int (&in_page)[2]) {
-        const uint8_t* run_ptr[4];
-#pragma unroll
-        for (int gidx = 0; gidx < 2; ++gidx) {
-            const bool live = pg[gidx] >= 0;
-            run_ptr[gidx] = live ? k_base + (size_t)pg[gidx] * L.k_page_stride_bytes +
-                                       (size_t)in_page[gidx] * L.k_token_stride_bytes
-                                 : nullptr;
-            run_ptr[2 + gidx] = live ? v_base + (size_t)pg[gidx] * L.v_page_stride_bytes +
-                                           (size_t)in_page[gidx] * L.v_token_stride_bytes
-                                     : nullptr;
+            const int in_page = pos - page_slot * L.block_size;
+            int rel = page_slot - slot_base;
+            if (rel >= 64) {  // wave-uniform, at most once per 64 slots
+                slot_base = page_slot;
+                load_page_vec();
+                rel = 0;
+            }
+            const int32_t pg = __builtin_amdgcn_readlane(page_vec, rel);
+            const bool live = pos <= u_hi && pos + 15 >= u_lo && pg >= 0;
+            const size_t koff = live ? (size_t)pg * L.k_page_stride_bytes + (size_t)in_page * L.k_token_stride_bytes : 0;
+            const size_t voff = live ? (size_t)pg * L.v_page_stride_bytes + (size_t)in_page * L.v_token_stride_bytes : 0;
+            run_ptr[gidx] = k_base + koff;
+            run_ptr[2 + gidx] = v_base + voff;
         }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            if (run_ptr[r] != nullptr) {  // wave-uniform
-                pf[2 * r] = *(global_cu4*)(run_ptr[r] + 16 * lane);
-                pf[2 * r + 1] = *(global_cu4*)(run_ptr[r] + 1024 + 16 * lane);
-            }
+            pf[2 * r] = *(global_cu4*)(run_ptr[r] + 16 * lane);
+            pf[2 * r + 1] = *(global_cu4*)(run_ptr[r] + 1024 + 16 * lane);
         }
         {
             const int r = lane >> 2;
             const uint8_t* base = r == 0 ? run_ptr[0] : r == 1 ? run_ptr[1] : r == 2 ? run_ptr[2] : run_ptr[3];
-            if (lane < 16 && base != nullptr) pf[8] = *(global_cu4*)(base + 2048 + 16 * (lane & 3));
+            pf[8] = *(global_cu4*)(base + 2048 + 16 * (lane & 3));
         }
     };
     auto commit_loads = [&]() {
@@ -390,76 +481,34 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
         if (lane < 16) *reinterpret_cast<u4*>(stage + (lane >> 2) * kRunBytes + 2048 + 16 * (lane & 3)) = pf[8];
     };
 
-    // first unit's data goes in flight before the prologue work, the second unit's page ids too
+    // first unit's data goes in flight before the rest of the prologue
     int unit = cu_first + wave;
-    int32_t pg_next[2];
-    int inpage_next[2];
-    {
-        int32_t pg0[2];
-        int inpage0[2];
-        lookup_pages(unit, pg0, inpage0);
-        lookup_pages(unit + kWaves, pg_next, inpage_next);
-        issue_loads(pg0, inpage0);
-    }
+    load_page_vec();
+    W34_TP(41);
+    issue_loads(unit);  // harmless for a wave without work: dead runs read page 0
+    W34_TP(42);
 
-    // ---- prologue: rotated queries -------------------------------------------------------------
-    // The rotated fp16 queries are staged in the (still unused) staging area as [16*NT][264]
-    // halves.  All the constant factors of the scores (softmax scale, log2 e, 1 / table gain)
-    // go into Q'.
+    // ---- prologue: rotated fp16 queries to LDS ---------------------------------------------------
+    // Staged in the (still unused) staging area as [16*NT][264] halves.  All the constant
+    // factors of the scores (softmax scale, log2 e, 1 / table gain) go into Q'.
     constexpr int kQStride = 264;
     _Float16* qlds = reinterpret_cast<_Float16*>(stage_all);
     const float q_scale = B.sm_scale * kLog2e * kLutInvGain;
-    {
-        float v[kColsPerWave][4];
-        bool okc[kColsPerWave];
 #pragma unroll
-        for (int c = 0; c < kColsPerWave; ++c) {
-            const int col = wave + c * kWaves;
-            okc[c] = col < 16 * NT && ((ok_mask[(col >> 4) & (NT - 1)] >> (col & 15)) & 1u);
-            v[c][0] = TQ::to_f32((uint16_t)(q_raw[c].x & 0xFFFFu));
-            v[c][1] = TQ::to_f32((uint16_t)(q_raw[c].x >> 16));
-            v[c][2] = TQ::to_f32((uint16_t)(q_raw[c].y & 0xFFFFu));
-            v[c][3] = TQ::to_f32((uint16_t)(q_raw[c].y >> 16));
-#pragma unroll
-            for (int k = 0; k < 4; ++k) v[c][k] = okc[c] ? apply_sign(v[c][k], 4 * lane + k) : 0.f;
-        }
-        bool any_col = false;
-#pragma unroll
-        for (int c = 0; c < kColsPerWave; ++c) any_col |= okc[c];
-        if (any_col) {  // wave-uniform; the columns of a wave are transformed together
-#pragma unroll
-            for (int c = 0; c < kColsPerWave; ++c) {
-                const float a0 = v[c][0] + v[c][1], a1 = v[c][0] - v[c][1];
-                const float a2 = v[c][2] + v[c][3], a3 = v[c][2] - v[c][3];
-                v[c][0] = a0 + a2;
-                v[c][1] = a1 + a3;
-                v[c][2] = a0 - a2;
-                v[c][3] = a1 - a3;
-            }
-#pragma unroll
-            for (int h = 1; h < 64; h <<= 1) {
-#pragma unroll
-                for (int c = 0; c < kColsPerWave; ++c) {
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        const float o = __shfl_xor(v[c][k], h, 64);
-                        v[c][k] = (lane & h) ? (o - v[c][k]) : (v[c][k] + o);
-                    }
-                }
-            }
-        }
-#pragma unroll
-        for (int c = 0; c < kColsPerWave; ++c) {
-            const int col = wave + c * kWaves;
-            if (col < 16 * NT) {
-                uint2 packed;
-                packed.x = pack_h2(v[c][0] * (0.0625f * q_scale), v[c][1] * (0.0625f * q_scale));
-                packed.y = pack_h2(v[c][2] * (0.0625f * q_scale), v[c][3] * (0.0625f * q_scale));
-                *reinterpret_cast<uint2*>(qlds + col * kQStride + 4 * lane) = packed;
-            }
+    for (int c = 0; c < kColsPerWave; ++c) {
+        const int col = wave + c * kWaves;
+        if (col < 16 * NT) {
+            const bool okc = (ok_mask[(col >> 4) & (NT - 1)] >> (col & 15)) & 1u;
+            const float sc_q = okc ? q_scale : 0.f;
+            uint2 packed;
+            packed.x = pack_h2(q_rot[c][0] * sc_q, q_rot[c][1] * sc_q);
+            packed.y = pack_h2(q_rot[c][2] * sc_q, q_rot[c][3] * sc_q);
+            *reinterpret_cast<uint2*>(qlds + col * kQStride + 4 * lane) = packed;
         }
     }
+    W34_TP(44);
     __syncthreads();
+    W34_TP(45);
 
     // B operands of the QK MFMAs: 9 per N tile (5 for the first half-row, 4 for the second)
     h8 bq[NT][9];
@@ -480,6 +529,7 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
             bq[nt][mf] = x;
         }
     }
+    W34_TP(46);
     __syncthreads();  // qlds is dead, the staging area may be overwritten; the table is complete
     W34_TP(2);
 
@@ -695,10 +745,15 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
 #ifdef W34_TRACE
         if (trace_it < 8) W34_TP(4 + 4 * trace_it);
 #endif
-        // next unit's data (page ids were fetched one iteration ago), next-next unit's page ids
-        issue_loads(pg_next, inpage_next);
-        lookup_pages(unit + 2 * kWaves, pg_next, inpage_next);
+        if (unit + kWaves < cu_end) issue_loads(unit + kWaves);
         const int t0 = unit * kUnit;
+        // The two waves that share a SIMD take turns at the higher issue priority, unit by
+        // unit; with equal priorities the older wave always wins and finishes ~25 % earlier.
+        if ((((unit - cu_first) / kWaves) ^ (wave >> 2)) & 1) {
+            __builtin_amdgcn_s_setprio(1);
+        } else {
+            __builtin_amdgcn_s_setprio(0);
+        }
         process_unit(t0, !(t0 >= i_lo && t0 + kUnit - 1 <= i_hi));
 #ifdef W34_TRACE
         if (trace_it < 8) W34_TP(4 + 4 * trace_it + 3);
@@ -706,6 +761,7 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
 #endif
     }
     W34_TP(36);
+    __builtin_amdgcn_s_setprio(0);
 
     // ---- combine the per-lane partial sums of l over the four k-block lanes of a column ------
 #pragma unroll
@@ -714,16 +770,17 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
     // ---- merge the waves' states through LDS ---------------------------------------------------
     // Every wave publishes (m, l), rescales its O by 2^(m - m_tot) and stores it in its own
     // region; then the waves split the columns and add the regions up in wave order.
-    // Region layout: element e of column c at dword c*258 + (e ^ ((e >> 5) & 1)): the lanes of a
-    // half-wave store (16 columns x 2 row groups that are 32 elements apart) hit 32 distinct
-    // banks.
-    __syncthreads();  // every wave is done with the table and with its staging area
-    constexpr int kColStride = 258;
-    constexpr int kRegion = NT * 16 * kColStride + 8;
+    // Region layout: column stride 260 dwords; inside a column the four values a lane holds for
+    // one MFMA result (rows 4b..4b+3 of (h, j)) are contiguous at ((h*8 + j)*4 + b)*4, so a
+    // lane stores them with one 128-bit write, and the 8 lanes of a write pass (8 columns)
+    // start 4 banks apart.
+    constexpr int kColStride = 260;
+    constexpr int kRegion = NT * 16 * kColStride;
     float* xbuf = reinterpret_cast<float*>(smem);
-    float* mlbuf = xbuf + kWaves * kRegion;  // [kWaves][NT*16][2]
+    float* mlbuf = xbuf + kWaves * kRegion;  // [kWaves][NT*16][2], behind the table + staging areas
     static_assert(kWaves * kRegion + (kWaves + 1) * NT * 16 * 2 == merge_floats_for(NT), "merge layout");
     static_assert(smem_bytes_for(NT) >= merge_floats_for(NT) * 4, "merge buffer must fit");
+    static_assert(kWaves * kRegion * 4 >= kLutBytes + kWaves * kStageTq4, "(m, l) table must not alias live LDS");
     if (b == 0) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
@@ -731,7 +788,9 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
             mlbuf[(wave * NT * 16 + nt * 16 + n) * 2 + 1] = l_run[nt];
         }
     }
-    __syncthreads();
+    W34_TP(49);
+    __syncthreads();  // every wave is done with the table and with its staging area
+    W34_TP(50);
     float m_tot[NT], l_tot[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
@@ -747,15 +806,13 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
         l_tot[nt] = lt;
         const float wgt = __builtin_amdgcn_exp2f(m_run[nt] - mt);
         float* c = xbuf + wave * kRegion + (nt * 16 + n) * kColStride;
+        if (col_ok[nt]) {  // dead columns are never read back
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
+            for (int h = 0; h < 2; ++h)
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int e = tq4_pv_elem(h, j, 4 * b + i);
-                    c[e ^ ((e >> 5) & 1)] = o_acc[nt][h][j][i] * wgt;
-                }
+                for (int j = 0; j < 8; ++j)
+                    *reinterpret_cast<f4*>(c + ((h * 8 + j) * 4 + b) * 4) = o_acc[nt][h][j] * wgt;
+        }
     }
     // (m_tot, l_tot) of every column for the epilogue, read back by column below
     float* mltot = mlbuf + kWaves * NT * 16 * 2;
@@ -766,10 +823,27 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
             mltot[(nt * 16 + n) * 2 + 1] = l_tot[nt];
         }
     }
+    W34_TP(51);
     __syncthreads();
     W34_TP(37);
 
     // ---- epilogue: per column, add the regions, then store the partial or finish the row -------
+    int merge_slot[4];  // region slot of element 4*lane + k (inverse of tq4_pv_elem)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int e = 4 * lane + k;
+        int h, j, r;
+        if (e >= 128) {
+            h = 1; r = (e - 128) >> 3; j = e & 7;
+        } else if (e < 4) {
+            h = 0; r = 0; j = e;
+        } else if (e >= 124) {
+            h = 0; r = 0; j = e - 120;
+        } else {
+            h = 0; r = (e + 4) >> 3; j = (e + 4) & 7;
+        }
+        merge_slot[k] = ((h * 8 + j) * 4 + (r >> 2)) * 4 + (r & 3);
+    }
     for (int col = wave; col < 16 * NT; col += kWaves) {
         const int t = col / P.q_group;
         const int a = col - t * P.q_group;
@@ -778,10 +852,10 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
         float v[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) {
-            const float* c = xbuf + w * kRegion + col * kColStride + 4 * lane;
-            const int f = (lane >> 3) & 1;
+            // element e = 4*lane + k is value (h, j, row r) with e = tq4_pv_elem(h, j, r)
+            const float* c = xbuf + w * kRegion + col * kColStride;
 #pragma unroll
-            for (int k = 0; k < 4; ++k) v[k] += c[k ^ f];
+            for (int k = 0; k < 4; ++k) v[k] += c[merge_slot[k]];
         }
         const float m_col = mltot[col * 2 + 0];
         const float l_col = mltot[col * 2 + 1];
