@@ -94,8 +94,7 @@ struct AttnParams {
     const uint16_t* q;
     uint16_t* out;
     float* part_acc;  // [rows][max_chunks][256] or null
-    float* part_ml;   // [rows][max_chunks][2]
-    int* part_cnt;    // [rows]
+    float* part_ml;   // [rows][max_chunks][4]: m, l, chunk count, unused
     int num_q_heads;
     int gqa;          // q heads per kv head
     int q_group;      // q heads of one kv head handled by one workgroup (<= 16)
@@ -864,9 +863,10 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
             float* dst = P.part_acc + (row * P.max_chunks + chunk) * kHeadDim;
             *reinterpret_cast<f4*>(dst + 4 * lane) = f4{v[0], v[1], v[2], v[3]};
             if (lane == 0) {
-                P.part_ml[(row * P.max_chunks + chunk) * 2 + 0] = m_col;
-                P.part_ml[(row * P.max_chunks + chunk) * 2 + 1] = l_col;
-                if (chunk == 0) P.part_cnt[row] = g.n_chunks;
+                // (m, l, number of chunks of this row, -): one record per chunk, every record
+                // carries the count so the merge needs no dependent load
+                *reinterpret_cast<f4*>(P.part_ml + (row * P.max_chunks + chunk) * 4) =
+                    f4{m_col, l_col, (float)g.n_chunks, 0.f};
             }
         } else {
             const float inv = l_col > 0.f ? kLutInvGain / l_col : 0.f;
@@ -894,44 +894,82 @@ extern "C" int warp34_debug_read_trace(unsigned long long* dst) {
 // w_s = 2^(m_s - m_tot), out = sum acc_s w_s / sum l_s w_s, then one inverse rotation.
 // One workgroup of 1024 threads per (token, q head) row: 16 groups of 64 threads stride the
 // chunks, each thread owns 4 of the 256 columns; the groups are summed through LDS.
+// Everything the row needs (validity, chunk records, accumulators) is requested in ONE memory
+// round trip: records and accumulators of all max_chunks slots are loaded speculatively and
+// the slots beyond the row's chunk count are discarded with selects.
 constexpr int kMergeGroups = 16;
+constexpr int kMergeMaxPerGroup = 16;  // max_chunks <= 256
 template <typename TQ>
 __global__ __launch_bounds__(1024) void split_merge_kernel(const AttnParams P, float out_scale, int rotate) {
     __shared__ f4 s_acc[kMergeGroups][64];
+    __shared__ f4 s_rec[256];
     __shared__ float s_red[kMergeGroups];
-    const int lane = (int)(threadIdx.x & 63);
-    const int grp = (int)(threadIdx.x >> 6);
+    __shared__ int s_valid;
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int grp = tid >> 6;
     const long long row = (long long)blockIdx.x;
     const int tok = (int)(row / P.num_q_heads);
-    const RowRange rr = row_range(P.B, tok);
-    if (rr.req < 0) return;  // masked row: output untouched (uniform for the block)
-    const int n_chunks = P.part_cnt[row];
-    const float* ml = P.part_ml + (size_t)row * P.max_chunks * 2;
+    const warp34_attention_batch& B = P.B;
+    const float* ml = P.part_ml + (size_t)row * P.max_chunks * 4;
     const float* acc = P.part_acc + (size_t)row * P.max_chunks * kHeadDim;
 
-    // pass 1: global maximum of m over chunks with l > 0
-    float m_loc = kNegBig;
-    for (int s = (int)threadIdx.x; s < n_chunks; s += 1024)
-        if (ml[2 * s + 1] > 0.f) m_loc = fmaxf(m_loc, ml[2 * s]);
+    // speculative loads: chunk records (one per thread) and this thread's accumulator slices
+    f4 rec = {kNegBig, 0.f, 0.f, 0.f};
+    if (tid < P.max_chunks) rec = *reinterpret_cast<const f4*>(ml + 4 * tid);
+    f4 a[kMergeMaxPerGroup];
 #pragma unroll
-    for (int off = 1; off < 64; off <<= 1) m_loc = fmaxf(m_loc, __shfl_xor(m_loc, off, 64));
-    if (lane == 0) s_red[grp] = m_loc;
+    for (int k = 0; k < kMergeMaxPerGroup; ++k) {
+        const int s = grp + k * kMergeGroups;
+        a[k] = f4{0.f, 0.f, 0.f, 0.f};
+        if (s < P.max_chunks) a[k] = *reinterpret_cast<const f4*>(acc + (size_t)s * kHeadDim + 4 * lane);
+    }
+    // row validity (wave 0): token mask and owning request, first match wins
+    if (grp == 0) {
+        bool ok = B.valid_token_mask == nullptr || B.valid_token_mask[tok] != 0;
+        bool found = false;
+        for (int base = 0; base < B.num_reqs && !found; base += 64) {
+            const int r = base + lane;
+            const bool inb = r < B.num_reqs;
+            const int lo = inb ? B.query_start_loc[r] : 0x7fffffff;
+            const int hi = inb ? B.query_start_loc[r + 1] : -0x7fffffff;
+            const int rm = (inb && B.valid_req_mask != nullptr) ? (int)B.valid_req_mask[r] : 1;
+            const unsigned long long hits = __ballot(inb && tok >= lo && tok < hi);
+            if (hits != 0ull) {
+                found = true;
+                ok = ok && __builtin_amdgcn_readlane(rm, __builtin_ctzll(hits)) != 0;
+            }
+        }
+        if (lane == 0) s_valid = (ok && found) ? 1 : 0;
+    }
+    if (tid < 256) s_rec[tid] = rec;
     __syncthreads();
-    float m_tot = kNegBig;
-#pragma unroll
-    for (int k = 0; k < kMergeGroups; ++k) m_tot = fmaxf(m_tot, s_red[k]);
-    __syncthreads();
+    if (!s_valid) return;  // masked row: output untouched (uniform for the block)
+    int n_chunks = (int)s_rec[0][2];
+    if (n_chunks > P.max_chunks) n_chunks = P.max_chunks;
 
-    // pass 2: weighted sums
+    // global maximum of m over chunks with l > 0 (every thread scans the LDS copy)
+    float m_tot = kNegBig;
+    for (int s = lane; s < n_chunks; s += 64) {
+        const f4 r = s_rec[s];
+        if (r[1] > 0.f) m_tot = fmaxf(m_tot, r[0]);
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) m_tot = fmaxf(m_tot, __shfl_xor(m_tot, off, 64));
+
     f4 v = {0.f, 0.f, 0.f, 0.f};
     float l_part = 0.f;
-    for (int s = grp; s < n_chunks; s += kMergeGroups) {
-        const float ls = ml[2 * s + 1];
-        if (!(ls > 0.f)) continue;
-        const float w = __builtin_amdgcn_exp2f(ml[2 * s] - m_tot);
-        l_part += ls * w;
-        const f4 a = *reinterpret_cast<const f4*>(acc + (size_t)s * kHeadDim + 4 * lane);
-        v += a * w;
+#pragma unroll
+    for (int k = 0; k < kMergeMaxPerGroup; ++k) {
+        const int s = grp + k * kMergeGroups;
+        if (s < n_chunks) {
+            const f4 r = s_rec[s];
+            if (r[1] > 0.f) {
+                const float w = __builtin_amdgcn_exp2f(r[0] - m_tot);
+                l_part += r[1] * w;
+                v += a[k] * w;
+            }
+        }
     }
     s_acc[grp][lane] = v;
     if (lane == 0) s_red[grp] = l_part;
@@ -963,7 +1001,7 @@ constexpr int kMinUnitsPerChunk = 16;  // 512 tokens: two units per wave
 constexpr int kTargetWorkgroupsPerHead = 128;
 
 static size_t partial_bytes(long long rows, int max_chunks) {
-    return (size_t)rows * (size_t)max_chunks * (kHeadDim + 2) * sizeof(float) + (size_t)rows * sizeof(int);
+    return (size_t)rows * (size_t)max_chunks * (kHeadDim + 4) * sizeof(float);
 }
 
 // Cap on chunks per tile: a function of total_tokens (tiles) and the scratch size only.
@@ -1028,13 +1066,11 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     P.max_chunks = force_single ? 1 : choose_max_chunks(ex, batch->total_tokens, num_q_heads, P.tok_tile);
     P.part_acc = nullptr;
     P.part_ml = nullptr;
-    P.part_cnt = nullptr;
     const long long rows = (long long)batch->total_tokens * num_q_heads;
     if (P.max_chunks > 1) {
         uint8_t* ws = reinterpret_cast<uint8_t*>((uintptr_t)ex->scratch_ptr);
         P.part_acc = reinterpret_cast<float*>(ws);
         P.part_ml = P.part_acc + (size_t)rows * P.max_chunks * kHeadDim;
-        P.part_cnt = reinterpret_cast<int*>(P.part_ml + (size_t)rows * P.max_chunks * 2);
     }
     // grid.x: chunks that can exist given the host's upper bound on the sequence length
     int grid_x = P.max_chunks;
