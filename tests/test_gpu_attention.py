@@ -12,7 +12,7 @@ import pytest
 
 import oracle
 from cases import make_case
-from oracle import DT_BF16, DT_F16, FMT_TQ4
+from oracle import DT_BF16, DT_F16, FMT_BF16, FMT_FP16, FMT_TQ4
 
 pytestmark = pytest.mark.gpu
 
@@ -146,3 +146,69 @@ def test_force_kernel_selector_agrees():
         rc, got, _ = G.dev_attention(dpool, hb, q, DT_F16, 8, force_kernel=sel)
         assert rc == 0
         G.assert_close(got, DT_F16, want, what="selector %d" % sel)
+
+
+# ---- 16-bit pages (FP16 pages with the f16 entry point, BF16 pages with the bf16 one) ----
+
+KV16 = [(FMT_FP16, DT_F16), (FMT_BF16, DT_BF16)]
+
+
+@pytest.mark.parametrize("fmt,dtype", KV16)
+@pytest.mark.parametrize("block_size", [16, 64])
+def test_kv16_decode_small_batch(fmt, dtype, block_size):
+    _check(fmt, dtype, block_size, [70, 33, 129, 1, 32], [1, 1, 1, 1, 1], 111)
+
+
+@pytest.mark.parametrize("fmt,dtype", KV16)
+@pytest.mark.parametrize("scratch", [0, SCRATCH])
+def test_kv16_decode_gqa8_long(fmt, dtype, scratch):
+    _check(fmt, dtype, 64, [5000], [1], 121, scratch=scratch, q_heads=16)
+
+
+def test_kv16_bf16_decode_ctx32k():
+    """BASELINE bf16 decode shape: ctx 32768, 16 q / 2 kv heads, 64-token pages."""
+    _check(FMT_BF16, DT_BF16, 64, [32768], [1], 131, scratch=64 << 20, q_heads=16)
+
+
+@pytest.mark.parametrize("fmt,dtype", KV16)
+@pytest.mark.parametrize("q_lens", [[4, 4], [2, 3], [16]])
+def test_kv16_verify_multi_token_causal(fmt, dtype, q_lens):
+    seq = [300 + 7 * i for i in range(len(q_lens))]
+    _check(fmt, dtype, 64, seq, q_lens, 141, q_heads=16)
+    _check(fmt, dtype, 16, seq, q_lens, 142, q_heads=8, scratch=0)
+
+
+@pytest.mark.parametrize("mask_mode,window", [(0, 40), (1, 0), (1, 100), (0, 5)])
+def test_kv16_windows(mask_mode, window):
+    _check(FMT_BF16, DT_BF16, 16, [333, 90], [3, 2], 151, mask_mode=mask_mode, window=window, ctx_null=True)
+
+
+def test_kv16_unwritten_pool_bytes_do_not_leak():
+    """Rows beyond the sequence hold 0xFF bytes (NaN patterns): they must not reach the output."""
+    import gpu_harness as G
+
+    pool, bt, k, v, q, aq, ctx = make_case(FMT_FP16, 64, [37, 100], [1, 2], 161, DT_F16)
+    hb = oracle.HostBatch(aq, [37, 100], bt, context_lens_before=ctx)
+    want = oracle.paged_attention(pool, hb, q, DT_F16, 8)
+    # poison every row the oracle's write did not touch
+    kk = pool.k.reshape(-1, pool.kv_heads, pool.block_size, 512)
+    vv = pool.v.reshape(-1, pool.kv_heads, pool.block_size, 512)
+    for r, s in enumerate([37, 100]):
+        last = bt[r, (s - 1) // 64]
+        kk[last, :, s % 64:, :] = 0xFF
+        vv[last, :, s % 64:, :] = 0xFF
+    dpool = _dev_pool(pool)
+    for scratch in (0, SCRATCH):
+        rc, got, _ = G.dev_attention(dpool, hb, q, DT_F16, 8, scratch_bytes=scratch)
+        assert rc == 0
+        G.assert_close(got, DT_F16, want, what="poisoned tail", scale=G.channel_scale(v, DT_F16, hb, 8))
+
+
+def test_kv16_mismatched_query_type_is_refused():
+    import gpu_harness as G
+
+    pool, bt, k, v, q, aq, ctx = make_case(FMT_BF16, 16, [40], [1], 171, DT_BF16)
+    hb = oracle.HostBatch(aq, [40], bt, context_lens_before=ctx)
+    dpool = _dev_pool(pool)
+    rc, got, _ = G.dev_attention(dpool, hb, q, DT_F16, 8)
+    assert rc == 801 and (got == 0x5500).all()

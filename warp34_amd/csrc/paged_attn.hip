@@ -995,6 +995,12 @@ __global__ __launch_bounds__(1024) void split_merge_kernel(const AttnParams P, f
     *reinterpret_cast<uint2*>(P.out + (size_t)row * kHeadDim + 4 * lane) = ob;
 }
 
+}  // namespace w34
+
+#include "paged_attn_kv16.h"
+
+namespace w34 {
+
 // ---- host side ---------------------------------------------------------------------------------
 constexpr int kMaxChunksCap = 256;
 constexpr int kMinUnitsPerChunk = 16;  // 512 tokens: two units per wave
@@ -1102,6 +1108,73 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     return rc;
 }
 
+template <typename TQ>
+static int launch_kv16(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
+                       const warp34_attention_batch* batch, const void* q, void* out, int num_q_heads,
+                       int force_single) {
+    AttnParams P;
+    P.L = *layout;
+    P.B = *batch;
+    P.q = (const uint16_t*)q;
+    P.out = (uint16_t*)out;
+    P.num_q_heads = num_q_heads;
+    P.gqa = num_q_heads / layout->local_kv_heads;
+    int q_group = P.gqa;
+    if (q_group > 16) {
+        for (int d = 16; d >= 1; --d)
+            if (P.gqa % d == 0) {
+                q_group = d;
+                break;
+            }
+    }
+    P.q_group = q_group;
+    P.q_subgroups = P.gqa / q_group;
+    P.tok_tile = 16 / q_group;  // one N tile
+    if (P.tok_tile < 1) P.tok_tile = 1;
+    P.min_upc = kMinUnitsPerChunk;
+    P.max_chunks = force_single ? 1 : choose_max_chunks(ex, batch->total_tokens, num_q_heads, P.tok_tile);
+    P.part_acc = nullptr;
+    P.part_ml = nullptr;
+    const long long rows = (long long)batch->total_tokens * num_q_heads;
+    if (P.max_chunks > 1) {
+        uint8_t* ws = reinterpret_cast<uint8_t*>((uintptr_t)ex->scratch_ptr);
+        P.part_acc = reinterpret_cast<float*>(ws);
+        P.part_ml = P.part_acc + (size_t)rows * P.max_chunks * kHeadDim;
+    }
+    int grid_x = P.max_chunks;
+    if (batch->max_seq_len > 0) {
+        const int units = (batch->max_seq_len + kUnit - 1) / kUnit + 1;
+        const int bound = (units + P.min_upc - 1) / P.min_upc;
+        if (bound < grid_x) grid_x = bound < 1 ? 1 : bound;
+    }
+    const dim3 grid((unsigned)grid_x, (unsigned)(layout->local_kv_heads * P.q_subgroups),
+                    (unsigned)batch->total_tokens);
+    hipStream_t stream = (hipStream_t)ex->stream;
+    int rc = ensure_dynamic_lds(paged_attn_kv16_kernel<TQ, 1>, kv16_smem_bytes(1));
+    if (rc) return rc;
+    hipLaunchKernelGGL((paged_attn_kv16_kernel<TQ, 1>), grid, dim3(kKv16Waves * 64), kv16_smem_bytes(1), stream, P);
+    rc = (int)hipGetLastError();
+    if (rc) return rc;
+    if (P.max_chunks > 1) {
+        hipLaunchKernelGGL((split_merge_kernel<TQ>), dim3((unsigned)rows), dim3(1024), 0, stream, P, 1.0f, 0);
+        rc = (int)hipGetLastError();
+    }
+    return rc;
+}
+
+static bool is_kv16(const warp34_kv_layer_layout* l, int format) {
+    return l->head_dim == 256 && l->k_format == format && l->v_format == format &&
+           l->k_transform == WARP34_KV_TRANSFORM_IDENTITY && l->v_transform == WARP34_KV_TRANSFORM_IDENTITY;
+}
+
+static bool kv16_geometry_ok(const warp34_kv_layer_layout* l, const void* q, const void* out) {
+    return l->block_size > 0 && (l->block_size % 16) == 0 && l->k_token_stride_bytes == 512 &&
+           l->v_token_stride_bytes == 512 && (l->k_base & 15u) == 0 && (l->v_base & 15u) == 0 &&
+           (l->k_page_stride_bytes & 15u) == 0 && (l->k_head_stride_bytes & 15u) == 0 &&
+           (l->v_page_stride_bytes & 15u) == 0 && (l->v_head_stride_bytes & 15u) == 0 &&
+           (((uintptr_t)q) & 15u) == 0 && (((uintptr_t)out) & 7u) == 0;
+}
+
 static bool is_tq4_wht(const warp34_kv_layer_layout* l) {
     return l->head_dim == 256 && l->k_format == WARP34_KV_FORMAT_TQ4 && l->v_format == WARP34_KV_FORMAT_TQ4 &&
            l->k_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 &&
@@ -1136,6 +1209,12 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
     if (is_tq4_wht(layout)) {
         if (!tq4_geometry_ok(layout, q) || (((uintptr_t)out) & 7u) != 0) return (int)hipErrorNotSupported;
         return launch_tq4<TQ>(ex, layout, batch, q, out, num_q_heads, force_single);
+    }
+    // 16-bit pages: the storage type must be the query type (FP16 pages with the f16 entry
+    // point, BF16 pages with the bf16 one, as in the reference)
+    if (is_kv16(layout, TQ::kStorageFormat)) {
+        if (!kv16_geometry_ok(layout, q, out)) return (int)hipErrorNotSupported;
+        return launch_kv16<TQ>(ex, layout, batch, q, out, num_q_heads, force_single);
     }
     return (int)hipErrorNotSupported;
 }

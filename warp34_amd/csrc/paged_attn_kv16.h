@@ -1,0 +1,458 @@
+// Paged GQA decode / verify attention over 16-bit KV pages (FP16 or BF16 storage, identity
+// transform) for gfx950.  Same work decomposition, chunk geometry, wave merge and split-K
+// partial format as the TQ4 kernel in paged_attn.hip (which includes this file); only the
+// per-unit body differs:
+//   * a 32-token unit is processed as two 16-token halves; the wave copies the 16 K rows and
+//     16 V rows of a half (512 B each) into its private LDS area with a 528-byte row stride
+//     (132 dwords: the 8 lanes of a 128-bit read pass land on 32 distinct banks);
+//   * S^T = K Q^T: A operand = 16 K rows read straight from LDS (8 x 128-bit reads),
+//     B operand = the query rows, loaded once from global memory in MFMA layout;
+//   * O^T += V^T P^T with 16x16x16 MFMAs: each lane reads the 8-element slice of its 4 tokens
+//     and transposes the 4x8 block of 16-bit values in registers with v_perm_b32;
+//   * BF16 storage: P is split into a bf16 high and low part (two MFMAs) so that the 8-bit
+//     mantissa of bf16 does not limit the accuracy of the weighted sum.
+// Replaces paged_attention_gqa_bf16_kernel (op_kv_cache.cu:873-1168) and the FP16 branch of
+// paged_attention_gqa_mma_f16_kernel (op_paged_attn.cu:186-588).
+#pragma once
+
+namespace w34 {
+
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef short s4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u2v __attribute__((ext_vector_type(2)));
+
+constexpr int kKv16Waves = 8;
+constexpr int kKv16RowStride = 528;                      // bytes, 512 + 16 pad
+constexpr int kKv16Stage = 2 * 16 * kKv16RowStride;      // K half + V half: 16896 B per wave
+// byte offset of the (m, l) exchange table: behind both the staging areas and the merge regions
+__host__ __device__ constexpr int kv16_ml_offset(int nt) {
+    const int loop_bytes = kKv16Waves * kKv16Stage;
+    const int region_bytes = kKv16Waves * (nt * 16 * 260) * 4;
+    return loop_bytes > region_bytes ? loop_bytes : region_bytes;
+}
+__host__ __device__ constexpr int kv16_smem_bytes(int nt) {
+    return kv16_ml_offset(nt) + (kKv16Waves + 1) * nt * 16 * 2 * 4 + 256;
+}
+
+template <bool IS_BF16>
+__device__ __forceinline__ f4 mfma_x32(u4 a, u4 b, f4 c) {
+    if constexpr (IS_BF16) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8, a), __builtin_bit_cast(bf8, b), c, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a), __builtin_bit_cast(h8, b), c, 0, 0, 0);
+    }
+}
+template <bool IS_BF16>
+__device__ __forceinline__ f4 mfma_x16(u2v a, u2v b, f4 c) {
+    if constexpr (IS_BF16) {
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s4, a), __builtin_bit_cast(s4, b), c, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h4, a), __builtin_bit_cast(h4, b), c, 0, 0, 0);
+    }
+}
+
+// TQ doubles as the storage type: F16 query/output over FP16 pages, BF16 over BF16 pages.
+template <typename TQ, int NT>
+__global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(const AttnParams P) {
+    constexpr bool IS_BF16 = TQ::kStorageFormat == WARP34_KV_FORMAT_BF16;
+    constexpr int kWaves = kKv16Waves;
+    extern __shared__ __align__(16) uint8_t smem[];
+
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15;
+    const int b = lane >> 4;
+    const warp34_kv_layer_layout& L = P.L;
+    const warp34_attention_batch& B = P.B;
+
+    const int tok0 = (int)blockIdx.z;
+    const int kv_sub = (int)blockIdx.y;
+    const int kv_head = kv_sub / P.q_subgroups;
+    const int q_head_base = kv_head * P.gqa + (kv_sub % P.q_subgroups) * P.q_group;
+    const int chunk = (int)blockIdx.x;
+    if (tok0 >= B.total_tokens) return;
+
+    // query rows in MFMA B layout straight from global memory: lane (n, b) holds
+    // Q[column n][32 m + 8 b .. + 7] for m = 0..7 (dead columns are zeroed below)
+    u4 bq[NT][8];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int col = nt * 16 + n;
+        const int t = col / P.q_group;
+        const int a = col - t * P.q_group;
+        const int tok = min(tok0 + t, B.total_tokens - 1);
+        const uint16_t* qrow = P.q + ((size_t)tok * P.num_q_heads + (size_t)(q_head_base + a)) * kHeadDim;
+#pragma unroll
+        for (int m = 0; m < 8; ++m) bq[nt][m] = *reinterpret_cast<const u4*>(qrow + 32 * m + 8 * b);
+    }
+
+    // request lookup in one round trip (see the TQ4 kernel)
+    bool req_hit = false;
+    int req = -1, rq_start = 0, rq_end = 0, seq_after = 0, ctx_before = 0;
+    for (int base = 0; base < B.num_reqs && !req_hit; base += 64) {
+        const int r = base + lane;
+        const bool inb = r < B.num_reqs;
+        const int lo = inb ? B.query_start_loc[r] : 0x7fffffff;
+        const int hi = inb ? B.query_start_loc[r + 1] : -0x7fffffff;
+        const int sa = inb ? B.seq_lens_after[r] : 0;
+        const int cb = (inb && B.context_lens_before != nullptr) ? B.context_lens_before[r] : 0;
+        const int rm = (inb && B.valid_req_mask != nullptr) ? (int)B.valid_req_mask[r] : 1;
+        const unsigned long long hits = __ballot(inb && tok0 >= lo && tok0 < hi);
+        if (hits != 0ull) {
+            const int src = __builtin_ctzll(hits);
+            req = base + src;
+            rq_start = __builtin_amdgcn_readlane(lo, src);
+            rq_end = __builtin_amdgcn_readlane(hi, src);
+            seq_after = __builtin_amdgcn_readlane(sa, src);
+            ctx_before = B.context_lens_before != nullptr ? __builtin_amdgcn_readlane(cb, src)
+                                                          : seq_after - (rq_end - rq_start);
+            req_hit = __builtin_amdgcn_readlane(rm, src) != 0;
+            if (!req_hit) break;
+        }
+    }
+    bool tok_ok[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int tok = tok0 + (nt * 16 + n) / P.q_group;
+        tok_ok[nt] = tok < B.total_tokens &&
+                     (B.valid_token_mask == nullptr || B.valid_token_mask[min(tok, B.total_tokens - 1)] != 0);
+    }
+    if (!req_hit) return;
+    if (((tok0 - rq_start) % P.tok_tile) != 0) return;
+    int tile_tokens = rq_end - tok0;
+    if (tile_tokens > P.tok_tile) tile_tokens = P.tok_tile;
+
+    int col_lo[NT], col_hi[NT];
+    bool col_ok[NT];
+    int u_lo = 0x7fffffff, u_hi = -1;
+    int i_lo = 0, i_hi = 0x7fffffff;
+    uint32_t ok_mask[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int col = nt * 16 + n;
+        const int t = col / P.q_group;
+        const int tok = tok0 + t;
+        const bool ok = t < tile_tokens && tok_ok[nt];
+        const int q_off = tok - rq_start;
+        int mx = (B.mask_mode == WARP34_ATTN_MASK_NONCAUSAL_WINDOW) ? seq_after - 1 : ctx_before + q_off;
+        if (mx >= seq_after) mx = seq_after - 1;
+        int mn = 0;
+        if (B.sliding_window > 0) mn = max(0, ctx_before + q_off - B.sliding_window + 1);
+        col_ok[nt] = ok;
+        col_lo[nt] = ok ? mn : 0;
+        col_hi[nt] = ok ? mx : -1;
+        if (ok) {
+            i_lo = max(i_lo, mn);
+            i_hi = min(i_hi, mx);
+            if (mn <= mx) {
+                u_lo = min(u_lo, mn);
+                u_hi = max(u_hi, mx);
+            }
+        } else {
+#pragma unroll
+            for (int m = 0; m < 8; ++m) bq[nt][m] = u4{0u, 0u, 0u, 0u};
+        }
+        ok_mask[nt] = (uint32_t)(__ballot(ok) & 0xFFFFull);
+    }
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+        u_lo = min(u_lo, __shfl_xor(u_lo, off, 64));
+        u_hi = max(u_hi, __shfl_xor(u_hi, off, 64));
+        i_lo = max(i_lo, __shfl_xor(i_lo, off, 64));
+        i_hi = min(i_hi, __shfl_xor(i_hi, off, 64));
+    }
+    {
+        uint32_t any = 0;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) any |= ok_mask[nt];
+        if (any == 0u) return;
+    }
+    if (u_hi < 0) u_lo = 0;
+    u_lo = __builtin_amdgcn_readfirstlane(u_lo);
+    u_hi = __builtin_amdgcn_readfirstlane(u_hi);
+    i_lo = __builtin_amdgcn_readfirstlane(i_lo);
+    i_hi = __builtin_amdgcn_readfirstlane(i_hi);
+
+    const ChunkGeom g = chunk_geom(u_lo, u_hi, P.max_chunks, P.min_upc);
+    if (chunk >= g.n_chunks) return;
+    const int cu_first = g.u_first + chunk * g.upc;
+    int cu_end = cu_first + g.upc;
+    if (cu_end > g.u_first + g.n_units) cu_end = g.u_first + g.n_units;
+
+    const uint8_t* k_base = reinterpret_cast<const uint8_t*>((uintptr_t)L.k_base) +
+                            (size_t)kv_head * L.k_head_stride_bytes;
+    const uint8_t* v_base = reinterpret_cast<const uint8_t*>((uintptr_t)L.v_base) +
+                            (size_t)kv_head * L.v_head_stride_bytes;
+    uint8_t* stage = smem + wave * kKv16Stage;  // [K rows 0..15][V rows 0..15], 528 B each
+    const int32_t* req_blocks = B.block_tables + (size_t)req * B.max_blocks_per_req;
+    int slot_base = (cu_first * kUnit) / L.block_size;
+    int page_vec;
+    auto load_page_vec = [&]() {
+        const int slot = slot_base + lane;
+        page_vec = slot < B.max_blocks_per_req ? req_blocks[slot] : -1;
+    };
+
+    // A half = 16 consecutive tokens: 8 KiB of K and 8 KiB of V, each contiguous inside one
+    // page.  Piece c = lane + 64 i (16 B) is element column c % 32 of row c / 32.
+    u4 pf[16];
+    auto issue_half = [&](int hidx) {  // hidx = 2 * unit + half
+        const int pos = hidx * 16;
+        const int page_slot = pos / L.block_size;
+        const int in_page = pos - page_slot * L.block_size;
+        int rel = page_slot - slot_base;
+        if (rel >= 64) {
+            slot_base = page_slot;
+            load_page_vec();
+            rel = 0;
+        }
+        const int32_t pg = __builtin_amdgcn_readlane(page_vec, rel);
+        const bool live = pos <= u_hi && pos + 15 >= u_lo && pg >= 0;
+        const uint8_t* kp = k_base + (live ? (size_t)pg * L.k_page_stride_bytes + (size_t)in_page * L.k_token_stride_bytes : 0);
+        const uint8_t* vp = v_base + (live ? (size_t)pg * L.v_page_stride_bytes + (size_t)in_page * L.v_token_stride_bytes : 0);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            pf[i] = *(global_cu4*)(kp + 16 * lane + 1024 * i);
+            pf[8 + i] = *(global_cu4*)(vp + 16 * lane + 1024 * i);
+        }
+    };
+    // rows outside [u_lo, u_hi] are stored as zeros: unwritten pool memory may hold NaN
+    // patterns, and 0 * NaN would poison the P V product
+    auto commit_half = [&](int hidx) {
+        const int pos0 = hidx * 16;
+        const bool edge = pos0 < u_lo || pos0 + 15 > u_hi;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int c = lane + 64 * i;
+            const int row = c >> 5;
+            u4 kv = pf[i], vv = pf[8 + i];
+            if (edge) {
+                const bool vis = pos0 + row >= u_lo && pos0 + row <= u_hi;
+                if (!vis) {
+                    kv = u4{0u, 0u, 0u, 0u};
+                    vv = u4{0u, 0u, 0u, 0u};
+                }
+            }
+            *reinterpret_cast<u4*>(stage + row * kKv16RowStride + 16 * (c & 31)) = kv;
+            *reinterpret_cast<u4*>(stage + 16 * kKv16RowStride + row * kKv16RowStride + 16 * (c & 31)) = vv;
+        }
+    };
+
+    f4 o_acc[NT][2][8];
+    float m_run[NT], l_run[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        m_run[nt] = kNegBig;
+        l_run[nt] = 0.f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o_acc[nt][h][j] = f4{0.f, 0.f, 0.f, 0.f};
+    }
+    const float score_scale = B.sm_scale * kLog2e;
+
+    auto process_half = [&](int pos0, const bool MASKED) {
+        const uint8_t* k_rows = stage;
+        const uint8_t* v_rows = stage + 16 * kKv16RowStride;
+        // ---- S^T = K Q^T: A row n = token n of the half ----
+        f4 s_acc[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) s_acc[nt] = f4{0.f, 0.f, 0.f, 0.f};
+        u4 ka[8];
+#pragma unroll
+        for (int m = 0; m < 8; ++m)
+            ka[m] = *reinterpret_cast<const u4*>(k_rows + n * kKv16RowStride + 64 * m + 16 * b);
+#pragma unroll
+        for (int m = 0; m < 8; ++m)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) s_acc[nt] = mfma_x32<IS_BF16>(ka[m], bq[nt][m], s_acc[nt]);
+
+        // raw V slices of this lane's 4 tokens (rows 4b..4b+3), both halves of the head dim
+        u4 vr[2][4];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                vr[h][i] = *reinterpret_cast<const u4*>(v_rows + (4 * b + i) * kKv16RowStride + 256 * h + 16 * n);
+
+        // ---- online softmax over this lane's 4 tokens ----
+        u2v pb_hi[NT], pb_lo[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            float sc[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                sc[i] = s_acc[nt][i] * score_scale;
+                if (MASKED) {
+                    const int pos = pos0 + 4 * b + i;
+                    const bool vis = col_ok[nt] && pos >= col_lo[nt] && pos <= col_hi[nt];
+                    sc[i] = vis ? sc[i] : kNegBig;
+                }
+            }
+            float mx = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+            mx = max_over_rows(mx);
+            const float m_new = fmaxf(m_run[nt], mx);
+            const float alpha = __builtin_amdgcn_exp2f(m_run[nt] - m_new);
+            m_run[nt] = m_new;
+            float p[4];
+            float psum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                p[i] = __builtin_amdgcn_exp2f(sc[i] - m_new);
+                if (MASKED) p[i] = sc[i] > 0.5f * kNegBig ? p[i] : 0.f;
+                psum += p[i];
+            }
+            l_run[nt] = l_run[nt] * alpha + psum;
+            if (__ballot(alpha != 1.0f) != 0ull) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) o_acc[nt][h][j] *= alpha;
+            }
+            if constexpr (IS_BF16) {
+                uint32_t hb[4], lb[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    hb[i] = BF16::from_f32(p[i]);
+                    lb[i] = BF16::from_f32(p[i] - BF16::to_f32((uint16_t)hb[i]));
+                }
+                pb_hi[nt] = u2v{hb[0] | (hb[1] << 16), hb[2] | (hb[3] << 16)};
+                pb_lo[nt] = u2v{lb[0] | (lb[1] << 16), lb[2] | (lb[3] << 16)};
+            } else {
+                pb_hi[nt] = u2v{pack_h2(p[0], p[1]), pack_h2(p[2], p[3])};
+                pb_lo[nt] = u2v{0u, 0u};
+            }
+        }
+
+        // ---- O^T += V^T P^T: row r = n of MFMA (h, j) is head dimension 128 h + 8 n + j ----
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                // 16-bit element j of the four token slices -> (t0,t1), (t2,t3)
+                const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+                u2v a;
+                a[0] = __builtin_amdgcn_perm(vr[h][1][j >> 1], vr[h][0][j >> 1], sel);
+                a[1] = __builtin_amdgcn_perm(vr[h][3][j >> 1], vr[h][2][j >> 1], sel);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    o_acc[nt][h][j] = mfma_x16<IS_BF16>(a, pb_hi[nt], o_acc[nt][h][j]);
+                    if constexpr (IS_BF16) o_acc[nt][h][j] = mfma_x16<IS_BF16>(a, pb_lo[nt], o_acc[nt][h][j]);
+                }
+            }
+        }
+    };
+
+    // halves of this wave's units, in order; the next half is in flight while one is processed
+    int unit = cu_first + wave;
+    load_page_vec();
+    int hidx = 2 * unit;
+    issue_half(hidx);
+    while (unit < cu_end) {
+        commit_half(hidx);
+        int next_h = hidx + 1, next_unit = unit;
+        if (next_h & 1) {
+            // second half of the same unit
+        } else {
+            next_unit = unit + kWaves;
+            next_h = 2 * next_unit;
+        }
+        if (next_unit < cu_end) issue_half(next_h);
+        const int pos0 = hidx * 16;
+        if (pos0 <= u_hi) process_half(pos0, !(pos0 >= i_lo && pos0 + 15 <= i_hi));
+        hidx = next_h;
+        unit = next_unit;
+    }
+
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) l_run[nt] = sum_over_rows(l_run[nt]);
+
+    // ---- merge of the waves' states (same scheme and region layout as the TQ4 kernel) ----
+    constexpr int kColStride = 260;
+    constexpr int kRegion = NT * 16 * kColStride;
+    float* xbuf = reinterpret_cast<float*>(smem);
+    float* mlbuf = reinterpret_cast<float*>(smem + kv16_ml_offset(NT));
+    static_assert(kv16_ml_offset(NT) >= kWaves * kRegion * 4 && kv16_ml_offset(NT) >= kWaves * kKv16Stage,
+                  "(m, l) table must not alias live LDS");
+    if (b == 0) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            mlbuf[(wave * NT * 16 + nt * 16 + n) * 2 + 0] = m_run[nt];
+            mlbuf[(wave * NT * 16 + nt * 16 + n) * 2 + 1] = l_run[nt];
+        }
+    }
+    __syncthreads();
+    float m_tot[NT], l_tot[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        float mt = kNegBig;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) mt = fmaxf(mt, mlbuf[(w * NT * 16 + nt * 16 + n) * 2]);
+        float lt = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w)
+            lt += mlbuf[(w * NT * 16 + nt * 16 + n) * 2 + 1] *
+                  __builtin_amdgcn_exp2f(mlbuf[(w * NT * 16 + nt * 16 + n) * 2] - mt);
+        m_tot[nt] = mt;
+        l_tot[nt] = lt;
+        const float wgt = __builtin_amdgcn_exp2f(m_run[nt] - mt);
+        float* c = xbuf + wave * kRegion + (nt * 16 + n) * kColStride;
+        if (col_ok[nt]) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    *reinterpret_cast<f4*>(c + ((h * 8 + j) * 4 + b) * 4) = o_acc[nt][h][j] * wgt;
+        }
+    }
+    float* mltot = mlbuf + kWaves * NT * 16 * 2;
+    if (wave == 0 && b == 0) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            mltot[(nt * 16 + n) * 2 + 0] = m_tot[nt];
+            mltot[(nt * 16 + n) * 2 + 1] = l_tot[nt];
+        }
+    }
+    __syncthreads();
+
+    // element e = 128 h + 8 r + j sits in slot ((h*8 + j)*4 + (r >> 2))*4 + (r & 3)
+    int merge_slot[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int e = 4 * lane + k;
+        const int h = e >> 7, r = (e >> 3) & 15, j = e & 7;
+        merge_slot[k] = ((h * 8 + j) * 4 + (r >> 2)) * 4 + (r & 3);
+    }
+    for (int col = wave; col < 16 * NT; col += kWaves) {
+        const int t = col / P.q_group;
+        const int a = col - t * P.q_group;
+        if (!((ok_mask[col >> 4] >> (col & 15)) & 1u)) continue;
+        const size_t row = (size_t)(tok0 + t) * P.num_q_heads + (size_t)(q_head_base + a);
+        float v[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            const float* c = xbuf + w * kRegion + col * kColStride;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) v[k] += c[merge_slot[k]];
+        }
+        const float m_col = mltot[col * 2 + 0];
+        const float l_col = mltot[col * 2 + 1];
+        if (P.max_chunks > 1) {
+            float* dst = P.part_acc + (row * P.max_chunks + chunk) * kHeadDim;
+            *reinterpret_cast<f4*>(dst + 4 * lane) = f4{v[0], v[1], v[2], v[3]};
+            if (lane == 0) {
+                *reinterpret_cast<f4*>(P.part_ml + (row * P.max_chunks + chunk) * 4) =
+                    f4{m_col, l_col, (float)g.n_chunks, 0.f};
+            }
+        } else {
+            const float inv = l_col > 0.f ? 1.0f / l_col : 0.f;
+            uint2 o;
+            o.x = (uint32_t)TQ::from_f32(v[0] * inv) | ((uint32_t)TQ::from_f32(v[1] * inv) << 16);
+            o.y = (uint32_t)TQ::from_f32(v[2] * inv) | ((uint32_t)TQ::from_f32(v[3] * inv) << 16);
+            *reinterpret_cast<uint2*>(P.out + row * kHeadDim + 4 * lane) = o;
+        }
+    }
+}
+
+}  // namespace w34
