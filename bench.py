@@ -25,7 +25,13 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 KV_HEADS, Q_HEADS, HEAD_DIM, BLOCK = 2, 16, 256, 64
-ROW_BYTES = 132
+ROW_BYTES = {"tq4": 132, "bf16": 512}
+WORKLOADS = {
+    # name: (kv format, context lengths or None for the seeded 32-sequence draw, pool tokens)
+    "tq4_decode_b1_ctx131072": ("tq4", [131072], 0),
+    "tq4_decode_b32_ctx1k_64k": ("tq4", None, 2 << 20),
+    "bf16_decode_b1_ctx32768": ("bf16", [32768], 0),
+}
 
 
 def parse():
@@ -34,7 +40,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="tq4_decode_b1_ctx131072",
-                    choices=["tq4_decode_b1_ctx131072", "tq4_decode_b32_ctx1k_64k"])
+                    choices=sorted(WORKLOADS))
     ap.add_argument("--ctx", type=int, default=0, help="override: one request with this context length")
     ap.add_argument("--layers", type=int, default=0, help="KV pools to cycle through (0 = auto, > 256 MB total)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -43,27 +49,26 @@ def parse():
 
 
 def build_workload(name, seed=0):
-    rng = np.random.default_rng(seed)
-    if name == "tq4_decode_b1_ctx131072":
-        ctx = np.array([131072], dtype=np.int64)
-    else:
-        ctx = rng.integers(1024, 65537, size=32).astype(np.int64)
-    return ctx
+    fmt, ctx, pool_tokens = WORKLOADS[name]
+    if ctx is None:
+        ctx = np.random.default_rng(seed).integers(1024, 65537, size=32)
+    return fmt, np.asarray(ctx, dtype=np.int64), pool_tokens
 
 
 class Layer:
-    """One layer's TQ4 pool on the device, filled through the append kernel."""
+    """One layer's KV pool on the device, filled through the append kernel."""
 
-    def __init__(self, torch, lib, ffi, ctx, pool_pages, seed):
+    def __init__(self, torch, lib, ffi, fmt, ctx, pool_pages, seed):
         dev = "cuda:0"
-        self.tok, self.head = ROW_BYTES, BLOCK * ROW_BYTES
+        self.tok, self.head = ROW_BYTES[fmt], BLOCK * ROW_BYTES[fmt]
         self.page = KV_HEADS * self.head
         self.k = torch.zeros(pool_pages * self.page, dtype=torch.uint8, device=dev)
         self.v = torch.zeros(pool_pages * self.page, dtype=torch.uint8, device=dev)
+        kv_format = ffi.WARP34_KV_FORMAT_TQ4 if fmt == "tq4" else ffi.WARP34_KV_FORMAT_BF16
+        xf = ffi.WARP34_KV_TRANSFORM_RADEMACHER_WHT256 if fmt == "tq4" else ffi.WARP34_KV_TRANSFORM_IDENTITY
         self.layout = ffi.Warp34KvLayerLayout(
             self.k.data_ptr(), self.v.data_ptr(), self.page, self.head, self.tok, self.page, self.head, self.tok,
-            0, seed, KV_HEADS, HEAD_DIM, BLOCK, ffi.WARP34_KV_FORMAT_TQ4, ffi.WARP34_KV_FORMAT_TQ4,
-            ffi.WARP34_KV_TRANSFORM_RADEMACHER_WHT256, ffi.WARP34_KV_TRANSFORM_RADEMACHER_WHT256, 0)
+            0, seed, KV_HEADS, HEAD_DIM, BLOCK, kv_format, kv_format, xf, xf, 0)
         g = torch.Generator(device=dev)
         g.manual_seed(1000 + seed)
         pages_per = [(int(c) + BLOCK - 1) // BLOCK for c in ctx]
@@ -130,7 +135,7 @@ def cpu_baseline(ctx_len, threads):
     t0 = time.perf_counter()
     oracle.paged_attention(pool, hb, q, oracle.DT_BF16, Q_HEADS, n_threads=threads)
     dt = time.perf_counter() - t0
-    kv_bytes = ctx_len * KV_HEADS * 2 * ROW_BYTES
+    kv_bytes = ctx_len * KV_HEADS * 2 * ROW_BYTES["tq4"]
     return {
         "value": round(kv_bytes / dt / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
         "sample": "CPU oracle (oracle/tq4_oracle.c), 1 layer decode attention, ctx %d tokens, %d pthreads: "
@@ -156,16 +161,17 @@ def main():
     lib = ffi.load()
     dev = "cuda:0"
     torch.cuda.set_device(0)
-    ctx = build_workload(args.workload)
+    fmt, ctx, pool_tokens = build_workload(args.workload)
     if args.ctx:
         ctx = np.array([args.ctx], dtype=np.int64)
-        args.workload = "tq4_decode_b1_ctx%d" % args.ctx
+        args.workload = "%s_decode_b1_ctx%d" % (fmt, args.ctx)
     total_tokens_kv = int(ctx.sum())
-    kv_bytes = total_tokens_kv * KV_HEADS * 2 * ROW_BYTES  # algorithmic bytes per step (K + V rows)
-    pool_pages = sum((int(c) + BLOCK - 1) // BLOCK for c in ctx) + 16
-    layer_bytes = 2 * pool_pages * KV_HEADS * BLOCK * ROW_BYTES
+    row_bytes = ROW_BYTES[fmt]
+    kv_bytes = total_tokens_kv * KV_HEADS * 2 * row_bytes  # algorithmic bytes per step (K + V rows)
+    pool_pages = max(sum((int(c) + BLOCK - 1) // BLOCK for c in ctx) + 16, pool_tokens // BLOCK)
+    layer_bytes = 2 * pool_pages * KV_HEADS * BLOCK * row_bytes
     n_layers = args.layers or max(2, -(-(640 << 20) // layer_bytes))
-    layers = [Layer(torch, lib, ffi, ctx, pool_pages, s) for s in range(n_layers)]
+    layers = [Layer(torch, lib, ffi, fmt, ctx, pool_pages, s) for s in range(n_layers)]
 
     R = len(ctx)
     g = torch.Generator(device=dev)
@@ -209,7 +215,7 @@ def main():
 
     gbs = kv_bytes / (ms_per_step * 1e-3) / 1e9
     result = {
-        "metric": "paged TQ4 decode attn: us/layer + achieved HBM GB/s (% peak) at 128K ctx",
+        "metric": "paged TQ4 decode attn: \u00b5s/layer + achieved HBM GB/s (% peak) at 128K ctx",
         "value": round(gbs, 1),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -221,14 +227,16 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f16 MFMA operands (TQ4 codes -> fp16 centroids), f32 accumulate, bf16 Q/out",
+        "dtype": "f16 MFMA operands (TQ4 codes -> fp16 centroids), f32 accumulate, bf16 Q/out" if fmt == "tq4"
+                 else "bf16 MFMA operands, f32 accumulate, bf16 Q/out",
         "data": "synthetic",
         "config": {
             "workload": args.workload,
             "requests": R,
             "context_tokens_total": total_tokens_kv,
             "q_heads": Q_HEADS, "kv_heads": KV_HEADS, "head_dim": HEAD_DIM, "page_tokens": BLOCK,
-            "kv_format": "tq4+wht256", "kv_pools_cycled": n_layers,
+            "kv_format": "tq4+wht256" if fmt == "tq4" else "bf16", "kv_pools_cycled": n_layers,
+            "pool_pages": pool_pages,
             "kv_bytes_per_step": kv_bytes,
         },
         "roofline": {
@@ -238,7 +246,8 @@ def main():
             "unit": "GB/s",
             "frac": round(gbs / HBM_PEAK_GBS, 4),
             "traffic": None,
-            "kernel": "paged_attn_tq4_kernel (+ split_merge_kernel, both inside the timed launch)",
+            "kernel": "paged_attn_%s_kernel (+ split_merge_kernel, both inside the timed launch)"
+                      % ("tq4" if fmt == "tq4" else "kv16"),
             "avg_launch_us": round(ms_per_step * 1e3, 3),
             "host_wall_us_per_step": round(t_wall / args.steps * 1e6, 2),
         },

@@ -25,6 +25,7 @@ SOURCES = [
     (os.path.join(CSRC, "paged_attn.hip"), []),
     (os.path.join(CSRC, "runtime.hip"), []),
     (os.path.join(HOST, "kv_host.cpp"), []),
+    (os.path.join(HOST, "kv_host_runtime.cpp"), []),
 ]
 
 
@@ -41,8 +42,6 @@ def build(verbose=False):
     os.makedirs(BUILD, exist_ok=True)
     objs = []
     for src, extra in SOURCES:
-        if not os.path.exists(src):
-            continue
         obj = os.path.join(BUILD, os.path.basename(src) + ".o")
         is_hip = src.endswith(".hip")
         cmd = ["hipcc"] + COMMON + (DEVICE if is_hip else ["-x", "c++"]) + extra + ["-c", src, "-o", obj]
