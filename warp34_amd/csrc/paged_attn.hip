@@ -111,6 +111,19 @@ __device__ __forceinline__ constexpr int unit_token(int s, int b, int i) {
 }
 
 // chunk geometry of a tile
+// a / b for 0 <= a < 2^21 and 0 < b: the float quotient is within one of the exact result,
+// one correction step makes it exact.  A runtime integer division costs ~40 dependent
+// instructions on this hardware, and the prologue and the per-unit address arithmetic
+// divide by block sizes and group sizes that only the descriptors know.
+__device__ __forceinline__ int fast_div(int a, int b) {
+    if (a >= (1 << 21)) return a / b;
+    int q = (int)((float)a * __builtin_amdgcn_rcpf((float)b));
+    const int r = a - q * b;
+    q += r >= b ? 1 : 0;
+    q -= r < 0 ? 1 : 0;
+    return q;
+}
+
 struct ChunkGeom {
     int u_first, n_units, upc, n_chunks;
 };
@@ -118,12 +131,12 @@ __device__ __forceinline__ ChunkGeom chunk_geom(int u_lo, int u_hi, int max_chun
     ChunkGeom g;
     g.u_first = u_lo >> 5;
     g.n_units = (u_hi >= u_lo) ? ((u_hi >> 5) - g.u_first + 1) : 0;
-    int nc = (g.n_units + min_upc - 1) / min_upc;
+    int nc = fast_div(g.n_units + min_upc - 1, min_upc);
     if (nc > max_chunks) nc = max_chunks;
     if (nc < 1) nc = 1;
-    g.upc = (g.n_units + nc - 1) / nc;
+    g.upc = fast_div(g.n_units + nc - 1, nc);
     if (g.upc < 1) g.upc = 1;
-    g.n_chunks = (g.n_units + g.upc - 1) / g.upc;
+    g.n_chunks = fast_div(g.n_units + g.upc - 1, g.upc);
     if (g.n_chunks < 1) g.n_chunks = 1;
     return g;
 }
@@ -268,8 +281,8 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
     // ---- tile identification (wave-uniform, scalar loads) -------------------------------------
     const int tok0 = (int)blockIdx.z;
     const int kv_sub = (int)blockIdx.y;
-    const int kv_head = kv_sub / P.q_subgroups;
-    const int q_head_base = kv_head * P.gqa + (kv_sub % P.q_subgroups) * P.q_group;
+    const int kv_head = fast_div(kv_sub, P.q_subgroups);
+    const int q_head_base = kv_head * P.gqa + (kv_sub - kv_head * P.q_subgroups) * P.q_group;
     const int chunk = (int)blockIdx.x;
 
     W34_TP(0);
@@ -282,7 +295,7 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
 #pragma unroll
     for (int c = 0; c < kColsPerWave; ++c) {
         const int col = wave + c * kWaves;
-        const int t = col / P.q_group;
+        const int t = fast_div(col, P.q_group);
         const int a = col - t * P.q_group;
         q_raw[c] = uint2{0u, 0u};
         if (col < 16 * NT && tok0 + t < B.total_tokens) {
@@ -295,6 +308,19 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
     // matching request wins, as in the linear scan of op_kv_cache.cu:385-398) and carries that
     // request's lengths, which are then broadcast with readlane.  Every token of the tile
     // belongs to this request, so its key ranges follow from two scalars (op_kv_cache.cu:406-424).
+    // Speculative block-table load, in flight together with the request lookup: it assumes
+    // that token t belongs to request t (a decode batch) and that the request's length is the
+    // host's bound max_seq_len.  When either guess is wrong the ids are fetched again below,
+    // so the guess changes the latency only, never the result.
+    const int spec_req = min(tok0, B.num_reqs - 1);
+    int spec_slot_base = -1, spec_vec = -1;
+    if (B.sliding_window <= 0 && B.max_seq_len > 0 && spec_req >= 0) {
+        const ChunkGeom sg = chunk_geom(0, B.max_seq_len - 1, P.max_chunks, P.min_upc);
+        spec_slot_base = fast_div((sg.u_first + chunk * sg.upc) * kUnit, L.block_size);
+        const int slot = spec_slot_base + lane;
+        if (slot < B.max_blocks_per_req)
+            spec_vec = B.block_tables[(size_t)spec_req * B.max_blocks_per_req + slot];
+    }
     bool req_hit = false;
     int req = -1, rq_start = 0, rq_end = 0, seq_after = 0, ctx_before = 0;
     for (int base = 0; base < B.num_reqs && !req_hit; base += 64) {
@@ -322,7 +348,7 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
     bool tok_ok[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-        const int tok = tok0 + (nt * 16 + n) / P.q_group;
+        const int tok = tok0 + fast_div(nt * 16 + n, P.q_group);
         tok_ok[nt] = tok < B.total_tokens &&
                      (B.valid_token_mask == nullptr || B.valid_token_mask[min(tok, B.total_tokens - 1)] != 0);
     }
@@ -354,7 +380,7 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
 
     W34_TP(47);
     if (!req_hit) return;  // no owning request (or masked request): outputs untouched
-    if (((tok0 - rq_start) % P.tok_tile) != 0) return;  // not a tile leader
+    if ((tok0 - rq_start) - fast_div(tok0 - rq_start, P.tok_tile) * P.tok_tile != 0) return;  // not a tile leader
     int tile_tokens = rq_end - tok0;
     if (tile_tokens > P.tok_tile) tile_tokens = P.tok_tile;
 
@@ -367,7 +393,7 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         const int col = nt * 16 + n;
-        const int t = col / P.q_group;
+        const int t = fast_div(col, P.q_group);
         const int tok = tok0 + t;
         const bool ok = t < tile_tokens && tok_ok[nt];
         const int q_off = tok - rq_start;
@@ -430,7 +456,7 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
     // loads remain in the loop (they share the LDS wait counter and would serialise it).
     u4 pf[9];
     const int32_t* req_blocks = B.block_tables + (size_t)req * B.max_blocks_per_req;
-    int slot_base = (cu_first * kUnit) / L.block_size;
+    int slot_base = fast_div(cu_first * kUnit, L.block_size);
     int page_vec;
     auto load_page_vec = [&]() {
         const int slot = slot_base + lane;
@@ -445,7 +471,7 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
 #pragma unroll
         for (int gidx = 0; gidx < 2; ++gidx) {
             const int pos = unit * kUnit + 16 * gidx;
-            const int page_slot = pos / L.block_size;
+            const int page_slot = fast_div(pos, L.block_size);
             const int in_page = pos - page_slot * L.block_size;
             int rel = page_slot - slot_base;
             if (rel >= 64) {  // wave-uniform, at most once per 64 slots
@@ -482,7 +508,11 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
 
     // first unit's data goes in flight before the rest of the prologue
     int unit = cu_first + wave;
-    load_page_vec();
+    if (req == spec_req && slot_base == spec_slot_base) {
+        page_vec = spec_vec;
+    } else {
+        load_page_vec();
+    }
     W34_TP(41);
     issue_loads(unit);  // harmless for a wave without work: dead runs read page 0
     W34_TP(42);
@@ -748,7 +778,7 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
         const int t0 = unit * kUnit;
         // The two waves that share a SIMD take turns at the higher issue priority, unit by
         // unit; with equal priorities the older wave always wins and finishes ~25 % earlier.
-        if ((((unit - cu_first) / kWaves) ^ (wave >> 2)) & 1) {
+        if ((((unit - cu_first) >> (kWaves == 8 ? 3 : 2)) ^ (wave >> 2)) & 1) {
             __builtin_amdgcn_s_setprio(1);
         } else {
             __builtin_amdgcn_s_setprio(0);
@@ -844,7 +874,7 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
         merge_slot[k] = ((h * 8 + j) * 4 + (r >> 2)) * 4 + (r & 3);
     }
     for (int col = wave; col < 16 * NT; col += kWaves) {
-        const int t = col / P.q_group;
+        const int t = fast_div(col, P.q_group);
         const int a = col - t * P.q_group;
         if (!((ok_mask[col >> 4] >> (col & 15)) & 1u)) continue;
         const size_t row = (size_t)(tok0 + t) * P.num_q_heads + (size_t)(q_head_base + a);

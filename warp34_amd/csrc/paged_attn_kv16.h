@@ -69,8 +69,8 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
 
     const int tok0 = (int)blockIdx.z;
     const int kv_sub = (int)blockIdx.y;
-    const int kv_head = kv_sub / P.q_subgroups;
-    const int q_head_base = kv_head * P.gqa + (kv_sub % P.q_subgroups) * P.q_group;
+    const int kv_head = fast_div(kv_sub, P.q_subgroups);
+    const int q_head_base = kv_head * P.gqa + (kv_sub - kv_head * P.q_subgroups) * P.q_group;
     const int chunk = (int)blockIdx.x;
     if (tok0 >= B.total_tokens) return;
 
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         const int col = nt * 16 + n;
-        const int t = col / P.q_group;
+        const int t = fast_div(col, P.q_group);
         const int a = col - t * P.q_group;
         const int tok = min(tok0 + t, B.total_tokens - 1);
         const uint16_t* qrow = P.q + ((size_t)tok * P.num_q_heads + (size_t)(q_head_base + a)) * kHeadDim;
@@ -89,6 +89,19 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
     }
 
     // request lookup in one round trip (see the TQ4 kernel)
+    // Speculative block-table load, in flight together with the request lookup: it assumes
+    // that token t belongs to request t (a decode batch) and that the request's length is the
+    // host's bound max_seq_len.  When either guess is wrong the ids are fetched again below,
+    // so the guess changes the latency only, never the result.
+    const int spec_req = min(tok0, B.num_reqs - 1);
+    int spec_slot_base = -1, spec_vec = -1;
+    if (B.sliding_window <= 0 && B.max_seq_len > 0 && spec_req >= 0) {
+        const ChunkGeom sg = chunk_geom(0, B.max_seq_len - 1, P.max_chunks, P.min_upc);
+        spec_slot_base = fast_div((sg.u_first + chunk * sg.upc) * kUnit, L.block_size);
+        const int slot = spec_slot_base + lane;
+        if (slot < B.max_blocks_per_req)
+            spec_vec = B.block_tables[(size_t)spec_req * B.max_blocks_per_req + slot];
+    }
     bool req_hit = false;
     int req = -1, rq_start = 0, rq_end = 0, seq_after = 0, ctx_before = 0;
     for (int base = 0; base < B.num_reqs && !req_hit; base += 64) {
@@ -115,12 +128,12 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
     bool tok_ok[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-        const int tok = tok0 + (nt * 16 + n) / P.q_group;
+        const int tok = tok0 + fast_div(nt * 16 + n, P.q_group);
         tok_ok[nt] = tok < B.total_tokens &&
                      (B.valid_token_mask == nullptr || B.valid_token_mask[min(tok, B.total_tokens - 1)] != 0);
     }
     if (!req_hit) return;
-    if (((tok0 - rq_start) % P.tok_tile) != 0) return;
+    if ((tok0 - rq_start) - fast_div(tok0 - rq_start, P.tok_tile) * P.tok_tile != 0) return;
     int tile_tokens = rq_end - tok0;
     if (tile_tokens > P.tok_tile) tile_tokens = P.tok_tile;
 
@@ -132,7 +145,7 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         const int col = nt * 16 + n;
-        const int t = col / P.q_group;
+        const int t = fast_div(col, P.q_group);
         const int tok = tok0 + t;
         const bool ok = t < tile_tokens && tok_ok[nt];
         const int q_off = tok - rq_start;
@@ -187,7 +200,7 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
                             (size_t)kv_head * L.v_head_stride_bytes;
     uint8_t* stage = smem + wave * kKv16Stage;  // [K rows 0..15][V rows 0..15], 528 B each
     const int32_t* req_blocks = B.block_tables + (size_t)req * B.max_blocks_per_req;
-    int slot_base = (cu_first * kUnit) / L.block_size;
+    int slot_base = fast_div(cu_first * kUnit, L.block_size);
     int page_vec;
     auto load_page_vec = [&]() {
         const int slot = slot_base + lane;
@@ -199,7 +212,7 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
     u4 pf[16];
     auto issue_half = [&](int hidx) {  // hidx = 2 * unit + half
         const int pos = hidx * 16;
-        const int page_slot = pos / L.block_size;
+        const int page_slot = fast_div(pos, L.block_size);
         const int in_page = pos - page_slot * L.block_size;
         int rel = page_slot - slot_base;
         if (rel >= 64) {
@@ -346,7 +359,11 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
 
     // halves of this wave's units, in order; the next half is in flight while one is processed
     int unit = cu_first + wave;
-    load_page_vec();
+    if (req == spec_req && slot_base == spec_slot_base) {
+        page_vec = spec_vec;
+    } else {
+        load_page_vec();
+    }
     int hidx = 2 * unit;
     issue_half(hidx);
     while (unit < cu_end) {
@@ -425,7 +442,7 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
         merge_slot[k] = ((h * 8 + j) * 4 + (r >> 2)) * 4 + (r & 3);
     }
     for (int col = wave; col < 16 * NT; col += kWaves) {
-        const int t = col / P.q_group;
+        const int t = fast_div(col, P.q_group);
         const int a = col - t * P.q_group;
         if (!((ok_mask[col >> 4] >> (col & 15)) & 1u)) continue;
         const size_t row = (size_t)(tok0 + t) * P.num_q_heads + (size_t)(q_head_base + a);
