@@ -31,21 +31,30 @@ WORKLOADS = {
     "tq4_decode_b1_ctx131072": ("tq4", [131072], 0),
     "tq4_decode_b32_ctx1k_64k": ("tq4", None, 2 << 20),
     "bf16_decode_b1_ctx32768": ("bf16", [32768], 0),
+    # 8 sequences, 16 384-token TQ4 prefix + 2 048-token bf16 chunk each: append + causal attention
+    "tq4_prefill_8x2048_ctx16384": ("tq4", [18432] * 8, 0),
 }
+PREFILL_CHUNK = 2048
 
 
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=0, help="timed steps (default 200; 10 for the prefill workload)")
+    ap.add_argument("--warmup", type=int, default=-1, help="untimed steps (default 20; 2 for the prefill workload)")
     ap.add_argument("--workload", default="tq4_decode_b1_ctx131072",
                     choices=sorted(WORKLOADS))
     ap.add_argument("--ctx", type=int, default=0, help="override: one request with this context length")
     ap.add_argument("--layers", type=int, default=0, help="KV pools to cycle through (0 = auto, > 256 MB total)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-ctx", type=int, default=32768, help="context length of the CPU-oracle sample")
-    return ap.parse_args()
+    args = ap.parse_args()
+    prefill = args.workload.startswith("tq4_prefill")
+    if args.steps <= 0:
+        args.steps = 10 if prefill else 200
+    if args.warmup < 0:
+        args.warmup = 2 if prefill else 20
+    return args
 
 
 def build_workload(name, seed=0):
@@ -88,7 +97,8 @@ class Layer:
             gain[h, idx] = 20.0
         stream = torch.cuda.current_stream().cuda_stream
         ex = ffi.Warp34Exec(stream, 0, 0, 0)
-        chunk = 8192
+        chunk = 2048
+        self.tail_k, self.tail_v, self.tail_slots = [], [], []
         for r, c in enumerate(ctx):
             c = int(c)
             for t0 in range(0, c, chunk):
@@ -106,6 +116,10 @@ class Layer:
                 if rc:
                     raise RuntimeError("warp34_kv_cache_write_bf16 rc=%d" % rc)
                 torch.cuda.synchronize()
+                if t0 + n == c:  # the request's last chunk, re-appended by the prefill workload
+                    self.tail_k.append(kk)
+                    self.tail_v.append(vv)
+                    self.tail_slots.append(slots)
 
 
 def cpu_baseline(ctx_len, threads):
@@ -145,6 +159,82 @@ def cpu_baseline(ctx_len, threads):
     }
 
 
+def run_prefill(args, torch, lib, ffi, layers, ctx, n_layers, pool_pages):
+    """Chunked prefill: every sequence re-appends its last PREFILL_CHUNK tokens (bf16 -> TQ4)
+    and attends causally over prefix + chunk.  One step = append + attention of one layer."""
+    dev = "cuda:0"
+    R, n = len(ctx), PREFILL_CHUNK
+    N = R * n
+    g = torch.Generator(device=dev)
+    g.manual_seed(7)
+    q = torch.randn((N, Q_HEADS, HEAD_DIM), generator=g, device=dev).to(torch.bfloat16)
+    out = torch.zeros_like(q)
+    qsl = (torch.arange(0, R + 1, dtype=torch.int32, device=dev) * n).to(torch.int32)
+    seq = torch.tensor(ctx, dtype=torch.int32, device=dev)
+    ctxb = (seq - n).to(torch.int32)
+    scratch_bytes = 32 << 20
+    scratch = torch.zeros(scratch_bytes, dtype=torch.uint8, device=dev)
+    ex = ffi.Warp34Exec(torch.cuda.current_stream().cuda_stream, scratch.data_ptr(), scratch_bytes, 0)
+    per_layer = []
+    for L in layers:
+        kk, vv, slots = torch.cat(L.tail_k), torch.cat(L.tail_v), torch.cat(L.tail_slots)
+        batch = ffi.Warp34AttentionBatch(
+            qsl.data_ptr(), ctxb.data_ptr(), seq.data_ptr(), L.block_tables.data_ptr(), slots.data_ptr(), None, None,
+            R, N, L.max_blocks, n, int(ctx.max()), 0, 0, 1.0 / 16.0, 0)
+        per_layer.append((L, kk, vv, slots, batch))
+
+    def step(i, append=True):
+        L, kk, vv, slots, batch = per_layer[i % n_layers]
+        if append:
+            rc = lib.warp34_kv_cache_write_bf16(C.byref(ex), C.byref(L.layout), C.byref(batch),
+                                                C.c_void_p(kk.data_ptr()), C.c_void_p(vv.data_ptr()))
+            if rc:
+                raise RuntimeError("warp34_kv_cache_write_bf16 rc=%d" % rc)
+        rc = lib.warp34_paged_attention_bf16(C.byref(ex), C.byref(L.layout), C.byref(batch),
+                                             C.c_void_p(q.data_ptr()), C.c_void_p(out.data_ptr()), Q_HEADS)
+        if rc:
+            raise RuntimeError("warp34_paged_attention_bf16 rc=%d" % rc)
+
+    def timed(append):
+        for i in range(args.warmup):
+            step(i, append)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(args.steps):
+            step(i, append)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    ms_attn = timed(False)
+    ms_step = timed(True)
+    assert torch.isfinite(out.float()).all()
+    # QK^T and PV: 2 x 2 x head_dim flops per (query row, visible key)
+    pairs = sum(sum(int(c) - n + i + 1 for i in range(n)) for c in ctx)
+    flops = 4.0 * HEAD_DIM * Q_HEADS * pairs
+    tf_step = flops / (ms_step * 1e-3) / 1e12
+    tf_attn = flops / (ms_attn * 1e-3) / 1e12
+    peak = 2500.0
+    print(json.dumps({
+        "metric": "chunked prefill over TQ4 pages (append + causal attention): ms/layer + achieved MFMA TFLOP/s",
+        "value": round(tf_step, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4), "ms_attention_only": round(ms_attn, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 MFMA operands (TQ4 codes -> fp16 centroids), f32 accumulate, bf16 Q/out",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "requests": R, "chunk_tokens": n, "prefix_tokens": int(ctx[0]) - n,
+                   "q_heads": Q_HEADS, "kv_heads": KV_HEADS, "head_dim": HEAD_DIM, "page_tokens": BLOCK,
+                   "kv_format": "tq4+wht256", "kv_pools_cycled": n_layers, "pool_pages": pool_pages,
+                   "attention_flops_per_step": flops, "rows_appended_per_step": N * KV_HEADS * 2},
+        "roofline": {"bound": "mfma", "achieved": round(tf_attn, 1), "peak": peak, "unit": "TFLOP/s",
+                     "frac": round(tf_attn / peak, 4), "traffic": None,
+                     "kernel": "paged_prefill_tq4_kernel (attention-only launches)",
+                     "avg_launch_us": round(ms_attn * 1e3, 1)},
+    }))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -172,6 +262,10 @@ def main():
     layer_bytes = 2 * pool_pages * KV_HEADS * BLOCK * row_bytes
     n_layers = args.layers or max(2, -(-(640 << 20) // layer_bytes))
     layers = [Layer(torch, lib, ffi, fmt, ctx, pool_pages, s) for s in range(n_layers)]
+
+    if args.workload.startswith("tq4_prefill"):
+        run_prefill(args, torch, lib, ffi, layers, ctx, n_layers, pool_pages)
+        return
 
     R = len(ctx)
     g = torch.Generator(device=dev)

@@ -212,3 +212,63 @@ def test_kv16_mismatched_query_type_is_refused():
     dpool = _dev_pool(pool)
     rc, got, _ = G.dev_attention(dpool, hb, q, DT_F16, 8)
     assert rc == 801 and (got == 0x5500).all()
+
+
+# ---- chunked prefill over TQ4 pages (128-row tile kernel) ----
+
+def _prefill_case(dtype, block_size, seq_lens, q_lens, seed, q_heads=16, force=None, **kw):
+    import gpu_harness as G
+
+    pool, bt, k, v, q, aq, ctx = make_case(FMT_TQ4, block_size, seq_lens, q_lens, seed, dtype, q_heads=q_heads)
+    hb = oracle.HostBatch(aq, seq_lens, bt, context_lens_before=ctx, **kw)
+    want = oracle.paged_attention(pool, hb, q, dtype, q_heads, n_threads=8)
+    dpool = _dev_pool(pool)
+    rc, got, _ = G.dev_attention(dpool, hb, q, dtype, q_heads, scratch_bytes=SCRATCH, force_kernel=force)
+    assert rc == 0
+    G.assert_close(got, dtype, want, what="prefill bs=%d seq=%s q=%s" % (block_size, seq_lens, q_lens),
+                   scale=G.channel_scale(v, dtype, hb, q_heads))
+    return pool, hb, q, got, want
+
+
+@pytest.mark.parametrize("block_size", [16, 64])
+def test_prefill_tile_kernel_forced_small(block_size):
+    """Ragged tiles: chunk lengths that are not multiples of the 16-token tile, one request with
+    no prefix, one whose chunk starts in the middle of a page."""
+    _prefill_case(DT_F16, block_size, [300, 77, 45], [150, 77, 3], 201, force=0)
+    _prefill_case(DT_F16, block_size, [33, 700], [1, 37], 202, q_heads=8, force=1)
+
+
+@pytest.mark.parametrize("dtype", [DT_BF16, DT_F16])
+def test_prefill_tile_kernel_auto_dispatch(dtype):
+    """Large enough for the dispatcher to pick the tile kernel by itself: 4 x 300 query tokens."""
+    _prefill_case(dtype, 64, [900, 300, 1300, 512], [300, 300, 300, 300], 211)
+
+
+@pytest.mark.parametrize("mask_mode,window", [(0, 100), (1, 0), (1, 64)])
+def test_prefill_tile_kernel_windows(mask_mode, window):
+    _prefill_case(DT_F16, 16, [400, 130], [90, 130], 221, force=0, mask_mode=mask_mode, sliding_window=window)
+
+
+def test_prefill_tile_kernel_masks_and_page_permutation():
+    import gpu_harness as G
+
+    seq_lens, q_lens = [200, 120, 64], [40, 50, 64]
+    outs = []
+    for perm_seed in (1, 2):
+        pool, bt, k, v, q, aq, ctx = make_case(FMT_TQ4, 16, seq_lens, q_lens, 231, DT_F16, perm_seed=perm_seed)
+        tmask = np.ones(sum(q_lens), dtype=np.uint8)
+        tmask[[0, 17, 41, 153]] = 0
+        rmask = np.array([1, 0, 1], dtype=np.uint8)
+        hb = oracle.HostBatch(aq, seq_lens, bt, context_lens_before=ctx, valid_token_mask=tmask, valid_req_mask=rmask)
+        want = oracle.paged_attention(pool, hb, q, DT_F16, 8)
+        dpool = _dev_pool(pool)
+        rc, got, _ = G.dev_attention(dpool, hb, q, DT_F16, 8, force_kernel=0, sentinel=0x5500)
+        assert rc == 0
+        dead = np.zeros(sum(q_lens), dtype=bool)
+        dead[[0, 17, 41, 153]] = True
+        dead[40:90] = True  # masked request
+        assert (got[dead] == 0x5500).all()
+        G.assert_close(got[~dead], DT_F16, want[~dead], what="prefill masks",
+                       scale=G.channel_scale(v, DT_F16, hb, 8)[~dead])
+        outs.append(got)
+    assert outs[0].tobytes() == outs[1].tobytes()

@@ -1028,6 +1028,7 @@ __global__ __launch_bounds__(1024) void split_merge_kernel(const AttnParams P, f
 }  // namespace w34
 
 #include "paged_attn_kv16.h"
+#include "paged_prefill_tq4.h"
 
 namespace w34 {
 
@@ -1192,6 +1193,55 @@ static int launch_kv16(const warp34_exec* ex, const warp34_kv_layer_layout* layo
     return rc;
 }
 
+// Chunked prefill over TQ4 pages: one workgroup per (128-row query tile, kv head x q subgroup,
+// request); no split (a prefill batch has thousands of tiles).
+static bool prefill_tq4_applicable(const warp34_kv_layer_layout* layout, const warp34_attention_batch* batch,
+                                   int num_q_heads) {
+    const int gqa = num_q_heads / layout->local_kv_heads;
+    int q_group = gqa;
+    if (q_group > 16) {
+        for (int d = 16; d >= 1; --d)
+            if (gqa % d == 0) {
+                q_group = d;
+                break;
+            }
+    }
+    return q_group > 0 && (q_group & (q_group - 1)) == 0 && batch->max_q_len > 0;
+}
+
+template <typename TQ>
+static int launch_prefill_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
+                              const warp34_attention_batch* batch, const void* q, void* out, int num_q_heads) {
+    AttnParams P;
+    P.L = *layout;
+    P.B = *batch;
+    P.q = (const uint16_t*)q;
+    P.out = (uint16_t*)out;
+    P.part_acc = nullptr;
+    P.part_ml = nullptr;
+    P.num_q_heads = num_q_heads;
+    P.gqa = num_q_heads / layout->local_kv_heads;
+    int q_group = P.gqa;
+    if (q_group > 16) {
+        for (int d = 16; d >= 1; --d)
+            if (P.gqa % d == 0) {
+                q_group = d;
+                break;
+            }
+    }
+    P.q_group = q_group;
+    P.q_subgroups = P.gqa / q_group;
+    P.tok_tile = kPfRows / q_group;
+    P.max_chunks = 1;
+    P.min_upc = kMinUnitsPerChunk;
+    const int tiles = (batch->max_q_len + P.tok_tile - 1) / P.tok_tile;
+    const dim3 grid((unsigned)tiles, (unsigned)(layout->local_kv_heads * P.q_subgroups), (unsigned)batch->num_reqs);
+    int rc = ensure_dynamic_lds(paged_prefill_tq4_kernel<TQ>, kPfSmem);
+    if (rc) return rc;
+    hipLaunchKernelGGL((paged_prefill_tq4_kernel<TQ>), grid, dim3(kPfWaves * 64), kPfSmem, (hipStream_t)ex->stream, P);
+    return (int)hipGetLastError();
+}
+
 static bool is_kv16(const warp34_kv_layer_layout* l, int format) {
     return l->head_dim == 256 && l->k_format == format && l->v_format == format &&
            l->k_transform == WARP34_KV_TRANSFORM_IDENTITY && l->v_transform == WARP34_KV_TRANSFORM_IDENTITY;
@@ -1238,6 +1288,12 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
     }
     if (is_tq4_wht(layout)) {
         if (!tq4_geometry_ok(layout, q) || (((uintptr_t)out) & 7u) != 0) return (int)hipErrorNotSupported;
+        // Many query rows per request and enough tiles to fill the chip: the tile kernel shares
+        // every dequantised key block between 128 query rows.  The test selector forces it.
+        const bool many_rows = batch->max_q_len >= 32 &&
+                               (long long)batch->total_tokens * num_q_heads >= 128ll * kPfRows;
+        if ((force_single || many_rows) && prefill_tq4_applicable(layout, batch, num_q_heads))
+            return launch_prefill_tq4<TQ>(ex, layout, batch, q, out, num_q_heads);
         return launch_tq4<TQ>(ex, layout, batch, q, out, num_q_heads, force_single);
     }
     // 16-bit pages: the storage type must be the query type (FP16 pages with the f16 entry
