@@ -30,8 +30,7 @@ constexpr int kPfDeqBytes = kPfKBytes + kPfVBytes + kPfScaleBytes;
 constexpr int kPfRawBytes = kStageTq4;                        // 64 raw rows of 132 B
 constexpr int kPfDeqBase = kLutBytes;
 constexpr int kPfRawBase = kPfDeqBase + 2 * kPfDeqBytes;
-constexpr int kPfDummy = kPfRawBase + 2 * kPfRawBytes;        // 256 B that absorb the writes of scale bytes
-constexpr int kPfSmem = kPfDummy + 256;
+constexpr int kPfSmem = kPfRawBase + 2 * kPfRawBytes + 256;
 static_assert(kPfSmem <= 160 * 1024, "prefill LDS budget");
 static_assert(kPfWaves * 16 * 260 * 4 <= kPfSmem, "epilogue regions must fit");
 static_assert(kPfWaves * 16 * 264 * 2 <= 2 * kPfDeqBytes, "query staging must fit in the dequant buffers");
@@ -50,6 +49,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     const int b = lane >> 4;
     const warp34_kv_layer_layout& L = P.L;
     const warp34_attention_batch& B = P.B;
+    W34_TP(0);
 
     // ---- tile identification: blockIdx = (tile of the request, kv head x q subgroup, request) ----
     const int req = (int)blockIdx.z;
@@ -153,139 +153,154 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         for (int m = 0; m < 4; ++m)
             bq[h][m] = *reinterpret_cast<const h8*>(qbuf + n * kQStride + 128 * h + 32 * m + 8 * b);
 
-    // ---- loader: this thread's 16-byte piece(s) of a raw unit ----
-    // A unit is four runs of 16 rows (2112 B = 132 pieces): K rows 0-15, K rows 16-31, V rows
-    // 0-15, V rows 16-31; piece i of the unit is piece i % 132 of run i / 132.  Threads 0-15
-    // also carry pieces 512-527.
+    // ---- loader ----
+    // A unit is four runs of 16 rows (2112 B = 132 16-byte pieces): K rows 0-15, K rows 16-31,
+    // V rows 0-15, V rows 16-31.  Waves 2r and 2r+1 load pieces 0-127 of run r (one piece per
+    // lane, wave-uniform base); lanes 0-3 of wave 2r also carry the tail pieces 128-131.
     const uint8_t* k_base = reinterpret_cast<const uint8_t*>((uintptr_t)L.k_base) +
                             (size_t)kv_head * L.k_head_stride_bytes;
     const uint8_t* v_base = reinterpret_cast<const uint8_t*>((uintptr_t)L.v_base) +
                             (size_t)kv_head * L.v_head_stride_bytes;
     const int32_t* req_blocks = B.block_tables + (size_t)req * B.max_blocks_per_req;
-    int ld_run[2], ld_pc[2];
-    ld_run[0] = tid >= 396 ? 3 : tid >= 264 ? 2 : tid >= 132 ? 1 : 0;
-    ld_pc[0] = tid - 132 * ld_run[0];
-    ld_run[1] = 3;
-    ld_pc[1] = 116 + tid;  // only for tid < 16
-    const bool two = tid < 16;
-    int32_t pg_cur[2] = {-1, -1};
+    const int ld_run = wave >> 1;
+    const bool ld_is_v = ld_run >= 2;
+    const bool ld_tail = (wave & 1) == 0;  // wave-uniform
+    const uint8_t* ld_base = ld_is_v ? v_base : k_base;
+    const uint64_t ld_page_stride = ld_is_v ? L.v_page_stride_bytes : L.k_page_stride_bytes;
+    const uint64_t ld_tok_stride = ld_is_v ? L.v_token_stride_bytes : L.k_token_stride_bytes;
+    const uint32_t ld_lane_off = (uint32_t)((wave & 1) * 1024 + 16 * lane);
+    const uint32_t ld_commit0 = (uint32_t)(ld_run * kRunBytes) + ld_lane_off;
+    const uint32_t ld_commit1 = (uint32_t)(ld_run * kRunBytes + 2048 + 16 * (lane & 3));
     u4 pf[2];
-    // page ids of unit k (relative to u_first) for this thread's runs
-    auto load_pages = [&](int k, int32_t (&pg)[2]) {
-#pragma unroll
-        for (int x = 0; x < 2; ++x) {
-            pg[x] = -1;
-            if (x == 1 && !two) continue;
-            const int pos = (u_first + k) * kUnit + 16 * (ld_run[x] & 1);
-            const int slot = fast_div(pos, L.block_size);
-            // only groups that overlap the visible key range are fetched (entries of the block
-            // table beyond the request's pages are unspecified)
-            const bool live = k < n_units && pos <= hi_all && pos + 15 >= lo_all && slot < B.max_blocks_per_req;
-            if (live) pg[x] = req_blocks[slot];
-        }
+    // page id of unit k (relative to u_first) for this wave's run; -1 = nothing to fetch.
+    // Only groups that overlap the visible key range are fetched: block-table entries beyond
+    // the request's pages are unspecified.
+    auto load_page = [&](int k) -> int32_t {
+        const int pos = (u_first + k) * kUnit + 16 * (ld_run & 1);
+        const int slot = __builtin_amdgcn_readfirstlane(fast_div(pos, L.block_size));
+        const bool live = k < n_units && pos <= hi_all && pos + 15 >= lo_all && slot < B.max_blocks_per_req;
+        int32_t pg = -1;
+        if (live) pg = req_blocks[slot];
+        return pg;  // wave-uniform value in a vector register: made scalar where it is used, an iteration later
     };
-    auto issue_loads = [&](int k, const int32_t (&pg)[2]) {
-#pragma unroll
-        for (int x = 0; x < 2; ++x) {
-            if (x == 1 && !two) continue;
-            const int pos = (u_first + k) * kUnit + 16 * (ld_run[x] & 1);
-            const int slot = fast_div(pos, L.block_size);
-            const int in_page = pos - slot * L.block_size;
-            const bool is_v = ld_run[x] >= 2;
-            const uint8_t* base = is_v ? v_base : k_base;
-            size_t off = 0;  // missing page: rows of page 0, every one of them is masked
-            if (pg[x] >= 0)
-                off = (size_t)pg[x] * (is_v ? L.v_page_stride_bytes : L.k_page_stride_bytes) +
-                      (size_t)in_page * (is_v ? L.v_token_stride_bytes : L.k_token_stride_bytes);
-            pf[x] = *(global_cu4*)(base + off + 16 * ld_pc[x]);
-        }
+    auto issue_loads = [&](int k, int32_t pg) {
+        const int pos = (u_first + k) * kUnit + 16 * (ld_run & 1);
+        const int slot = __builtin_amdgcn_readfirstlane(fast_div(pos, L.block_size));
+        const int in_page = pos - slot * L.block_size;
+        size_t off = 0;  // missing page: rows of page 0, every one of them is masked
+        if (pg >= 0) off = (size_t)pg * ld_page_stride + (size_t)in_page * ld_tok_stride;
+        const uint8_t* src = ld_base + off;
+        pf[0] = *(global_cu4*)(src + ld_lane_off);
+        if (ld_tail) pf[1] = *(global_cu4*)(src + 2048 + 16 * (lane & 3));
     };
     auto commit_loads = [&](int buf) {
         uint8_t* raw = smem + kPfRawBase + buf * kPfRawBytes;
-        *reinterpret_cast<u4*>(raw + 16 * tid) = pf[0];
-        if (two) *reinterpret_cast<u4*>(raw + 16 * (512 + tid)) = pf[1];
+        *reinterpret_cast<u4*>(raw + ld_commit0) = pf[0];
+        if (ld_tail && lane < 4) *reinterpret_cast<u4*>(raw + ld_commit1) = pf[1];
     };
 
-    // ---- dequantiser: this thread's items ----
-    // K: dword idx of the 32 x 33 raw dwords (idx = tid, tid + 512, and tid + 1024 for tid < 32);
-    // row r = idx / 33, dword w = idx % 33.  Byte q of the dword is row byte 4 w + q: bytes
-    // 2..65 are code bytes 0..63 of the first half (elements 2 i, 2 i + 1), bytes 68..131 the
-    // second half; the others are scale bytes, their writes go to a dummy area.
+    // ---- dequantiser ----
+    // A raw row is 33 dwords; dwords 0 and 16 hold two scale bytes and two code bytes each.
+    // They are fused into one synthetic dword [code bytes 0,1 | code bytes 62,63], which leaves
+    // exactly 32 four-code-byte items per row:
+    //   item 0      : alignbit(dword 16, dword 0, 16)  -> elements 0..3 and 124..127
+    //   item j 1..15: dword j                          -> elements 8 j - 4 .. 8 j + 3
+    //   item j 16..31: dword j + 1                     -> elements 8 j .. 8 j + 7
+    // K: 32 rows x 32 items = two per thread (item idx = tid, tid + 512: row idx >> 5, j = idx & 31);
+    //    the four looked-up pairs are written as two 8-byte stores into the row-major fp16 tile.
+    // V: 16 token pairs x 32 items = one per thread (pair p = tid & 15, j = tid >> 4).  Tokens
+    //    2p, 2p+1 sit in key slots 8 b' + 4 s + {0,1} (+2 for odd p), s = p >> 3, b' = (p >> 1) & 3;
+    //    element d lives in V^T row d, 16-byte piece b' ^ ((d >> 1) & 3).  Lanes whose
+    //    (lane >> 4) is odd write the odd elements first so that a 32-lane write pass covers
+    //    32 banks.
     const uint32_t lut_lane = (uint32_t)lane << 2;
-    uint32_t k_src[3], k_dst[3][2];
-#pragma unroll
-    for (int it = 0; it < 3; ++it) {
-        const int idx = tid + 512 * it;
-        const int r = idx / 33;
-        const int w = idx - 33 * r;
-        k_src[it] = 4u * (uint32_t)idx;
-        const int d0 = r * kPfKStride + 16 * w - (w <= 16 ? 8 : 16);
-        k_dst[it][0] = (w == 0) ? (uint32_t)(kPfDummy + 8 * (tid & 15)) : (uint32_t)d0;
-        k_dst[it][1] = (w == 16) ? (uint32_t)(kPfDummy + 8 * (tid & 15)) : (uint32_t)(d0 + 8);
-    }
-    // V: item = (token pair p, dword w) with p = idx & 15, w = idx >> 4 (idx = tid, and
-    // tid + 512 for tid < 16).  Tokens 2p, 2p+1 sit in key slots 8 b' + 4 s + {0,1} (+2 for odd p)
-    // with s = p >> 3, b' = (p >> 1) & 3; element d lives at V^T row d, 16-byte piece
-    // b' ^ ((d >> 1) & 3).  Lanes whose (lane >> 4) is odd write the odd elements first so
-    // that the 32 lanes of a write pass cover 32 banks.
-    const int nibsel = (lane >> 4) & 1;
-    uint32_t v_src[2], v_dst[2][4];
+    auto item_src = [](int j, uint32_t (&src)[2], uint32_t& shift) {
+        // byte offsets of the two dwords inside the row, and the alignbit shift
+        if (j == 0) {
+            src[0] = 0;
+            src[1] = 64;
+            shift = 16;
+        } else {
+            const int w = j < 16 ? j : j + 1;
+            src[0] = src[1] = 4u * (uint32_t)w;
+            shift = 0;
+        }
+    };
+    uint32_t k_src[2][2], k_shift[2], k_dst[2][2];
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
         const int idx = tid + 512 * it;
-        const int p = idx & 15;
-        const int w = idx >> 4;
-        v_src[it] = (uint32_t)(kPfRawBytes / 2 + (2 * p) * kTq4RowBytes + 4 * w);
-        const int base_d = w <= 16 ? 8 * w - 4 : 8 * w - 8;
+        const int r = idx >> 5, j = idx & 31;
+        uint32_t src[2];
+        item_src(j, src, k_shift[it]);
+        k_src[it][0] = (uint32_t)(r * kTq4RowBytes) + src[0];
+        k_src[it][1] = (uint32_t)(r * kTq4RowBytes) + src[1];
+        const int d_lo = j == 0 ? 0 : j < 16 ? 8 * j - 4 : 8 * j;   // element of code byte 0
+        const int d_hi = j == 0 ? 124 : d_lo + 4;                    // element of code byte 2
+        k_dst[it][0] = (uint32_t)(r * kPfKStride + 2 * d_lo);
+        k_dst[it][1] = (uint32_t)(r * kPfKStride + 2 * d_hi);
+    }
+    const int nibsel = (lane >> 4) & 1;
+    uint32_t v_src[2], v_shift, v_dst[4];
+    {
+        const int p = tid & 15, j = tid >> 4;
+        uint32_t src[2];
+        item_src(j, src, v_shift);
+        v_src[0] = (uint32_t)(kPfRawBytes / 2 + (2 * p) * kTq4RowBytes) + src[0];
+        v_src[1] = (uint32_t)(kPfRawBytes / 2 + (2 * p) * kTq4RowBytes) + src[1];
         const int bp = (p >> 1) & 3, s = p >> 3;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const int d = base_d + 2 * q;  // even element of byte q
-            const bool valid = !((w == 0 && q < 2) || (w == 16 && q >= 2)) && w <= 32;
-            const int addr = kPfKBytes + d * 64 + 16 * (bp ^ ((d >> 1) & 3)) + 8 * s + 4 * (p & 1) + 64 * nibsel;
-            v_dst[it][q] = valid ? (uint32_t)addr : (uint32_t)(kPfDummy + 128 + 4 * (tid & 15));
+            const int d = j == 0 ? (q < 2 ? 2 * q : 120 + 2 * q) : (j < 16 ? 8 * j - 4 : 8 * j) + 2 * q;
+            v_dst[q] = (uint32_t)(kPfKBytes + d * 64 + 16 * (bp ^ ((d >> 1) & 3)) + 8 * s + 4 * (p & 1) + 64 * nibsel);
         }
     }
+    // ---- per-wave attention state ----
+    f4 o_acc[2][8];
+    float m_run = kNegBig, l_run = 0.f;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o_acc[h][j] = f4{0.f, 0.f, 0.f, 0.f};
+
     auto dequant_unit = [&](int rawbuf, int deqbuf) {
         const uint32_t raw = (uint32_t)(kPfRawBase + rawbuf * kPfRawBytes);
         const uint32_t deq = (uint32_t)(kPfDeqBase + deqbuf * kPfDeqBytes);
-        const uint32_t dummy_lo = (uint32_t)kPfDummy;
         // K
 #pragma unroll
-        for (int it = 0; it < 3; ++it) {
-            if (it == 2 && tid >= 32) continue;
-            const uint32_t word = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + k_src[it]));
+        for (int it = 0; it < 2; ++it) {
+            const uint32_t w0 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + k_src[it][0]));
+            const uint32_t w1 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + k_src[it][1]));
+            const uint32_t word = __builtin_amdgcn_alignbit(w1, w0, k_shift[it]);
             uint2 lo, hi;
             lo.x = lut_read(word, lut_lane, 0x0c0c0400u);
             lo.y = lut_read(word, lut_lane, 0x0c0c0500u);
             hi.x = lut_read(word, lut_lane, 0x0c0c0600u);
             hi.y = lut_read(word, lut_lane, 0x0c0c0700u);
-            const uint32_t a0 = k_dst[it][0] >= dummy_lo ? k_dst[it][0] : deq + k_dst[it][0];
-            const uint32_t a1 = k_dst[it][1] >= dummy_lo ? k_dst[it][1] : deq + k_dst[it][1];
-            *reinterpret_cast<uint2*>(smem + a0) = lo;
-            *reinterpret_cast<uint2*>(smem + a1) = hi;
+            *reinterpret_cast<uint2*>(smem + deq + k_dst[it][0]) = lo;
+            *reinterpret_cast<uint2*>(smem + deq + k_dst[it][1]) = hi;
         }
         // V
-#pragma unroll
-        for (int it = 0; it < 2; ++it) {
-            if (it == 1 && !two) continue;
-            const uint32_t wa = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[it]));
-            const uint32_t wb = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[it] + kTq4RowBytes));
+        {
+            const uint32_t a0 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[0]));
+            const uint32_t a1 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[1]));
+            const uint32_t b0 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[0] + kTq4RowBytes));
+            const uint32_t b1 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[1] + kTq4RowBytes));
+            const uint32_t wa = __builtin_amdgcn_alignbit(a1, a0, v_shift);
+            const uint32_t wb = __builtin_amdgcn_alignbit(b1, b0, v_shift);
             // byte q of ev / od = (even / odd element of token 2p) | (same of token 2p+1) << 4
             const uint32_t ev = (wa & 0x0F0F0F0Fu) | ((wb << 4) & 0xF0F0F0F0u);
             const uint32_t od = ((wa >> 4) & 0x0F0F0F0Fu) | (wb & 0xF0F0F0F0u);
-            const uint32_t first = nibsel ? od : ev;   // element parity nibsel, written at v_dst
-            const uint32_t second = nibsel ? ev : od;  // the other parity, 64 bytes away
+            const uint32_t first = nibsel ? od : ev;   // elements of parity nibsel, stored at v_dst
+            const uint32_t second = nibsel ? ev : od;  // the other parity, one V^T row (64 B) away
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const uint32_t sel = 0x0c0c0400u + ((uint32_t)q << 8);
                 const uint32_t x0 = lut_read(first, lut_lane, sel);
                 const uint32_t x1 = lut_read(second, lut_lane, sel);
-                const bool dm = v_dst[it][q] >= dummy_lo;
-                const uint32_t a0 = dm ? v_dst[it][q] : deq + v_dst[it][q];
-                const uint32_t a1 = dm ? v_dst[it][q] : (deq + v_dst[it][q]) ^ 64u;
-                *reinterpret_cast<uint32_t*>(smem + a0) = x0;
-                *reinterpret_cast<uint32_t*>(smem + a1) = x1;
+                const uint32_t addr = deq + v_dst[q];
+                *reinterpret_cast<uint32_t*>(smem + addr) = x0;
+                *reinterpret_cast<uint32_t*>(smem + (addr ^ 64u)) = x1;
             }
         }
         // scales: thread x * 32 + r (x = 0: K d0, 1: K d1, 2: V d0, 3: V d1) of waves 0 and 1
@@ -297,14 +312,6 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
                 (float)__builtin_bit_cast(_Float16, bits);
         }
     };
-
-    // ---- per-wave attention state ----
-    f4 o_acc[2][8];
-    float m_run = kNegBig, l_run = 0.f;
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) o_acc[h][j] = f4{0.f, 0.f, 0.f, 0.f};
 
     auto compute_unit = [&](int deqbuf, int t0, const bool MASKED) {
         const uint8_t* kb = smem + kPfDeqBase + deqbuf * kPfDeqBytes;
@@ -390,24 +397,41 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
 
     // ---- pipeline ----
     __syncthreads();  // table complete; query staging (aliases the dequant buffers) consumed
-    int32_t pg_next[2];
-    load_pages(0, pg_cur);
-    load_pages(1, pg_next);
-    if (n_units > 0) issue_loads(0, pg_cur);
+    const int32_t pg_first = __builtin_amdgcn_readfirstlane(load_page(0));
+    int32_t pg_next = load_page(1);
+    if (n_units > 0) issue_loads(0, pg_first);
+    W34_TP(1);
     for (int it = -2; it < n_units; ++it) {
         // commit unit it + 2 (loaded during the previous iteration), then start unit it + 3
         if (it + 2 < n_units) commit_loads((it + 2) & 1);
-        pg_cur[0] = pg_next[0];
-        pg_cur[1] = pg_next[1];
-        if (it + 3 < n_units) issue_loads(it + 3, pg_cur);
-        load_pages(it + 4, pg_next);
+#ifdef W34_TRACE
+        if (it >= 8 && it < 16) W34_TP(4 + 5 * (it - 8));
+#endif
+        // The page id of unit it + 4 is requested BEFORE the key loads of unit it + 3: a
+        // write to its register after them would have to wait for all of them to return.
+        const int32_t pg_s = __builtin_amdgcn_readfirstlane(pg_next);
+        pg_next = load_page(it + 4);
+        if (it + 3 < n_units) issue_loads(it + 3, pg_s);
+#ifdef W34_TRACE
+        if (it >= 8 && it < 16) W34_TP(4 + 5 * (it - 8) + 1);
+#endif
         if (it + 1 >= 0 && it + 1 < n_units) dequant_unit((it + 1) & 1, (it + 1) & 1);
+#ifdef W34_TRACE
+        if (it >= 8 && it < 16) W34_TP(4 + 5 * (it - 8) + 2);
+#endif
         if (it >= 0) {
             const int t0 = (u_first + it) * kUnit;
             compute_unit(it & 1, t0, !(t0 >= i_lo && t0 + kUnit - 1 <= i_hi));
         }
+#ifdef W34_TRACE
+        if (it >= 8 && it < 16) W34_TP(4 + 5 * (it - 8) + 3);
+#endif
         __syncthreads();
+#ifdef W34_TRACE
+        if (it >= 8 && it < 16) W34_TP(4 + 5 * (it - 8) + 4);
+#endif
     }
+    W34_TP(50);
 
     // ---- epilogue: normalise, transpose through LDS, rotate back, store ----
     l_run = sum_over_rows(l_run);
