@@ -33,7 +33,11 @@ WORKLOADS = {
     "bf16_decode_b1_ctx32768": ("bf16", [32768], 0),
     # 8 sequences, 16 384-token TQ4 prefix + 2 048-token bf16 chunk each: append + causal attention
     "tq4_prefill_8x2048_ctx16384": ("tq4", [18432] * 8, 0),
+    # 16 sequences of 262 144 tokens that share the pages of a 200 000-token prefix; 4 query tokens each
+    "tq4_verify_16x4_ctx262144_shared200k": ("tq4", [262144] * 16, 0),
 }
+SHARED_PREFIX = {"tq4_verify_16x4_ctx262144_shared200k": 200000}
+VERIFY_Q = {"tq4_verify_16x4_ctx262144_shared200k": 4}
 PREFILL_CHUNK = 2048
 
 
@@ -67,7 +71,7 @@ def build_workload(name, seed=0):
 class Layer:
     """One layer's KV pool on the device, filled through the append kernel."""
 
-    def __init__(self, torch, lib, ffi, fmt, ctx, pool_pages, seed):
+    def __init__(self, torch, lib, ffi, fmt, ctx, pool_pages, seed, shared_prefix=0):
         dev = "cuda:0"
         self.tok, self.head = ROW_BYTES[fmt], BLOCK * ROW_BYTES[fmt]
         self.page = KV_HEADS * self.head
@@ -85,9 +89,15 @@ class Layer:
         mb = max(pages_per)
         bt = torch.zeros((len(ctx), mb), dtype=torch.int32, device=dev)
         at = 0
+        shared_pages = shared_prefix // BLOCK  # whole pages, owned by request 0
         for r, n in enumerate(pages_per):
-            bt[r, :n] = perm[at:at + n]
-            at += n
+            if r > 0 and shared_pages:
+                bt[r, :shared_pages] = bt[0, :shared_pages]
+                bt[r, shared_pages:n] = perm[at:at + n - shared_pages]
+                at += n - shared_pages
+            else:
+                bt[r, :n] = perm[at:at + n]
+                at += n
         self.block_tables = bt
         self.max_blocks = mb
         # outlier channels: 3 of 256 per kv head scaled x20
@@ -101,7 +111,8 @@ class Layer:
         self.tail_k, self.tail_v, self.tail_slots = [], [], []
         for r, c in enumerate(ctx):
             c = int(c)
-            for t0 in range(0, c, chunk):
+            first = shared_pages * BLOCK if r > 0 else 0  # shared pages were filled by request 0
+            for t0 in range(first, c, chunk):
                 n = min(chunk, c - t0)
                 kk = (torch.randn((n, KV_HEADS, HEAD_DIM), generator=g, device=dev) * gain).to(torch.bfloat16)
                 vv = (torch.randn((n, KV_HEADS, HEAD_DIM), generator=g, device=dev) * gain).to(torch.bfloat16)
@@ -258,23 +269,28 @@ def main():
     total_tokens_kv = int(ctx.sum())
     row_bytes = ROW_BYTES[fmt]
     kv_bytes = total_tokens_kv * KV_HEADS * 2 * row_bytes  # algorithmic bytes per step (K + V rows)
+    shared = 0 if os.environ.get("W34_NOSHARE") else SHARED_PREFIX.get(args.workload, 0)
     pool_pages = max(sum((int(c) + BLOCK - 1) // BLOCK for c in ctx) + 16, pool_tokens // BLOCK)
+    pool_pages -= (len(ctx) - 1) * (shared // BLOCK)
+    if shared:  # unique bytes: the prefix once, every private suffix once
+        kv_bytes = (shared + sum(int(c) - shared for c in ctx)) * KV_HEADS * 2 * row_bytes
     layer_bytes = 2 * pool_pages * KV_HEADS * BLOCK * row_bytes
     n_layers = args.layers or max(2, -(-(640 << 20) // layer_bytes))
-    layers = [Layer(torch, lib, ffi, fmt, ctx, pool_pages, s) for s in range(n_layers)]
+    layers = [Layer(torch, lib, ffi, fmt, ctx, pool_pages, s, shared) for s in range(n_layers)]
 
     if args.workload.startswith("tq4_prefill"):
         run_prefill(args, torch, lib, ffi, layers, ctx, n_layers, pool_pages)
         return
 
     R = len(ctx)
+    ql = int(os.environ.get("W34_QL", VERIFY_Q.get(args.workload, 1)))  # query tokens per request (1 = decode)
     g = torch.Generator(device=dev)
     g.manual_seed(7)
-    q = torch.randn((R, Q_HEADS, HEAD_DIM), generator=g, device=dev).to(torch.bfloat16)
+    q = torch.randn((R * ql, Q_HEADS, HEAD_DIM), generator=g, device=dev).to(torch.bfloat16)
     out = torch.zeros_like(q)
-    qsl = torch.arange(0, R + 1, dtype=torch.int32, device=dev)
+    qsl = (torch.arange(0, R + 1, dtype=torch.int32, device=dev) * ql).to(torch.int32)
     seq = torch.tensor(ctx, dtype=torch.int32, device=dev)
-    ctxb = seq - 1
+    ctxb = (seq - ql).to(torch.int32)
     scratch_bytes = 32 << 20
     scratch = torch.zeros(scratch_bytes, dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
@@ -283,7 +299,7 @@ def main():
     for L in layers:
         batches.append(ffi.Warp34AttentionBatch(
             qsl.data_ptr(), ctxb.data_ptr(), seq.data_ptr(), L.block_tables.data_ptr(), None, None, None,
-            R, R, L.max_blocks, 1, int(ctx.max()), 0, 0, 1.0 / 16.0, 0))
+            R, R * ql, L.max_blocks, ql, int(ctx.max()), 0, 0, 1.0 / 16.0, 0))
 
     def step(i):
         L = layers[i % n_layers]
@@ -326,7 +342,7 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": args.workload,
-            "requests": R,
+            "requests": R, "query_tokens_per_request": ql, "shared_prefix_tokens": shared,
             "context_tokens_total": total_tokens_kv,
             "q_heads": Q_HEADS, "kv_heads": KV_HEADS, "head_dim": HEAD_DIM, "page_tokens": BLOCK,
             "kv_format": "tq4+wht256" if fmt == "tq4" else "bf16", "kv_pools_cycled": n_layers,

@@ -272,3 +272,49 @@ def test_prefill_tile_kernel_masks_and_page_permutation():
                        scale=G.channel_scale(v, DT_F16, hb, 8)[~dead])
         outs.append(got)
     assert outs[0].tobytes() == outs[1].tobytes()
+
+
+def test_verify_with_shared_prefix_pages():
+    """MTP-style verify: three requests share the block-table entries of a 640-token prefix
+    (whole pages, as the prefix cache hands them out), each has a private suffix and verifies
+    4 query tokens with causal masking among them."""
+    import gpu_harness as G
+
+    bs, prefix, suffixes, ql, q_heads, kv_heads = 64, 640, [130, 71, 200], 4, 16, 2
+    n_prefix_pages = prefix // bs
+    priv_pages = [(prefix + s + bs - 1) // bs - n_prefix_pages for s in suffixes]
+    num_pages = n_prefix_pages + sum(priv_pages) + 2
+    perm = oracle.permutation(num_pages, 9)
+    pool = oracle.HostPool(num_pages, kv_heads, 256, bs, FMT_TQ4, oracle.XF_WHT256)
+    mb = n_prefix_pages + max(priv_pages)
+    bt = np.zeros((len(suffixes), mb), dtype=np.int32)
+    at = n_prefix_pages
+    for r, pp in enumerate(priv_pages):
+        bt[r, :n_prefix_pages] = perm[:n_prefix_pages]
+        bt[r, n_prefix_pages:n_prefix_pages + pp] = perm[at:at + pp]
+        at += pp
+    # the prefix is appended once (through request 0's table), every suffix separately
+    k = oracle.fill_kv_rows(prefix, kv_heads, 256, 301, DT_BF16, 3)
+    v = oracle.fill_kv_rows(prefix, kv_heads, 256, 302, DT_BF16, 3)
+    wb = oracle.HostBatch([0, prefix], [prefix], bt[:1], context_lens_before=[0],
+                          write_slot_mapping=oracle.slot_mapping(bt[0], 0, prefix, bs))
+    oracle.kv_cache_write(pool, wb, k, v, DT_BF16)
+    v_rows = []
+    for r, s in enumerate(suffixes):
+        ks = oracle.fill_kv_rows(s, kv_heads, 256, 310 + r, DT_BF16, 3)
+        vs = oracle.fill_kv_rows(s, kv_heads, 256, 320 + r, DT_BF16, 3)
+        v_rows += [v, vs]
+        wb = oracle.HostBatch([0, s], [prefix + s], bt[r:r + 1], context_lens_before=[prefix],
+                              write_slot_mapping=oracle.slot_mapping(bt[r], prefix, s, bs))
+        oracle.kv_cache_write(pool, wb, ks, vs, DT_BF16)
+    seq = [prefix + s for s in suffixes]
+    aq = [0, ql, 2 * ql, 3 * ql]
+    q = oracle.fill_normal(3 * ql * q_heads * 256, 330, DT_BF16).reshape(3 * ql, q_heads, 256)
+    hb = oracle.HostBatch(aq, seq, bt, context_lens_before=[s - ql for s in seq])
+    want = oracle.paged_attention(pool, hb, q, DT_BF16, q_heads, n_threads=4)
+    dpool = _dev_pool(pool)
+    for scratch in (0, SCRATCH):
+        rc, got, _ = G.dev_attention(dpool, hb, q, DT_BF16, q_heads, scratch_bytes=scratch)
+        assert rc == 0
+        G.assert_close(got, DT_BF16, want, what="shared prefix, scratch %d" % scratch,
+                       scale=G.channel_scale(np.concatenate(v_rows), DT_BF16, hb, q_heads))

@@ -38,6 +38,7 @@
 //
 // MFMA use: v_mfma_f32_16x16x32_f16.  A = K rows (QK) or V^T (PV) so that every lane owns one
 // query column: softmax state and the O rescale are per-lane scalars.
+#include <cstdlib>
 #include <type_traits>
 
 #include "kv_common.h"
@@ -78,7 +79,7 @@ constexpr float kLutInvGain = 1.0f / kLutGain;
 __device__ unsigned long long g_trace[64 * 64];
 #define W34_TP(slot)                                                                   \
     do {                                                                               \
-        if (lane == 0 && (blockIdx.x == 0 || blockIdx.x == 77) && blockIdx.y == 0) {  \
+        if (lane == 0 && (blockIdx.x == 0 || blockIdx.x == 77) && blockIdx.y == 0 && blockIdx.z == 0) {  \
             g_trace[((blockIdx.x ? 8 : 0) + wave) * 64 + (slot)] = __builtin_readcyclecounter(); \
             if ((slot) == 0) g_trace[((blockIdx.x ? 8 : 0) + wave) * 64 + 63] = wall_clock64(); \
             if ((slot) == 40) g_trace[((blockIdx.x ? 8 : 0) + wave) * 64 + 62] = wall_clock64(); \
@@ -102,6 +103,7 @@ struct AttnParams {
     int tok_tile;     // query tokens per tile
     int max_chunks;   // cap on chunks per tile (1 = no split, scratch untouched)
     int min_upc;      // minimum units per chunk
+    int tiles_by_request;  // 1: blockIdx.z is a request (no request has more than one tile)
 };
 
 // token of k-slot (s, b, i) inside a unit: spreads the four 4-row groups of an MFMA over LDS
@@ -278,79 +280,113 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
     const warp34_kv_layer_layout& L = P.L;
     const warp34_attention_batch& B = P.B;
 
-    // ---- tile identification (wave-uniform, scalar loads) -------------------------------------
-    const int tok0 = (int)blockIdx.z;
+    // ---- tile identification ---------------------------------------------------------------------
+    // blockIdx.z counts TILES (groups of tok_tile consecutive query tokens of one request), so
+    // every workgroup that is launched has work.  When no request can have more than one tile
+    // (max_q_len <= tok_tile, e.g. decode) tile z is request z; otherwise the tile is located
+    // with a prefix sum over the requests' tile counts.
+    const int tile_z = (int)blockIdx.z;
     const int kv_sub = (int)blockIdx.y;
     const int kv_head = fast_div(kv_sub, P.q_subgroups);
     const int q_head_base = kv_head * P.gqa + (kv_sub - kv_head * P.q_subgroups) * P.q_group;
     const int chunk = (int)blockIdx.x;
 
     W34_TP(0);
-    if (tok0 >= B.total_tokens) return;
 
     // Work that depends on nothing goes first so that it overlaps the request lookup below:
-    // the raw query rows of this wave's columns (validity is decided later) and the table.
+    // the raw query rows of this wave's columns and the table.  The first token of the tile is
+    // guessed (exact when every request has a whole number of tiles); a wrong guess is
+    // corrected after the lookup.
+    const int tok_guess = min(P.tiles_by_request ? tile_z : tile_z * P.tok_tile, B.total_tokens - 1);
     constexpr int kColsPerWave = (16 * NT + kWaves - 1) / kWaves;
     uint2 q_raw[kColsPerWave];
+    auto load_q = [&](int tokbase) {
 #pragma unroll
-    for (int c = 0; c < kColsPerWave; ++c) {
-        const int col = wave + c * kWaves;
-        const int t = fast_div(col, P.q_group);
-        const int a = col - t * P.q_group;
-        q_raw[c] = uint2{0u, 0u};
-        if (col < 16 * NT && tok0 + t < B.total_tokens) {
-            const uint16_t* qrow =
-                P.q + ((size_t)(tok0 + t) * P.num_q_heads + (size_t)(q_head_base + a)) * kHeadDim;
-            q_raw[c] = *reinterpret_cast<const uint2*>(qrow + 4 * lane);
+        for (int c = 0; c < kColsPerWave; ++c) {
+            const int col = wave + c * kWaves;
+            const int t = fast_div(col, P.q_group);
+            const int a = col - t * P.q_group;
+            q_raw[c] = uint2{0u, 0u};
+            if (col < 16 * NT && tokbase + t < B.total_tokens) {
+                const uint16_t* qrow =
+                    P.q + ((size_t)(tokbase + t) * P.num_q_heads + (size_t)(q_head_base + a)) * kHeadDim;
+                q_raw[c] = *reinterpret_cast<const uint2*>(qrow + 4 * lane);
+            }
         }
-    }
-    // Request lookup in one memory round trip: lane l examines request base+l (the first
-    // matching request wins, as in the linear scan of op_kv_cache.cu:385-398) and carries that
-    // request's lengths, which are then broadcast with readlane.  Every token of the tile
-    // belongs to this request, so its key ranges follow from two scalars (op_kv_cache.cu:406-424).
-    // Speculative block-table load, in flight together with the request lookup: it assumes
-    // that token t belongs to request t (a decode batch) and that the request's length is the
-    // host's bound max_seq_len.  When either guess is wrong the ids are fetched again below,
-    // so the guess changes the latency only, never the result.
-    const int spec_req = min(tok0, B.num_reqs - 1);
-    int spec_slot_base = -1, spec_vec = -1;
-    if (B.sliding_window <= 0 && B.max_seq_len > 0 && spec_req >= 0) {
-        const ChunkGeom sg = chunk_geom(0, B.max_seq_len - 1, P.max_chunks, P.min_upc);
-        spec_slot_base = fast_div((sg.u_first + chunk * sg.upc) * kUnit, L.block_size);
-        const int slot = spec_slot_base + lane;
-        if (slot < B.max_blocks_per_req)
-            spec_vec = B.block_tables[(size_t)spec_req * B.max_blocks_per_req + slot];
-    }
-    bool req_hit = false;
-    int req = -1, rq_start = 0, rq_end = 0, seq_after = 0, ctx_before = 0;
-    for (int base = 0; base < B.num_reqs && !req_hit; base += 64) {
-        const int r = base + lane;
-        const bool inb = r < B.num_reqs;
-        const int lo = inb ? B.query_start_loc[r] : 0x7fffffff;
-        const int hi = inb ? B.query_start_loc[r + 1] : -0x7fffffff;
-        const int sa = inb ? B.seq_lens_after[r] : 0;
-        const int cb = (inb && B.context_lens_before != nullptr) ? B.context_lens_before[r] : 0;
-        const int rm = (inb && B.valid_req_mask != nullptr) ? (int)B.valid_req_mask[r] : 1;
-        const unsigned long long hits = __ballot(inb && tok0 >= lo && tok0 < hi);
-        if (hits != 0ull) {
-            const int src = __builtin_ctzll(hits);
-            req = base + src;
-            rq_start = __builtin_amdgcn_readlane(lo, src);
-            rq_end = __builtin_amdgcn_readlane(hi, src);
-            seq_after = __builtin_amdgcn_readlane(sa, src);
-            ctx_before = B.context_lens_before != nullptr ? __builtin_amdgcn_readlane(cb, src)
-                                                          : seq_after - (rq_end - rq_start);
-            req_hit = __builtin_amdgcn_readlane(rm, src) != 0;
-            if (!req_hit) break;  // masked request
-        }
-    }
-    // per-token validity of this lane's columns (independent of the request lookup)
+    };
+    load_q(tok_guess);
+    // per-token validity of this lane's columns
     bool tok_ok[NT];
+    auto load_tok_ok = [&](int tokbase) {
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        const int tok = tok0 + fast_div(nt * 16 + n, P.q_group);
-        tok_ok[nt] = tok < B.total_tokens &&
-                     (B.valid_token_mask == nullptr || B.valid_token_mask[min(tok, B.total_tokens - 1)] != 0);
+        for (int nt = 0; nt < NT; ++nt) {
+            const int tok = tokbase + fast_div(nt * 16 + n, P.q_group);
+            tok_ok[nt] = tok < B.total_tokens &&
+                         (B.valid_token_mask == nullptr || B.valid_token_mask[min(tok, B.total_tokens - 1)] != 0);
+        }
+    };
+    load_tok_ok(tok_guess);
+
+    bool req_hit = false;
+    int req = -1, rq_start = 0, rq_end = 0, seq_after = 0, ctx_before = 0, tile_in_req = 0;
+    int spec_slot_base = -1, spec_vec = -1;
+    int a_lo = 0, a_hi = 0, a_sa = 0, a_cb = 0, a_rm = 0;
+    if (P.tiles_by_request) {
+        req = tile_z;  // < num_reqs by the launch geometry
+        // Speculative block-table load, in flight together with the request's lengths: it
+        // assumes that the request's length is the host's bound max_seq_len.  When the guess is
+        // wrong the ids are fetched again below, so it changes the latency only, never the result.
+        if (B.sliding_window <= 0 && B.max_seq_len > 0) {
+            const ChunkGeom sg = chunk_geom(0, B.max_seq_len - 1, P.max_chunks, P.min_upc);
+            spec_slot_base = fast_div((sg.u_first + chunk * sg.upc) * kUnit, L.block_size);
+            const int slot = spec_slot_base + lane;
+            if (slot < B.max_blocks_per_req)
+                spec_vec = B.block_tables[(size_t)req * B.max_blocks_per_req + slot];
+        }
+        // one vector load per array (all lanes the same address), no scalar-cache round trip;
+        // the values are made scalar after the table has been built, so that the build overlaps
+        // the round trip
+        a_lo = B.query_start_loc[req];
+        a_hi = B.query_start_loc[req + 1];
+        a_sa = B.seq_lens_after[req];
+        a_cb = B.context_lens_before != nullptr ? B.context_lens_before[req] : 0;
+        a_rm = B.valid_req_mask != nullptr ? (int)B.valid_req_mask[req] : 1;
+    } else {
+        // lane l examines request base + l; an inclusive prefix sum of the tile counts over the
+        // lanes locates the request that owns tile z (requests are disjoint, ascending ranges
+        // of tokens: op_kv_cache.cu:385-398)
+        int tiles_before = 0;
+        for (int base = 0; base < B.num_reqs; base += 64) {
+            const int r = base + lane;
+            const bool inb = r < B.num_reqs;
+            const int lo = inb ? B.query_start_loc[r] : 0;
+            const int hi = inb ? B.query_start_loc[r + 1] : 0;
+            const int sa = inb ? B.seq_lens_after[r] : 0;
+            const int cb = (inb && B.context_lens_before != nullptr) ? B.context_lens_before[r] : 0;
+            const int rm = (inb && B.valid_req_mask != nullptr) ? (int)B.valid_req_mask[r] : 1;
+            const int cnt = hi > lo ? fast_div(hi - lo + P.tok_tile - 1, P.tok_tile) : 0;
+            int incl = cnt;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const int up = __shfl_up(incl, off, 64);
+                if (lane >= off) incl += up;
+            }
+            const int first = tiles_before + incl - cnt;
+            const unsigned long long hits = __ballot(cnt > 0 && tile_z >= first && tile_z < first + cnt);
+            if (hits != 0ull) {
+                const int src = __builtin_ctzll(hits);
+                req = base + src;
+                rq_start = __builtin_amdgcn_readlane(lo, src);
+                rq_end = __builtin_amdgcn_readlane(hi, src);
+                seq_after = __builtin_amdgcn_readlane(sa, src);
+                ctx_before = B.context_lens_before != nullptr ? __builtin_amdgcn_readlane(cb, src)
+                                                              : seq_after - (rq_end - rq_start);
+                tile_in_req = tile_z - __builtin_amdgcn_readlane(first, src);
+                req_hit = __builtin_amdgcn_readlane(rm, src) != 0;
+                break;
+            }
+            tiles_before += __builtin_amdgcn_readlane(incl, 63);
+        }
     }
     {
         // entry e = (gain*centroid[e & 15], gain*centroid[e >> 4]) as packed fp16, 64 copies
@@ -362,6 +398,21 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
         u4* dst = reinterpret_cast<u4*>(smem + e * 256 + (tid % kThreadsPerEntry) * kBytesPerThread);
 #pragma unroll
         for (int k = 0; k < kBytesPerThread / 16; ++k) dst[k] = vv;
+    }
+
+    if (P.tiles_by_request) {
+        rq_start = __builtin_amdgcn_readfirstlane(a_lo);
+        rq_end = __builtin_amdgcn_readfirstlane(a_hi);
+        seq_after = __builtin_amdgcn_readfirstlane(a_sa);
+        ctx_before = B.context_lens_before != nullptr ? __builtin_amdgcn_readfirstlane(a_cb)
+                                                      : seq_after - (rq_end - rq_start);
+        req_hit = __builtin_amdgcn_readfirstlane(a_rm) != 0 && rq_end > rq_start;
+    }
+    if (!req_hit) return;  // no such tile, empty or masked request: outputs untouched
+    const int tok0 = rq_start + tile_in_req * P.tok_tile;
+    if (tok0 != tok_guess) {  // wave-uniform, rare
+        load_q(tok0);
+        load_tok_ok(tok0);
     }
 
     // Rotate the query rows now (dead columns are zeroed when they are stored below): the
@@ -379,8 +430,6 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
     }
 
     W34_TP(47);
-    if (!req_hit) return;  // no owning request (or masked request): outputs untouched
-    if ((tok0 - rq_start) - fast_div(tok0 - rq_start, P.tok_tile) * P.tok_tile != 0) return;  // not a tile leader
     int tile_tokens = rq_end - tok0;
     if (tile_tokens > P.tok_tile) tile_tokens = P.tok_tile;
 
@@ -414,12 +463,28 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
         }
         ok_mask[nt] = (uint32_t)(__ballot(ok) & 0xFFFFull);
     }
+    if (B.valid_token_mask == nullptr && B.sliding_window <= 0) {
+        // Common case, no cross-lane traffic: every token of the tile is live, the ranges start
+        // at 0 and their ends grow with the token, so the union is the last token's range and
+        // the intersection the first one's.
+        const int q_off0 = tok0 - rq_start;
+        const bool window = B.mask_mode == WARP34_ATTN_MASK_NONCAUSAL_WINDOW;
+        int hi_first = window ? seq_after - 1 : ctx_before + q_off0;
+        int hi_last = window ? seq_after - 1 : ctx_before + q_off0 + tile_tokens - 1;
+        if (hi_first >= seq_after) hi_first = seq_after - 1;
+        if (hi_last >= seq_after) hi_last = seq_after - 1;
+        u_lo = 0;
+        u_hi = hi_last >= 0 ? hi_last : -1;
+        i_lo = 0;
+        i_hi = hi_first;
+    } else {
 #pragma unroll
-    for (int off = 1; off < 16; off <<= 1) {
-        u_lo = min(u_lo, __shfl_xor(u_lo, off, 64));
-        u_hi = max(u_hi, __shfl_xor(u_hi, off, 64));
-        i_lo = max(i_lo, __shfl_xor(i_lo, off, 64));
-        i_hi = min(i_hi, __shfl_xor(i_hi, off, 64));
+        for (int off = 1; off < 16; off <<= 1) {
+            u_lo = min(u_lo, __shfl_xor(u_lo, off, 64));
+            u_hi = max(u_hi, __shfl_xor(u_hi, off, 64));
+            i_lo = max(i_lo, __shfl_xor(i_lo, off, 64));
+            i_hi = min(i_hi, __shfl_xor(i_hi, off, 64));
+        }
     }
     {
         uint32_t any = 0;
@@ -508,7 +573,7 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
 
     // first unit's data goes in flight before the rest of the prologue
     int unit = cu_first + wave;
-    if (req == spec_req && slot_base == spec_slot_base) {
+    if (slot_base == spec_slot_base) {
         page_vec = spec_vec;
     } else {
         load_page_vec();
@@ -1025,6 +1090,66 @@ __global__ __launch_bounds__(1024) void split_merge_kernel(const AttnParams P, f
     *reinterpret_cast<uint2*>(P.out + (size_t)row * kHeadDim + 4 * lane) = ob;
 }
 
+// Tile lookup shared by the kernels that do not split it around other work (see the TQ4
+// decode kernel for the scheme): blockIdx.z counts tiles; request z when no request can have
+// two tiles, a prefix sum over the requests' tile counts otherwise.
+struct TileInfo {
+    bool hit;
+    int req, rq_start, rq_end, seq_after, ctx_before, tile_in_req;
+};
+__device__ __forceinline__ TileInfo locate_tile(const AttnParams& P, int tile_z, int lane) {
+    const warp34_attention_batch& B = P.B;
+    TileInfo t{false, -1, 0, 0, 0, 0, 0};
+    if (P.tiles_by_request) {
+        t.req = tile_z;
+        const int lo = B.query_start_loc[tile_z];
+        const int hi = B.query_start_loc[tile_z + 1];
+        const int sa = B.seq_lens_after[tile_z];
+        const int cb = B.context_lens_before != nullptr ? B.context_lens_before[tile_z] : 0;
+        const int rm = B.valid_req_mask != nullptr ? (int)B.valid_req_mask[tile_z] : 1;
+        t.rq_start = __builtin_amdgcn_readfirstlane(lo);
+        t.rq_end = __builtin_amdgcn_readfirstlane(hi);
+        t.seq_after = __builtin_amdgcn_readfirstlane(sa);
+        t.ctx_before = B.context_lens_before != nullptr ? __builtin_amdgcn_readfirstlane(cb)
+                                                        : t.seq_after - (t.rq_end - t.rq_start);
+        t.hit = __builtin_amdgcn_readfirstlane(rm) != 0 && t.rq_end > t.rq_start;
+        return t;
+    }
+    int tiles_before = 0;
+    for (int base = 0; base < B.num_reqs; base += 64) {
+        const int r = base + lane;
+        const bool inb = r < B.num_reqs;
+        const int lo = inb ? B.query_start_loc[r] : 0;
+        const int hi = inb ? B.query_start_loc[r + 1] : 0;
+        const int sa = inb ? B.seq_lens_after[r] : 0;
+        const int cb = (inb && B.context_lens_before != nullptr) ? B.context_lens_before[r] : 0;
+        const int rm = (inb && B.valid_req_mask != nullptr) ? (int)B.valid_req_mask[r] : 1;
+        const int cnt = hi > lo ? fast_div(hi - lo + P.tok_tile - 1, P.tok_tile) : 0;
+        int incl = cnt;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int up = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += up;
+        }
+        const int first = tiles_before + incl - cnt;
+        const unsigned long long hits = __ballot(cnt > 0 && tile_z >= first && tile_z < first + cnt);
+        if (hits != 0ull) {
+            const int src = __builtin_ctzll(hits);
+            t.req = base + src;
+            t.rq_start = __builtin_amdgcn_readlane(lo, src);
+            t.rq_end = __builtin_amdgcn_readlane(hi, src);
+            t.seq_after = __builtin_amdgcn_readlane(sa, src);
+            t.ctx_before = B.context_lens_before != nullptr ? __builtin_amdgcn_readlane(cb, src)
+                                                            : t.seq_after - (t.rq_end - t.rq_start);
+            t.tile_in_req = tile_z - __builtin_amdgcn_readlane(first, src);
+            t.hit = __builtin_amdgcn_readlane(rm, src) != 0;
+            return t;
+        }
+        tiles_before += __builtin_amdgcn_readlane(incl, 63);
+    }
+    return t;
+}
+
 }  // namespace w34
 
 #include "paged_attn_kv16.h"
@@ -1095,8 +1220,10 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     }
     P.q_group = q_group;
     P.q_subgroups = P.gqa / q_group;
-    // two N tiles when a request brings enough query rows to fill them
-    const int nt = (batch->max_q_len * q_group > 16) ? 2 : 1;
+    // One N tile (16 query columns) per workgroup, also for verify batches: the two-tile variant
+    // (4 waves, 32 columns) halves the key reads but runs at half the occupancy and measured
+    // slower (2.04 ms against 1.64 ms on 16 requests x 4 query tokens at 262 144 keys).
+    const int nt = 1;
     P.tok_tile = (16 * nt) / q_group;
     if (P.tok_tile < 1) P.tok_tile = 1;
     P.min_upc = kMinUnitsPerChunk;
@@ -1116,19 +1243,16 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
         const int bound = (units + P.min_upc - 1) / P.min_upc;
         if (bound < grid_x) grid_x = bound < 1 ? 1 : bound;
     }
-    const dim3 grid((unsigned)grid_x, (unsigned)(layout->local_kv_heads * P.q_subgroups),
-                    (unsigned)batch->total_tokens);
+    // grid.z: tiles.  One per request when no request can have two; otherwise the upper bound
+    // sum_r ceil(q_r / tok_tile) <= total_tokens / tok_tile + num_reqs
+    P.tiles_by_request = (batch->max_q_len > 0 && batch->max_q_len <= P.tok_tile) ? 1 : 0;
+    const int grid_z = P.tiles_by_request ? batch->num_reqs : batch->total_tokens / P.tok_tile + batch->num_reqs;
+    const dim3 grid((unsigned)grid_x, (unsigned)(layout->local_kv_heads * P.q_subgroups), (unsigned)grid_z);
     hipStream_t stream = (hipStream_t)ex->stream;
     int rc;
-    if (nt == 1) {
-        rc = ensure_dynamic_lds(paged_attn_tq4_kernel<TQ, 1>, smem_bytes_for(1));
-        if (rc) return rc;
-        hipLaunchKernelGGL((paged_attn_tq4_kernel<TQ, 1>), grid, dim3(waves_for(1) * 64), smem_bytes_for(1), stream, P);
-    } else {
-        rc = ensure_dynamic_lds(paged_attn_tq4_kernel<TQ, 2>, smem_bytes_for(2));
-        if (rc) return rc;
-        hipLaunchKernelGGL((paged_attn_tq4_kernel<TQ, 2>), grid, dim3(waves_for(2) * 64), smem_bytes_for(2), stream, P);
-    }
+    rc = ensure_dynamic_lds(paged_attn_tq4_kernel<TQ, 1>, smem_bytes_for(1));
+    if (rc) return rc;
+    hipLaunchKernelGGL((paged_attn_tq4_kernel<TQ, 1>), grid, dim3(waves_for(1) * 64), smem_bytes_for(1), stream, P);
     rc = (int)hipGetLastError();
     if (rc) return rc;
     if (P.max_chunks > 1) {
@@ -1178,8 +1302,9 @@ static int launch_kv16(const warp34_exec* ex, const warp34_kv_layer_layout* layo
         const int bound = (units + P.min_upc - 1) / P.min_upc;
         if (bound < grid_x) grid_x = bound < 1 ? 1 : bound;
     }
-    const dim3 grid((unsigned)grid_x, (unsigned)(layout->local_kv_heads * P.q_subgroups),
-                    (unsigned)batch->total_tokens);
+    P.tiles_by_request = (batch->max_q_len > 0 && batch->max_q_len <= P.tok_tile) ? 1 : 0;
+    const int grid_z = P.tiles_by_request ? batch->num_reqs : batch->total_tokens / P.tok_tile + batch->num_reqs;
+    const dim3 grid((unsigned)grid_x, (unsigned)(layout->local_kv_heads * P.q_subgroups), (unsigned)grid_z);
     hipStream_t stream = (hipStream_t)ex->stream;
     int rc = ensure_dynamic_lds(paged_attn_kv16_kernel<TQ, 1>, kv16_smem_bytes(1));
     if (rc) return rc;

@@ -67,64 +67,49 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
     const warp34_kv_layer_layout& L = P.L;
     const warp34_attention_batch& B = P.B;
 
-    const int tok0 = (int)blockIdx.z;
+    const int tile_z = (int)blockIdx.z;  // tile index (see locate_tile)
     const int kv_sub = (int)blockIdx.y;
     const int kv_head = fast_div(kv_sub, P.q_subgroups);
     const int q_head_base = kv_head * P.gqa + (kv_sub - kv_head * P.q_subgroups) * P.q_group;
     const int chunk = (int)blockIdx.x;
-    if (tok0 >= B.total_tokens) return;
 
     // query rows in MFMA B layout straight from global memory: lane (n, b) holds
-    // Q[column n][32 m + 8 b .. + 7] for m = 0..7 (dead columns are zeroed below)
+    // Q[column n][32 m + 8 b .. + 7] for m = 0..7 (dead columns are zeroed below).  The first
+    // token of the tile is guessed so that these loads overlap the lookup; a wrong guess is
+    // corrected after it.
+    const int tok_guess = min(P.tiles_by_request ? tile_z : tile_z * P.tok_tile, B.total_tokens - 1);
     u4 bq[NT][8];
+    auto load_q = [&](int tokbase) {
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        const int col = nt * 16 + n;
-        const int t = fast_div(col, P.q_group);
-        const int a = col - t * P.q_group;
-        const int tok = min(tok0 + t, B.total_tokens - 1);
-        const uint16_t* qrow = P.q + ((size_t)tok * P.num_q_heads + (size_t)(q_head_base + a)) * kHeadDim;
+        for (int nt = 0; nt < NT; ++nt) {
+            const int col = nt * 16 + n;
+            const int t = fast_div(col, P.q_group);
+            const int a = col - t * P.q_group;
+            const int tok = min(tokbase + t, B.total_tokens - 1);
+            const uint16_t* qrow = P.q + ((size_t)tok * P.num_q_heads + (size_t)(q_head_base + a)) * kHeadDim;
 #pragma unroll
-        for (int m = 0; m < 8; ++m) bq[nt][m] = *reinterpret_cast<const u4*>(qrow + 32 * m + 8 * b);
-    }
+            for (int m = 0; m < 8; ++m) bq[nt][m] = *reinterpret_cast<const u4*>(qrow + 32 * m + 8 * b);
+        }
+    };
+    load_q(tok_guess);
 
-    // request lookup in one round trip (see the TQ4 kernel)
-    // Speculative block-table load, in flight together with the request lookup: it assumes
-    // that token t belongs to request t (a decode batch) and that the request's length is the
-    // host's bound max_seq_len.  When either guess is wrong the ids are fetched again below,
-    // so the guess changes the latency only, never the result.
-    const int spec_req = min(tok0, B.num_reqs - 1);
+    // Speculative block-table load, in flight together with the lookup: it assumes that the
+    // request's length is the host's bound max_seq_len.  A wrong guess is fetched again below,
+    // so it changes the latency only, never the result.
     int spec_slot_base = -1, spec_vec = -1;
-    if (B.sliding_window <= 0 && B.max_seq_len > 0 && spec_req >= 0) {
+    if (P.tiles_by_request && B.sliding_window <= 0 && B.max_seq_len > 0) {
         const ChunkGeom sg = chunk_geom(0, B.max_seq_len - 1, P.max_chunks, P.min_upc);
         spec_slot_base = fast_div((sg.u_first + chunk * sg.upc) * kUnit, L.block_size);
         const int slot = spec_slot_base + lane;
         if (slot < B.max_blocks_per_req)
-            spec_vec = B.block_tables[(size_t)spec_req * B.max_blocks_per_req + slot];
+            spec_vec = B.block_tables[(size_t)tile_z * B.max_blocks_per_req + slot];
     }
-    bool req_hit = false;
-    int req = -1, rq_start = 0, rq_end = 0, seq_after = 0, ctx_before = 0;
-    for (int base = 0; base < B.num_reqs && !req_hit; base += 64) {
-        const int r = base + lane;
-        const bool inb = r < B.num_reqs;
-        const int lo = inb ? B.query_start_loc[r] : 0x7fffffff;
-        const int hi = inb ? B.query_start_loc[r + 1] : -0x7fffffff;
-        const int sa = inb ? B.seq_lens_after[r] : 0;
-        const int cb = (inb && B.context_lens_before != nullptr) ? B.context_lens_before[r] : 0;
-        const int rm = (inb && B.valid_req_mask != nullptr) ? (int)B.valid_req_mask[r] : 1;
-        const unsigned long long hits = __ballot(inb && tok0 >= lo && tok0 < hi);
-        if (hits != 0ull) {
-            const int src = __builtin_ctzll(hits);
-            req = base + src;
-            rq_start = __builtin_amdgcn_readlane(lo, src);
-            rq_end = __builtin_amdgcn_readlane(hi, src);
-            seq_after = __builtin_amdgcn_readlane(sa, src);
-            ctx_before = B.context_lens_before != nullptr ? __builtin_amdgcn_readlane(cb, src)
-                                                          : seq_after - (rq_end - rq_start);
-            req_hit = __builtin_amdgcn_readlane(rm, src) != 0;
-            if (!req_hit) break;
-        }
-    }
+    const TileInfo ti = locate_tile(P, tile_z, lane);
+    if (!ti.hit) return;  // no such tile, empty or masked request: outputs untouched
+    const int req = ti.req, rq_start = ti.rq_start, rq_end = ti.rq_end;
+    const int seq_after = ti.seq_after, ctx_before = ti.ctx_before;
+    const int tok0 = rq_start + ti.tile_in_req * P.tok_tile;
+    if (tok0 != tok_guess) load_q(tok0);  // wave-uniform, rare
     bool tok_ok[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
@@ -132,8 +117,6 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
         tok_ok[nt] = tok < B.total_tokens &&
                      (B.valid_token_mask == nullptr || B.valid_token_mask[min(tok, B.total_tokens - 1)] != 0);
     }
-    if (!req_hit) return;
-    if ((tok0 - rq_start) - fast_div(tok0 - rq_start, P.tok_tile) * P.tok_tile != 0) return;
     int tile_tokens = rq_end - tok0;
     if (tile_tokens > P.tok_tile) tile_tokens = P.tok_tile;
 
@@ -359,7 +342,7 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
 
     // halves of this wave's units, in order; the next half is in flight while one is processed
     int unit = cu_first + wave;
-    if (req == spec_req && slot_base == spec_slot_base) {
+    if (slot_base == spec_slot_base) {
         page_vec = spec_vec;
     } else {
         load_page_vec();
