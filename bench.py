@@ -9,7 +9,7 @@ the figure is an HBM figure.  K/V are synthetic bf16 N(0,1) with 1 % outlier cha
 TQ4-encoded by the library's own quantize-on-append kernel into 64-token pages whose
 physical order is a random permutation.
 
-Prints ONE JSON line (see README / DESIGN for the fields).
+Prints ONE JSON line.
 """
 import argparse
 import ctypes as C
@@ -36,6 +36,10 @@ WORKLOADS = {
     # 16 sequences of 262 144 tokens that share the pages of a 200 000-token prefix; 4 query tokens each
     "tq4_verify_16x4_ctx262144_shared200k": ("tq4", [262144] * 16, 0),
 }
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by
+# a plain copy of known size (profiles/paged_attn_tq4_decode_b1_ctx131072_hbm_traffic.txt); counters cannot
+# be read from inside this process, so workloads without such a profile report null.
+MEASURED_TRAFFIC = {"tq4_decode_b1_ctx131072": 71_824_000}
 SHARED_PREFIX = {"tq4_verify_16x4_ctx262144_shared200k": 200000}
 VERIFY_Q = {"tq4_verify_16x4_ctx262144_shared200k": 4}
 PREFILL_CHUNK = 2048
@@ -51,6 +55,9 @@ def parse():
     ap.add_argument("--ctx", type=int, default=0, help="override: one request with this context length")
     ap.add_argument("--layers", type=int, default=0, help="KV pools to cycle through (0 = auto, > 256 MB total)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run plain 256 MiB device copies instead of a workload (scale reference for the "
+                         "FETCH_SIZE / WRITE_SIZE counters of rocprofv3 --pmc)")
     ap.add_argument("--cpu-ctx", type=int, default=32768, help="context length of the CPU-oracle sample")
     args = ap.parse_args()
     prefill = args.workload.startswith("tq4_prefill")
@@ -262,6 +269,15 @@ def main():
     lib = ffi.load()
     dev = "cuda:0"
     torch.cuda.set_device(0)
+    if args.calibrate_copy:
+        n = 256 << 20
+        src = torch.full((n,), 7, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes": n, "copies": 10}))
+        return
     fmt, ctx, pool_tokens = build_workload(args.workload)
     if args.ctx:
         ctx = np.array([args.ctx], dtype=np.int64)
@@ -355,7 +371,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(gbs / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC.get(args.workload),
             "kernel": "paged_attn_%s_kernel (+ split_merge_kernel, both inside the timed launch)"
                       % ("tq4" if fmt == "tq4" else "kv16"),
             "avg_launch_us": round(ms_per_step * 1e3, 3),

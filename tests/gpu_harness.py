@@ -161,7 +161,7 @@ def channel_scale(v_bits, dtype, hbatch, num_q_heads):
 
 
 def assert_close(got_bits, dtype, want_f32, atol=2e-3, rtol=1e-2, what="", scale=None):
-    """BASELINE tolerance (max-abs 2e-3, max-rel 1e-2 against the fp32-dequant / fp64-accumulate
+    """Target tolerance (max-abs 2e-3, max-rel 1e-2 against the fp32-dequant / fp64-accumulate
     oracle), with the absolute part relative to the magnitude of the data being averaged:
 
         |got - want| <= atol * scale + rtol * |want|
@@ -169,7 +169,7 @@ def assert_close(got_bits, dtype, want_f32, atol=2e-3, rtol=1e-2, what="", scale
     An attention output is a probability-weighted mean of V rows, so an error eps in the
     probabilities moves channel c by up to eps * max_t |V[t, c]|; `scale` is that magnitude
     (channel_scale()), or, when not given, max(1, max|want_row|).  It differs from 1 only for
-    the x20 outlier channels of the BASELINE inputs, where a single fp16 / bf16 output ulp
+    the x20 outlier channels of the benchmark inputs, where a single fp16 / bf16 output ulp
     already exceeds 2e-3.  On unit-scale data this is exactly 2e-3 + 1e-2 |want|.
     The max-rel figure max|err| / max|want| must also stay below rtol.
     """

@@ -1,7 +1,7 @@
 """GPU parity: quantize-on-append through the C ABI vs the CPU oracle -- bit-exact.
 
 Cases follow the reference's write tests (tests/backbone_and_collectives.rs:455-572 page
-placement and 132-byte strides, tests/paged_fa2.rs:618-691 mask contract) and BASELINE
+placement and 132-byte strides, tests/paged_fa2.rs:618-691 mask contract) and benchmark
 config 1 (4096 tokens, 2 kv heads, 64-token pages in a seeded random physical order,
 1 % outlier channels).
 """
@@ -48,7 +48,7 @@ def _run_append(fmt, xf, block_size, n_tokens, in_dtype, seed, kv_heads=2, tmask
 
 @pytest.mark.parametrize("in_dtype", [DT_BF16, DT_F16])
 def test_config1_tq4_append_bit_exact(in_dtype):
-    """BASELINE config 1: 4096 tokens x 2 kv heads, 64-token pages, permuted physical order."""
+    """Benchmark configuration 1: 4096 tokens x 2 kv heads, 64-token pages, permuted physical order."""
     hpool, gk, gv = _run_append(FMT_TQ4, XF_WHT256, 64, 4096, in_dtype, seed=0)
     assert hpool.tok == 132 and hpool.head == 64 * 132 and hpool.page == 2 * 64 * 132
     assert gk.tobytes() == hpool.k.tobytes()

@@ -1,6 +1,6 @@
 """GPU parity: paged GQA decode / verify attention through the C ABI vs the CPU oracle.
 
-Tolerance (BASELINE): |got - want| <= 2e-3 * scale + 1e-2 |want| against the fp64-accumulating oracle,
+Tolerance: |got - want| <= 2e-3 * scale + 1e-2 |want| against the fp64-accumulating oracle,
 scale = magnitude of the V channel being averaged (1 on unit-scale data, see gpu_harness.assert_close).
 Invariants follow the reference's GPU tests: page-permutation 0-ULP
 (tests/backbone_and_collectives.rs:455-572), split vs single pass < 2e-3 and graph-bucket
@@ -166,7 +166,7 @@ def test_kv16_decode_gqa8_long(fmt, dtype, scratch):
 
 
 def test_kv16_bf16_decode_ctx32k():
-    """BASELINE bf16 decode shape: ctx 32768, 16 q / 2 kv heads, 64-token pages."""
+    """Benchmark bf16 decode shape: ctx 32768, 16 q / 2 kv heads, 64-token pages."""
     _check(FMT_BF16, DT_BF16, 64, [32768], [1], 131, scratch=64 << 20, q_heads=16)
 
 

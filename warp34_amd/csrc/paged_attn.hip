@@ -38,7 +38,6 @@
 //
 // MFMA use: v_mfma_f32_16x16x32_f16.  A = K rows (QK) or V^T (PV) so that every lane owns one
 // query column: softmax state and the O rescale are per-lane scalars.
-#include <cstdlib>
 #include <type_traits>
 
 #include "kv_common.h"
@@ -76,10 +75,13 @@ constexpr float kLutGain = 1.908032f;
 constexpr float kLutInvGain = 1.0f / kLutGain;
 
 #ifdef W34_TRACE
+#ifndef W34_TRACE_Z
+#define W34_TRACE_Z 0
+#endif
 __device__ unsigned long long g_trace[64 * 64];
 #define W34_TP(slot)                                                                   \
     do {                                                                               \
-        if (lane == 0 && (blockIdx.x == 0 || blockIdx.x == 77) && blockIdx.y == 0 && blockIdx.z == 0) {  \
+        if (lane == 0 && (blockIdx.x == 0 || blockIdx.x == 77) && blockIdx.y == 0 && blockIdx.z == W34_TRACE_Z) {  \
             g_trace[((blockIdx.x ? 8 : 0) + wave) * 64 + (slot)] = __builtin_readcyclecounter(); \
             if ((slot) == 0) g_trace[((blockIdx.x ? 8 : 0) + wave) * 64 + 63] = wall_clock64(); \
             if ((slot) == 40) g_trace[((blockIdx.x ? 8 : 0) + wave) * 64 + 62] = wall_clock64(); \
@@ -841,13 +843,6 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
 #endif
         if (unit + kWaves < cu_end) issue_loads(unit + kWaves);
         const int t0 = unit * kUnit;
-        // The two waves that share a SIMD take turns at the higher issue priority, unit by
-        // unit; with equal priorities the older wave always wins and finishes ~25 % earlier.
-        if ((((unit - cu_first) >> (kWaves == 8 ? 3 : 2)) ^ (wave >> 2)) & 1) {
-            __builtin_amdgcn_s_setprio(1);
-        } else {
-            __builtin_amdgcn_s_setprio(0);
-        }
         process_unit(t0, !(t0 >= i_lo && t0 + kUnit - 1 <= i_hi));
 #ifdef W34_TRACE
         if (trace_it < 8) W34_TP(4 + 4 * trace_it + 3);
@@ -855,7 +850,6 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
 #endif
     }
     W34_TP(36);
-    __builtin_amdgcn_s_setprio(0);
 
     // ---- combine the per-lane partial sums of l over the four k-block lanes of a column ------
 #pragma unroll
