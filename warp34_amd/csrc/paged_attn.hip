@@ -989,7 +989,9 @@ extern "C" int warp34_debug_read_trace(unsigned long long* dst) {
 constexpr int kMergeGroups = 16;
 constexpr int kMergeMaxPerGroup = 16;  // max_chunks <= 256
 template <typename TQ>
-__global__ __launch_bounds__(1024) void split_merge_kernel(const AttnParams P, float out_scale, int rotate) {
+__global__ __launch_bounds__(1024) void split_merge_kernel(const float* part_acc_in, const float* part_ml_in,
+                                                           int max_chunks_in, const AttnParams P,
+                                                           float out_scale, int rotate) {
     __shared__ f4 s_acc[kMergeGroups][64];
     __shared__ f4 s_rec[256];
     __shared__ float s_red[kMergeGroups];
@@ -1000,18 +1002,21 @@ __global__ __launch_bounds__(1024) void split_merge_kernel(const AttnParams P, f
     const long long row = (long long)blockIdx.x;
     const int tok = (int)(row / P.num_q_heads);
     const warp34_attention_batch& B = P.B;
-    const float* ml = P.part_ml + (size_t)row * P.max_chunks * 4;
-    const float* acc = P.part_acc + (size_t)row * P.max_chunks * kHeadDim;
+    // the leading arguments repeat P.part_acc / P.part_ml / P.max_chunks: they are preloaded into
+    // scalar registers at wave launch, so the speculative loads below do not wait for the
+    // kernel-argument fetch
+    const float* ml = part_ml_in + (size_t)row * max_chunks_in * 4;
+    const float* acc = part_acc_in + (size_t)row * max_chunks_in * kHeadDim;
 
     // speculative loads: chunk records (one per thread) and this thread's accumulator slices
     f4 rec = {kNegBig, 0.f, 0.f, 0.f};
-    if (tid < P.max_chunks) rec = *reinterpret_cast<const f4*>(ml + 4 * tid);
+    if (tid < max_chunks_in) rec = *reinterpret_cast<const f4*>(ml + 4 * tid);
     f4 a[kMergeMaxPerGroup];
 #pragma unroll
     for (int k = 0; k < kMergeMaxPerGroup; ++k) {
         const int s = grp + k * kMergeGroups;
         a[k] = f4{0.f, 0.f, 0.f, 0.f};
-        if (s < P.max_chunks) a[k] = *reinterpret_cast<const f4*>(acc + (size_t)s * kHeadDim + 4 * lane);
+        if (s < max_chunks_in) a[k] = *reinterpret_cast<const f4*>(acc + (size_t)s * kHeadDim + 4 * lane);
     }
     // row validity (wave 0): token mask and owning request, first match wins
     if (grp == 0) {
@@ -1250,8 +1255,8 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     rc = (int)hipGetLastError();
     if (rc) return rc;
     if (P.max_chunks > 1) {
-        hipLaunchKernelGGL((split_merge_kernel<TQ>), dim3((unsigned)rows), dim3(1024), 0, stream, P,
-                           kLutInvGain, 1);
+        hipLaunchKernelGGL((split_merge_kernel<TQ>), dim3((unsigned)rows), dim3(1024), 0, stream,
+                           (const float*)P.part_acc, (const float*)P.part_ml, P.max_chunks, P, kLutInvGain, 1);
         rc = (int)hipGetLastError();
     }
     return rc;
@@ -1306,7 +1311,8 @@ static int launch_kv16(const warp34_exec* ex, const warp34_kv_layer_layout* layo
     rc = (int)hipGetLastError();
     if (rc) return rc;
     if (P.max_chunks > 1) {
-        hipLaunchKernelGGL((split_merge_kernel<TQ>), dim3((unsigned)rows), dim3(1024), 0, stream, P, 1.0f, 0);
+        hipLaunchKernelGGL((split_merge_kernel<TQ>), dim3((unsigned)rows), dim3(1024), 0, stream,
+                           (const float*)P.part_acc, (const float*)P.part_ml, P.max_chunks, P, 1.0f, 0);
         rc = (int)hipGetLastError();
     }
     return rc;
