@@ -1,0 +1,176 @@
+"""GPU parity at the full benchmark sizes (batched decode, chunked prefill, shared-prefix verify).
+
+The pools are too large to build with the CPU oracle in test time, so each test
+  1. appends bf16 rows through the library's append entry point (its bit-exactness against the
+     oracle is established row by row in test_gpu_append.py) and re-checks a random sample of
+     the appended rows against the oracle's encoder, byte for byte, at this size;
+  2. downloads the pool and lets the oracle attend over those very bytes;
+  3. compares the library's attention output with it under the usual tolerance
+     (|err| <= 2e-3 * scale + 1e-2 |want|, scale = magnitude of the V channel, see gpu_harness).
+Where the oracle would take minutes (prefill: 16 384 query tokens) it is run on a sample of the
+query tokens through its own token mask; the library computes every token.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle
+from oracle import DT_BF16, FMT_TQ4
+
+pytestmark = pytest.mark.gpu
+
+KV_HEADS, Q_HEADS, D, BS = 2, 16, 256, 64
+
+
+class BigPool:
+    """TQ4 pool on the device, filled request by request through warp34_kv_cache_write_bf16."""
+
+    def __init__(self, ctx, num_pages, seed, shared_prefix=0, sample_rows=512):
+        import torch
+
+        import gpu_harness as G
+        from warp34_amd import ffi
+
+        self.torch, self.G, self.ffi = torch, G, ffi
+        self.ctx = [int(c) for c in ctx]
+        self.host = oracle.HostPool(num_pages, KV_HEADS, D, BS, FMT_TQ4, oracle.XF_WHT256)
+        self.dev = G.DevPool(self.host, fill=0)
+        g = torch.Generator(device=G.DEV)
+        g.manual_seed(seed)
+        pages_per = [(c + BS - 1) // BS for c in self.ctx]
+        shared_pages = shared_prefix // BS
+        perm = oracle.permutation(num_pages, seed).astype(np.int32)
+        self.bt = np.zeros((len(ctx), max(pages_per)), dtype=np.int32)
+        at = 0
+        for r, n in enumerate(pages_per):
+            if r > 0 and shared_pages:
+                self.bt[r, :shared_pages] = self.bt[0, :shared_pages]
+                self.bt[r, shared_pages:n] = perm[at:at + n - shared_pages]
+                at += n - shared_pages
+            else:
+                self.bt[r, :n] = perm[at:at + n]
+                at += n
+        gain = torch.ones((KV_HEADS, D), device=G.DEV)
+        for h in range(KV_HEADS):
+            gain[h, torch.randperm(D, generator=g, device=G.DEV)[:3]] = 20.0
+        self.v_absmax = np.zeros((len(ctx), KV_HEADS, D), dtype=np.float32)
+        self.samples = []  # (k rows, v rows, slots) of a few chunks, for the encoder re-check
+        lib = G.lib()
+        L = self.dev.layout()
+        ex, _ = G.make_exec()
+        bt_dev = G.to_dev(self.bt)
+        chunk = 4096
+        rng = np.random.default_rng(seed)
+        shared_v_absmax = None
+        for r, c in enumerate(self.ctx):
+            first = shared_pages * BS if r > 0 else 0
+            vmax = torch.zeros((KV_HEADS, D), device=G.DEV)
+            for t0 in range(first, c, chunk):
+                n = min(chunk, c - t0)
+                kk = (torch.randn((n, KV_HEADS, D), generator=g, device=G.DEV) * gain).to(torch.bfloat16)
+                vv = (torch.randn((n, KV_HEADS, D), generator=g, device=G.DEV) * gain).to(torch.bfloat16)
+                pos = np.arange(t0, t0 + n)
+                slots = (self.bt[r, pos // BS].astype(np.int64) * BS + pos % BS).astype(np.int32)
+                sl = G.to_dev(slots)
+                qsl = G.to_dev(np.array([0, n], dtype=np.int32))
+                seq = G.to_dev(np.array([t0 + n], dtype=np.int32))
+                b = ffi.Warp34AttentionBatch(qsl.data_ptr(), None, seq.data_ptr(), bt_dev[r].data_ptr(), sl.data_ptr(),
+                                             None, None, 1, n, self.bt.shape[1], n, t0 + n, 0, 0, 0.0625, 0)
+                rc = lib.warp34_kv_cache_write_bf16(C.byref(ex), C.byref(L), C.byref(b),
+                                                    C.c_void_p(kk.data_ptr()), C.c_void_p(vv.data_ptr()))
+                assert rc == 0
+                vmax = torch.maximum(vmax, vv.float().abs().amax(dim=0))
+                if len(self.samples) < 6 and rng.random() < 0.2:
+                    pick = rng.choice(n, size=min(sample_rows // 6 + 1, n), replace=False)
+                    self.samples.append((kk[pick].cpu().view(torch.int16).numpy().view(np.uint16),
+                                         vv[pick].cpu().view(torch.int16).numpy().view(np.uint16), slots[pick]))
+            torch.cuda.synchronize()
+            if shared_pages:  # later requests also average over request 0's (shared) rows
+                if r == 0:
+                    shared_v_absmax = vmax.clone()
+                else:
+                    vmax = torch.maximum(vmax, shared_v_absmax)
+            self.v_absmax[r] = vmax.cpu().numpy()
+        k, v = self.dev.download()
+        self.host.k[:] = k
+        self.host.v[:] = v
+
+    def check_sampled_rows_bit_exact(self):
+        """Rows appended by the library == rows encoded by the oracle, byte for byte."""
+        h = self.host
+        checked = 0
+        for kk, vv, slots in self.samples:
+            for i, slot in enumerate(slots):
+                page, off = int(slot) // BS, int(slot) % BS
+                for head in range(KV_HEADS):
+                    base = page * h.page + head * h.head + off * h.tok
+                    for src, slab in ((kk, h.k), (vv, h.v)):
+                        want = oracle.encode_row(oracle.bf16_bits_to_f32(src[i, head]))
+                        assert bytes(slab[base:base + 132]) == bytes(want), "row at slot %d differs" % slot
+                        checked += 1
+        assert checked >= 256
+        return checked
+
+    def scale_for(self, hb):
+        g = Q_HEADS // KV_HEADS
+        out = np.ones((hb.total_tokens, Q_HEADS, D))
+        for r in range(hb.num_reqs):
+            s = np.maximum(1.0, np.repeat(self.v_absmax[r], g, axis=0))
+            out[int(hb.qsl[r]):int(hb.qsl[r + 1])] = s
+        return out
+
+
+def _attend_and_compare(pool, hb, q, rows=None, oracle_batch=None, scratch=32 << 20):
+    G = pool.G
+    want = oracle.paged_attention(pool.host, oracle_batch or hb, q, DT_BF16, Q_HEADS, n_threads=oracle.hw_threads())
+    rc, got, _ = G.dev_attention(pool.dev, hb, q, DT_BF16, Q_HEADS, scratch_bytes=scratch)
+    assert rc == 0
+    scale = pool.scale_for(hb)
+    if rows is not None:
+        got, want, scale = got[rows], want[rows], scale[rows]
+    return G.assert_close(got, DT_BF16, want, what="full size", scale=scale)
+
+
+def test_batched_decode_32_sequences_1k_to_64k():
+    """32 sequences, context lengths drawn from 1K..64K (seeded), pages scattered over a
+    2M-token pool, one query token each."""
+    ctx = np.random.default_rng(0).integers(1024, 65537, size=32)
+    pool = BigPool(ctx, (2 << 20) // BS, seed=401)
+    pool.check_sampled_rows_bit_exact()
+    R = len(ctx)
+    q = oracle.fill_normal(R * Q_HEADS * D, 402, DT_BF16).reshape(R, Q_HEADS, D)
+    hb = oracle.HostBatch(np.arange(R + 1), pool.ctx, pool.bt, context_lens_before=[c - 1 for c in pool.ctx])
+    _attend_and_compare(pool, hb, q)
+
+
+def test_verify_16x4_tokens_262144_keys_shared_prefix():
+    """16 sequences of 262 144 tokens sharing the pages of a 200 000-token prefix, 4 query
+    tokens each with causal masking among them."""
+    R, n, ql, shared = 16, 262144, 4, 200000
+    pages = shared // BS + R * ((n + BS - 1) // BS - shared // BS) + 8
+    pool = BigPool([n] * R, pages, seed=411, shared_prefix=shared)
+    assert (pool.bt[1:, :shared // BS] == pool.bt[0, :shared // BS]).all()
+    pool.check_sampled_rows_bit_exact()
+    q = oracle.fill_normal(R * ql * Q_HEADS * D, 412, DT_BF16).reshape(R * ql, Q_HEADS, D)
+    hb = oracle.HostBatch(np.arange(R + 1) * ql, pool.ctx, pool.bt, context_lens_before=[n - ql] * R)
+    _attend_and_compare(pool, hb, q)
+
+
+def test_chunked_prefill_8x2048_on_16k_prefix():
+    """8 sequences: 16 384-token prefix + 2 048-token chunk, causal attention of the whole chunk
+    (tile kernel); the oracle checks 96 of the 16 384 query tokens."""
+    R, prefix, chunk = 8, 16384, 2048
+    pool = BigPool([prefix + chunk] * R, R * ((prefix + chunk) // BS) + 8, seed=421)
+    pool.check_sampled_rows_bit_exact()
+    N = R * chunk
+    q = oracle.fill_normal(N * Q_HEADS * D, 422, DT_BF16).reshape(N, Q_HEADS, D)
+    hb = oracle.HostBatch(np.arange(R + 1) * chunk, pool.ctx, pool.bt, context_lens_before=[prefix] * R)
+    rng = np.random.default_rng(423)
+    rows = np.unique(np.concatenate([rng.choice(N, size=80, replace=False),
+                                     np.arange(R) * chunk, np.arange(R) * chunk + chunk - 1]))
+    mask = np.zeros(N, dtype=np.uint8)
+    mask[rows] = 1
+    ob = oracle.HostBatch(np.arange(R + 1) * chunk, pool.ctx, pool.bt, context_lens_before=[prefix] * R,
+                          valid_token_mask=mask)
+    _attend_and_compare(pool, hb, q, rows=rows, oracle_batch=ob)
