@@ -270,13 +270,24 @@ def main():
     dev = "cuda:0"
     torch.cuda.set_device(0)
     if args.calibrate_copy:
+        # plain device copies: scale reference for the traffic counters, and the streaming rate this
+        # device reaches on the simplest possible kernel (read + written bytes per second)
         n = 256 << 20
         src = torch.full((n,), 7, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
-        for _ in range(10):
+        for _ in range(3):
             dst.copy_(src)
         torch.cuda.synchronize()
-        print(json.dumps({"calibrate_copy_bytes": n, "copies": 10}))
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            dst.copy_(src)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / 10
+        print(json.dumps({"calibrate_copy_bytes": n, "copies": 13,
+                          "copy_GBps_read_plus_write": round(2 * n / ms / 1e6, 1)}))
         return
     fmt, ctx, pool_tokens = build_workload(args.workload)
     if args.ctx:
@@ -285,7 +296,7 @@ def main():
     total_tokens_kv = int(ctx.sum())
     row_bytes = ROW_BYTES[fmt]
     kv_bytes = total_tokens_kv * KV_HEADS * 2 * row_bytes  # algorithmic bytes per step (K + V rows)
-    shared = 0 if os.environ.get("W34_NOSHARE") else SHARED_PREFIX.get(args.workload, 0)
+    shared = SHARED_PREFIX.get(args.workload, 0)
     pool_pages = max(sum((int(c) + BLOCK - 1) // BLOCK for c in ctx) + 16, pool_tokens // BLOCK)
     pool_pages -= (len(ctx) - 1) * (shared // BLOCK)
     if shared:  # unique bytes: the prefix once, every private suffix once
@@ -299,7 +310,7 @@ def main():
         return
 
     R = len(ctx)
-    ql = int(os.environ.get("W34_QL", VERIFY_Q.get(args.workload, 1)))  # query tokens per request (1 = decode)
+    ql = VERIFY_Q.get(args.workload, 1)  # query tokens per request (1 = decode)
     g = torch.Generator(device=dev)
     g.manual_seed(7)
     q = torch.randn((R * ql, Q_HEADS, HEAD_DIM), generator=g, device=dev).to(torch.bfloat16)
