@@ -121,4 +121,31 @@ __device__ __forceinline__ float xor_lane(float v) {
     return __shfl_xor(v, MASK, 64);
 }
 
+// value of lane (lane ^ H) for every lane of a wave, built from DPP / lane-swap VALU ops
+// (no LDS round trip): quad permutes for 1 and 2, row shifts for 4, a row rotate for 8 and
+// the gfx950 row / half swaps for 16 and 32.
+template <int H>
+__device__ __forceinline__ float lane_xor(float x, int lane) {
+    const int xi = __float_as_int(x);
+    if constexpr (H == 1) {
+        return __int_as_float(__builtin_amdgcn_mov_dpp(xi, 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
+    } else if constexpr (H == 2) {
+        return __int_as_float(__builtin_amdgcn_mov_dpp(xi, 0x4E, 0xF, 0xF, true));  // quad_perm [2,3,0,1]
+    } else if constexpr (H == 4) {
+        // banks 0,2 (lanes 0-3, 8-11 of a row) take lane+4, banks 1,3 take lane-4
+        int r = __builtin_amdgcn_update_dpp(0, xi, 0x104, 0xF, 0x5, false);  // row_shl:4
+        r = __builtin_amdgcn_update_dpp(r, xi, 0x114, 0xF, 0xA, false);      // row_shr:4
+        return __int_as_float(r);
+    } else if constexpr (H == 8) {
+        return __int_as_float(__builtin_amdgcn_mov_dpp(xi, 0x128, 0xF, 0xF, true));  // row_ror:8
+    } else if constexpr (H == 16) {
+        const auto r = __builtin_amdgcn_permlane16_swap((uint32_t)xi, (uint32_t)xi, false, false);
+        return __uint_as_float((lane & 16) ? r[0] : r[1]);
+    } else {
+        const auto r = __builtin_amdgcn_permlane32_swap((uint32_t)xi, (uint32_t)xi, false, false);
+        return __uint_as_float((lane & 32) ? r[0] : r[1]);
+    }
+}
+
+
 }  // namespace w34

@@ -17,28 +17,41 @@
 
 namespace w34 {
 
+// Cross-lane moves are DPP / lane-swap VALU operations (lane_xor), not LDS permutes: the encode
+// of one row needs 168 of them.  They only move bits, so the arithmetic (and its order) is the
+// one of the 32-lane shuffle tree it replaces.
+__device__ __forceinline__ int lane_xor1_int(int x, int lane) {
+    return __float_as_int(lane_xor<1>(__int_as_float(x), lane));
+}
+
 // 32-lane xor butterfly sum, offsets 16,8,4,2,1 (tq4_kv_common.cuh:54-60).
-__device__ __forceinline__ float half_wave_sum(float v) {
-    v += __shfl_xor(v, 16, 64);
-    v += __shfl_xor(v, 8, 64);
-    v += __shfl_xor(v, 4, 64);
-    v += __shfl_xor(v, 2, 64);
-    v += __shfl_xor(v, 1, 64);
+__device__ __forceinline__ float half_wave_sum(float v, int lane) {
+    v += lane_xor<16>(v, lane);
+    v += lane_xor<8>(v, lane);
+    v += lane_xor<4>(v, lane);
+    v += lane_xor<2>(v, lane);
+    v += lane_xor<1>(v, lane);
     return v;
+}
+
+template <int H>
+__device__ __forceinline__ float wht_lane_stage(float val, int lane) {
+    const float o = lane_xor<H>(val, lane);
+    return (lane & H) ? (o - val) : (val + o);
 }
 
 // 256-point Walsh-Hadamard over 32 lanes x 8 registers (tq4_kv_common.cuh:75-107):
 // stages over index bits 0..4 cross lanes, bits 5..7 stay in registers; the last stage
 // carries the 1/16 scale.
-__device__ __forceinline__ void wht256_half_wave(float (&v)[8], int l32) {
+__device__ __forceinline__ void wht256_half_wave(float (&v)[8], int lane) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         float val = v[j];
-#pragma unroll
-        for (int h = 1; h < 32; h <<= 1) {
-            const float o = __shfl_xor(val, h, 64);
-            val = (l32 & h) ? (o - val) : (val + o);
-        }
+        val = wht_lane_stage<1>(val, lane);
+        val = wht_lane_stage<2>(val, lane);
+        val = wht_lane_stage<4>(val, lane);
+        val = wht_lane_stage<8>(val, lane);
+        val = wht_lane_stage<16>(val, lane);
         v[j] = val;
     }
 #pragma unroll
@@ -65,16 +78,18 @@ __device__ __forceinline__ void wht256_half_wave(float (&v)[8], int l32) {
 }
 
 // TQ4 encode of one 256-wide row held as v[j] = x[l32 + 32 j] (op_kv_cache.cu:152-218).
-__device__ __forceinline__ void tq4_encode_row(float (&v)[8], int l32, uint8_t* dst) {
+// The 132 row bytes are assembled in `row` (LDS, private to this half-wave).
+__device__ __forceinline__ void tq4_encode_row(float (&v)[8], int lane, uint8_t* row) {
+    const int l32 = lane & 31;
 #pragma unroll
     for (int j = 0; j < 8; ++j) v[j] = apply_sign(v[j], l32 + 32 * j);
-    wht256_half_wave(v, l32);
+    wht256_half_wave(v, lane);
 
     float s_sq0 = 0.0f, s_sq1 = 0.0f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        s_sq0 += half_wave_sum(v[j] * v[j]);
-        s_sq1 += half_wave_sum(v[j + 4] * v[j + 4]);
+        s_sq0 += half_wave_sum(v[j] * v[j], lane);
+        s_sq1 += half_wave_sum(v[j + 4] * v[j + 4], lane);
     }
     const float rs0 = (float)(1.0 / sqrt((double)s_sq0));
     const float rs1 = (float)(1.0 / sqrt((double)s_sq1));
@@ -91,13 +106,13 @@ __device__ __forceinline__ void tq4_encode_row(float (&v)[8], int l32, uint8_t* 
         for (int i = 0; i < 15; ++i) q += (rv > kBoundaries[i]) ? 1 : 0;
         // byte m of a 64-byte block holds elements 2m (low nibble) and 2m+1 (high nibble);
         // elements l32 and l32^1 of register j are neighbours.
-        const int partner = __shfl_xor(q, 1, 64);
+        const int partner = lane_xor1_int(q, lane);
         if ((l32 & 1) == 0) {
-            dst[66 * (j >> 2) + 2 + (((j & 3) * 32 + l32) >> 1)] = (uint8_t)(q | (partner << 4));
+            row[66 * (j >> 2) + 2 + (((j & 3) * 32 + l32) >> 1)] = (uint8_t)(q | (partner << 4));
         }
         const float c = kCentroids[q];
-        const float vc = half_wave_sum(raw_v * c);
-        const float cc = half_wave_sum(c * c);
+        const float vc = half_wave_sum(raw_v * c, lane);
+        const float cc = half_wave_sum(c * c, lane);
         if (j < 4) {
             vc_dot0 += vc;
             c_sq0 += cc;
@@ -109,8 +124,8 @@ __device__ __forceinline__ void tq4_encode_row(float (&v)[8], int l32, uint8_t* 
     if (l32 == 0) {
         const float d0 = (c_sq0 > 1e-10f) ? (vc_dot0 / c_sq0) : 0.0f;
         const float d1 = (c_sq1 > 1e-10f) ? (vc_dot1 / c_sq1) : 0.0f;
-        *reinterpret_cast<uint16_t*>(dst) = F16::from_f32(d0);
-        *reinterpret_cast<uint16_t*>(dst + 66) = F16::from_f32(d1);
+        *reinterpret_cast<uint16_t*>(row) = F16::from_f32(d0);
+        *reinterpret_cast<uint16_t*>(row + 66) = F16::from_f32(d1);
     }
 }
 
@@ -155,7 +170,26 @@ __global__ __launch_bounds__(256) void kv_append_kernel(warp34_kv_layer_layout L
         float v[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] = TIn::to_f32(src[l32 + 32 * j]);
-        tq4_encode_row(v, l32, dst);
+        // the row is assembled in LDS and leaves with one 32-bit store per lane (16-bit stores
+        // when the destination is only 2-byte aligned, which is all the row format promises)
+        __shared__ __align__(4) uint8_t rows[4][2][136];
+        uint8_t* row = rows[wave][is_v];
+        tq4_encode_row(v, lane, row);
+        __atomic_signal_fence(__ATOMIC_SEQ_CST);
+        __builtin_amdgcn_wave_barrier();
+        __atomic_signal_fence(__ATOMIC_SEQ_CST);
+        if ((reinterpret_cast<uintptr_t>(dst) & 3u) == 0) {
+            const uint32_t* r32 = reinterpret_cast<const uint32_t*>(row);
+            uint32_t* d32 = reinterpret_cast<uint32_t*>(dst);
+            d32[l32] = r32[l32];
+            if (l32 == 0) d32[32] = r32[32];
+        } else {
+            const uint16_t* r16 = reinterpret_cast<const uint16_t*>(row);
+            uint16_t* d16 = reinterpret_cast<uint16_t*>(dst);
+            d16[l32] = r16[l32];
+            d16[l32 + 32] = r16[l32 + 32];
+            if (l32 < 2) d16[l32 + 64] = r16[l32 + 64];
+        }
         return;
     }
     // 16-bit storage formats: plain copy when the storage type is the source type,
