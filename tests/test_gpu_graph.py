@@ -1,0 +1,122 @@
+"""The append and attention entry points inside a captured HIP graph.
+
+The reference replays one captured decode step with mutated DEVICE-side lengths, block tables
+and slots while the host-side scalars (max_seq_len, max_blocks_per_req) stay at their bucket
+bounds (crates/warp34-host/src/model/graph_io.rs, tests/tq4_vision_and_moe.rs:1580-1603).  The
+library must therefore be capturable (no synchronisation, no allocation, no memset node) and a
+replay must give what an eager call on the same device state gives, bit for bit.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle
+from cases import make_case
+from oracle import DT_BF16, FMT_TQ4
+
+pytestmark = pytest.mark.gpu
+
+
+def test_decode_step_replays_with_growing_sequences():
+    import torch
+
+    import gpu_harness as G
+    from warp34_amd import ffi
+
+    lib = G.lib()
+    bs, q_heads, kv_heads = 64, 16, 2
+    seq0 = [700, 65, 1290]
+    steps = 4
+    # pool with room for the tokens the replays append
+    pool, bt, k, v, _, _, _ = make_case(FMT_TQ4, bs, [s + steps for s in seq0], [1, 1, 1], 501, DT_BF16,
+                                        kv_heads=kv_heads, q_heads=q_heads)
+    R = len(seq0)
+    # start from pools that hold only the first seq0 tokens: rebuild by writing a fresh pool
+    host = oracle.HostPool(pool.num_pages, kv_heads, 256, bs, FMT_TQ4, oracle.XF_WHT256)
+    starts = np.concatenate([[0], np.cumsum([s + steps for s in seq0])])
+    for r, s in enumerate(seq0):
+        wb = oracle.HostBatch([0, s], [s], bt[r:r + 1], context_lens_before=[0],
+                              write_slot_mapping=oracle.slot_mapping(bt[r], 0, s, bs))
+        oracle.kv_cache_write(host, wb, k[starts[r]:starts[r] + s], v[starts[r]:starts[r] + s], DT_BF16)
+    dpool = G.DevPool(host)
+    dpool.upload()
+    L = dpool.layout()
+
+    # device-side state of the captured step
+    qsl = G.to_dev(np.arange(R + 1, dtype=np.int32))
+    seq = G.to_dev(np.array(seq0, dtype=np.int32))
+    ctx = G.to_dev(np.array(seq0, dtype=np.int32))
+    slots = G.to_dev(np.zeros(R, dtype=np.int32))
+    btd = G.to_dev(bt)
+    k_in = torch.zeros((R, kv_heads, 256), dtype=torch.int16, device=G.DEV)
+    v_in = torch.zeros_like(k_in)
+    q_in = torch.zeros((R, q_heads, 256), dtype=torch.int16, device=G.DEV)
+    out = torch.zeros_like(q_in)
+    scratch = torch.zeros(16 << 20, dtype=torch.uint8, device=G.DEV)
+    bound = 4096  # graph bucket: an upper bound on every sequence length
+
+    def batch():
+        return ffi.Warp34AttentionBatch(qsl.data_ptr(), ctx.data_ptr(), seq.data_ptr(), btd.data_ptr(), slots.data_ptr(),
+                                        None, None, R, R, bt.shape[1], 1, bound, 0, 0, 0.0625, 0)
+
+    def step_calls():
+        ex = ffi.Warp34Exec(torch.cuda.current_stream().cuda_stream, scratch.data_ptr(), scratch.numel(), 0)
+        b = batch()
+        rc = lib.warp34_kv_cache_write_bf16(C.byref(ex), C.byref(L), C.byref(b), C.c_void_p(k_in.data_ptr()),
+                                            C.c_void_p(v_in.data_ptr()))
+        assert rc == 0
+        rc = lib.warp34_paged_attention_bf16(C.byref(ex), C.byref(L), C.byref(b), C.c_void_p(q_in.data_ptr()),
+                                             C.c_void_p(out.data_ptr()), q_heads)
+        assert rc == 0
+
+    def set_state(t):
+        """Device state of decode step t: each request appends its token seq0 + t."""
+        cur = np.array([s + t for s in seq0], dtype=np.int32)
+        ctx.copy_(G.to_dev(cur))
+        seq.copy_(G.to_dev(cur + 1))
+        slots.copy_(G.to_dev(np.array([oracle.slot_mapping(bt[r], int(cur[r]), 1, bs)[0] for r in range(R)],
+                                      dtype=np.int32)))
+        rows = [starts[r] + int(cur[r]) for r in range(R)]
+        k_in.copy_(G.to_dev(k[rows]))
+        v_in.copy_(G.to_dev(v[rows]))
+        q_in.copy_(G.to_dev(oracle.fill_normal(R * q_heads * 256, 600 + t, DT_BF16).reshape(R, q_heads, 256)))
+
+    # eager warm-up (configures the kernels' dynamic LDS once), on a scratch copy of the pools
+    snap_k, snap_v = dpool.k.clone(), dpool.v.clone()
+    set_state(0)
+    step_calls()
+    torch.cuda.synchronize()
+    dpool.k.copy_(snap_k)
+    dpool.v.copy_(snap_v)
+
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        step_calls()
+    dpool.k.copy_(snap_k)  # capture does not execute, but keep the state explicit
+    dpool.v.copy_(snap_v)
+
+    for t in range(steps):
+        set_state(t)
+        before_k, before_v = dpool.k.clone(), dpool.v.clone()
+        g.replay()
+        torch.cuda.synchronize()
+        got = out.cpu().numpy().view(np.uint16).copy()
+        after_k, after_v = dpool.k.clone(), dpool.v.clone()
+        # the same step eagerly from the same starting state
+        dpool.k.copy_(before_k)
+        dpool.v.copy_(before_v)
+        out.zero_()
+        step_calls()
+        torch.cuda.synchronize()
+        want = out.cpu().numpy().view(np.uint16)
+        assert torch.equal(dpool.k, after_k) and torch.equal(dpool.v, after_v), "replay %d: pool bytes differ" % t
+        assert got.tobytes() == want.tobytes(), "replay %d: attention output differs from the eager call" % t
+        # and against the oracle on the downloaded pool
+        hk, hv = dpool.download()
+        host.k[:] = hk
+        host.v[:] = hv
+        cur = [s + t for s in seq0]
+        hb = oracle.HostBatch(np.arange(R + 1), [c + 1 for c in cur], bt, context_lens_before=cur)
+        ref = oracle.paged_attention(host, hb, q_in.cpu().numpy().view(np.uint16), DT_BF16, q_heads, n_threads=4)
+        G.assert_close(got, DT_BF16, ref, what="replay %d vs oracle" % t)

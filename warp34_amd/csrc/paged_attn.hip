@@ -400,9 +400,14 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
         q_rot[c][1] = TQ::to_f32((uint16_t)(q_raw[c].x >> 16));
         q_rot[c][2] = TQ::to_f32((uint16_t)(q_raw[c].y & 0xFFFFu));
         q_rot[c][3] = TQ::to_f32((uint16_t)(q_raw[c].y >> 16));
+        // columns of tokens beyond the tile (every second column of a one-token decode tile)
+        // are stored as zeros below: no need to rotate them (wave-uniform branch)
+        const int col = wave + c * kWaves;
+        if (col < 16 * NT && fast_div(col, P.q_group) < rq_end - tok0) {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) q_rot[c][k] = apply_sign(q_rot[c][k], 4 * lane + k);
-        wht256_wave(q_rot[c], lane);
+            for (int k = 0; k < 4; ++k) q_rot[c][k] = apply_sign(q_rot[c][k], 4 * lane + k);
+            wht256_wave(q_rot[c], lane);
+        }
     }
 
     W34_TP(47);
