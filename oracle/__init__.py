@@ -13,7 +13,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libtq4_oracle.so")
 
-FMT_FP16, FMT_BF16, FMT_TQ4 = 0, 1, 2
+FMT_FP16, FMT_BF16, FMT_TQ4, FMT_Q8_0, FMT_FP8 = 0, 1, 2, 3, 4
 XF_IDENTITY, XF_WHT256 = 0, 1
 DT_F16, DT_BF16 = 0, 1
 
@@ -71,6 +71,12 @@ def lib():
         L.tq4o_wht256.argtypes = [C.c_void_p]
         L.tq4o_encode_row.argtypes = [C.c_void_p, C.c_void_p]
         L.tq4o_dequant_row.argtypes = [C.c_void_p, C.c_void_p]
+        for name in ("tq4o_encode_row_fp8", "tq4o_encode_row_q8", "tq4o_dequant_row_fp8", "tq4o_dequant_row_q8"):
+            getattr(L, name).argtypes = [C.c_void_p, C.c_void_p]
+        L.tq4o_f32_to_e4m3.restype = C.c_uint8
+        L.tq4o_f32_to_e4m3.argtypes = [C.c_float]
+        L.tq4o_e4m3_to_f32.restype = C.c_float
+        L.tq4o_e4m3_to_f32.argtypes = [C.c_uint8]
         L.tq4o_unrotate_row.argtypes = [C.c_void_p, C.c_void_p]
         L.tq4o_kv_cache_write.restype = C.c_int
         L.tq4o_kv_cache_write.argtypes = [C.POINTER(Layout), C.POINTER(Batch), C.c_void_p, C.c_void_p,
@@ -120,6 +126,32 @@ def encode_row(x):
     out = np.zeros(132, dtype=np.uint8)
     lib().tq4o_encode_row(x.ctypes.data, out.ctypes.data)
     return out
+
+
+def encode_row_fmt(x, fmt):
+    """256 fp32 values (already transformed) -> one stored row of an 8-bit format."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    assert x.shape == (256,)
+    out = np.zeros(row_bytes(fmt, 256), dtype=np.uint8)
+    fn = lib().tq4o_encode_row_fp8 if fmt == FMT_FP8 else lib().tq4o_encode_row_q8
+    fn(x.ctypes.data, out.ctypes.data)
+    return out
+
+
+def dequant_row_fmt(row, fmt):
+    row = np.ascontiguousarray(row, dtype=np.uint8)
+    out = np.zeros(256, dtype=np.float32)
+    fn = lib().tq4o_dequant_row_fp8 if fmt == FMT_FP8 else lib().tq4o_dequant_row_q8
+    fn(row.ctypes.data, out.ctypes.data)
+    return out
+
+
+def f32_to_e4m3(f):
+    return int(lib().tq4o_f32_to_e4m3(float(f)))
+
+
+def e4m3_to_f32(c):
+    return float(lib().tq4o_e4m3_to_f32(int(c)))
 
 
 def dequant_row(row):
@@ -195,6 +227,10 @@ def row_bytes(fmt, head_dim):
         return head_dim * 2
     if fmt == FMT_TQ4:
         return 66 * (head_dim // 128)
+    if fmt == FMT_Q8_0:
+        return 68 * (head_dim // 64)
+    if fmt == FMT_FP8:
+        return head_dim + 4 * (head_dim // 128)
     raise ValueError(fmt)
 
 

@@ -195,6 +195,77 @@ void tq4o_dequant_row(const uint8_t* src, float* y) {
     }
 }
 
+/* ---- OCP FP8 E4M3: sign, 4 exponent bits (bias 7), 3 mantissa bits; no infinities, 0x7f/0xff
+ * are NaN, largest finite 448 (0x7e) ---- */
+float tq4o_e4m3_to_f32(uint8_t c) {
+    const int e = (c >> 3) & 15, m = c & 7;
+    float v;
+    if (e == 15 && m == 7) return u2f(0x7fc00000u);
+    if (e == 0) v = (float)m * 0.001953125f;                    /* m * 2^-9 */
+    else v = u2f((uint32_t)(e - 7 + 127) << 23 | (uint32_t)m << 20);
+    return (c & 0x80) ? -v : v;
+}
+
+uint8_t tq4o_f32_to_e4m3(float f) {
+    const uint32_t u = f2u(f);
+    const uint8_t sign = (uint8_t)((u >> 24) & 0x80);
+    const uint32_t ax = u & 0x7fffffffu;
+    if (ax > 0x7f800000u) return (uint8_t)(sign | 0x7f);        /* NaN */
+    const float a = u2f(ax);
+    if (a >= 448.0f) return (uint8_t)(sign | 0x7e);             /* saturate (also +-inf) */
+    if (a < 0.015625f) {                                        /* below 2^-6: multiples of 2^-9 */
+        const float q = rintf(a * 512.0f);                      /* exact product, ties to even */
+        return (uint8_t)(sign | (uint8_t)q);                    /* 8 == 0x08 == 2^-6 */
+    }
+    /* normal: keep 3 mantissa bits, round the other 20 to nearest even */
+    uint32_t r = ax + 0x7ffffu + ((ax >> 20) & 1u);
+    r >>= 20;                                                   /* exponent (8 bits) and 3 mantissa bits */
+    const int code = (int)r - ((127 - 7) << 3);
+    return (uint8_t)(sign | (uint8_t)(code > 0x7e ? 0x7e : code));
+}
+
+void tq4o_encode_row_fp8(const float* x, uint8_t* dst) {
+    for (int h = 0; h < 2; ++h) {
+        float amax = 0.0f;
+        for (int c = 0; c < 128; ++c) amax = fmaxf(amax, fabsf(x[128 * h + c]));
+        const float d = amax * (1.0f / 448.0f);
+        const float inv_d = (d > 1e-30f) ? (1.0f / d) : 0.0f;
+        memcpy(dst + 256 + 4 * h, &d, 4);
+        for (int c = 0; c < 128; ++c) dst[128 * h + c] = tq4o_f32_to_e4m3(x[128 * h + c] * inv_d);
+    }
+}
+
+void tq4o_dequant_row_fp8(const uint8_t* src, float* y) {
+    for (int h = 0; h < 2; ++h) {
+        float d;
+        memcpy(&d, src + 256 + 4 * h, 4);
+        for (int c = 0; c < 128; ++c) y[128 * h + c] = d * tq4o_e4m3_to_f32(src[128 * h + c]);
+    }
+}
+
+void tq4o_encode_row_q8(const float* x, uint8_t* dst) {
+    for (int sb = 0; sb < 4; ++sb) {
+        float amax = 0.0f;
+        for (int c = 0; c < 64; ++c) amax = fmaxf(amax, fabsf(x[64 * sb + c]));
+        const float d = amax / 127.0f;
+        const float inv_d = (d > 1e-12f) ? (1.0f / d) : 0.0f;
+        memcpy(dst + 68 * sb, &d, 4);
+        for (int c = 0; c < 64; ++c) {
+            float q = roundf(x[64 * sb + c] * inv_d);           /* half away from zero */
+            q = fminf(127.0f, fmaxf(-127.0f, q));
+            dst[68 * sb + 4 + c] = (uint8_t)(int8_t)q;
+        }
+    }
+}
+
+void tq4o_dequant_row_q8(const uint8_t* src, float* y) {
+    for (int sb = 0; sb < 4; ++sb) {
+        float d;
+        memcpy(&d, src + 68 * sb, 4);
+        for (int c = 0; c < 64; ++c) y[64 * sb + c] = d * (float)(int8_t)src[68 * sb + 4 + c];
+    }
+}
+
 void tq4o_unrotate_row(const float* y, float* x) {
     const float* sg = tq4o_signs256();
     float t[256];
@@ -238,6 +309,18 @@ static int write_row(uint8_t* dst, int format, int transform, const uint16_t* sr
         tq4o_encode_row(x, dst);
         return 0;
     }
+    if ((format == TQ4O_FMT_Q8_0 || format == TQ4O_FMT_FP8) && head_dim == 256) {
+        float x[256];
+        for (int c = 0; c < 256; ++c) x[c] = load16(src + c, in_dtype);
+        if (transform == TQ4O_XF_WHT256) { /* op_kv_cache.cu:39-45,68-74: sign diagonal, then WHT */
+            const float* sg = tq4o_signs256();
+            for (int c = 0; c < 256; ++c) x[c] *= sg[c];
+            tq4o_wht256(x);
+        }
+        if (format == TQ4O_FMT_FP8) tq4o_encode_row_fp8(x, dst);
+        else tq4o_encode_row_q8(x, dst);
+        return 0;
+    }
     return -1;
 }
 
@@ -272,6 +355,14 @@ int tq4o_kv_cache_write(const tq4o_layout* L, const tq4o_batch* B, const uint16_
 static void read_row(const uint8_t* row, int format, int head_dim, float* y) {
     if (format == TQ4O_FMT_TQ4) {
         tq4o_dequant_row(row, y);
+        return;
+    }
+    if (format == TQ4O_FMT_FP8) { /* op_paged_attn.cu:73-103 */
+        tq4o_dequant_row_fp8(row, y);
+        return;
+    }
+    if (format == TQ4O_FMT_Q8_0) { /* op_paged_attn.cu:59-71 */
+        tq4o_dequant_row_q8(row, y);
         return;
     }
     const uint16_t* p = (const uint16_t*)row;

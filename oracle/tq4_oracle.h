@@ -30,6 +30,11 @@
  *   tq4o_attention    closed forms (Q=K=0 -> running mean of V, single key -> that V row),
  *                     brute-force fp64 softmax over independently dequantised rows
  *   tq4o_split_merge  equality with the single-pass result
+ *   fp8 e4m3 / q8_0   conversion: brute force over all 256 codes (nearest finite code, ties to
+ *                     the even code, saturation at 448); rows: scale = amax / 448 (amax / 127),
+ *                     round trip error bounds, layout pins (264 B: codes then two fp32 scales;
+ *                     272 B: four {fp32 scale, 64 int8}) -- exact BYTES for general inputs are
+ *                     pinned by no reference-held vector: "parity unpinned" beyond that
  */
 #ifndef TQ4_ORACLE_H
 #define TQ4_ORACLE_H
@@ -41,7 +46,7 @@
 extern "C" {
 #endif
 
-enum { TQ4O_FMT_FP16 = 0, TQ4O_FMT_BF16 = 1, TQ4O_FMT_TQ4 = 2 };
+enum { TQ4O_FMT_FP16 = 0, TQ4O_FMT_BF16 = 1, TQ4O_FMT_TQ4 = 2, TQ4O_FMT_Q8_0 = 3, TQ4O_FMT_FP8 = 4 };
 enum { TQ4O_XF_IDENTITY = 0, TQ4O_XF_WHT256 = 1 };
 enum { TQ4O_DT_F16 = 0, TQ4O_DT_BF16 = 1 };
 
@@ -86,6 +91,21 @@ void tq4o_wht256(float* x);
 /* --- op_kv_cache.cu:152-218 : quantize one 256-wide row (fp32 values of the fp16/bf16
  * source) into 132 bytes --- */
 void tq4o_encode_row(const float* x, uint8_t* dst132);
+
+/* OCP FP8 E4M3 (finite-only, max 448) <-> fp32: round to nearest even, saturating
+ * (__nv_cvt_float2_to_fp8x2(.., __NV_SATFINITE, __NV_E4M3) in op_kv_cache.cu:83-86). */
+uint8_t tq4o_f32_to_e4m3(float f);
+float tq4o_e4m3_to_f32(uint8_t c);
+
+/* 8-bit rows of a 256-wide head (x already transformed if the layer rotates):
+ *   fp8:  264 B = 256 e4m3 codes, then fp32 d0 (elements 0..127) and d1 (128..255);
+ *         d = amax / 448, code = e4m3(x / d)                  (op_kv_cache.cu:64-140)
+ *   q8_0: 272 B = 4 x {fp32 d, 64 int8}; d = amax / 127, q = clamp(roundf(x / d), +-127)
+ *                                                             (op_kv_cache.cu:32-62) */
+void tq4o_encode_row_fp8(const float* x, uint8_t* dst);
+void tq4o_encode_row_q8(const float* x, uint8_t* dst);
+void tq4o_dequant_row_fp8(const uint8_t* src, float* y);
+void tq4o_dequant_row_q8(const uint8_t* src, float* y);
 
 /* --- op_kv_cache.cu:298-306 : dequantise one 132-byte row into the ROTATED domain --- */
 void tq4o_dequant_row(const uint8_t* src132, float* y);

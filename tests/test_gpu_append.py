@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 
 import oracle
-from oracle import DT_BF16, DT_F16, FMT_BF16, FMT_FP16, FMT_TQ4, XF_IDENTITY, XF_WHT256
+from oracle import DT_BF16, DT_F16, FMT_BF16, FMT_FP8, FMT_FP16, FMT_Q8_0, FMT_TQ4, XF_IDENTITY, XF_WHT256
 
 pytestmark = pytest.mark.gpu
 
@@ -113,6 +113,53 @@ def test_tq4_strided_source_bf16():
     assert gk.tobytes() == hpool.k.tobytes() and gv.tobytes() == hpool.v.tobytes()
 
 
+@pytest.mark.parametrize("fmt", [FMT_FP8, FMT_Q8_0])
+@pytest.mark.parametrize("xf", [XF_IDENTITY, XF_WHT256])
+@pytest.mark.parametrize("in_dtype", [DT_BF16, DT_F16])
+def test_8bit_formats_append_bit_exact(fmt, xf, in_dtype):
+    """FP8-E4M3 (264-byte) and Q8_0 (272-byte) rows, un-rotated as the default policy's tail layers
+    store them and rotated (op_kv_cache.cu:32-140); 1 % outlier channels, ragged last page."""
+    hpool, gk, gv = _run_append(fmt, xf, 64, 1000, in_dtype, seed=11)
+    assert hpool.tok == (264 if fmt == FMT_FP8 else 272)
+    assert gk.tobytes() == hpool.k.tobytes() and gv.tobytes() == hpool.v.tobytes()
+    assert gk.any()
+
+
+@pytest.mark.parametrize("fmt", [FMT_FP8, FMT_Q8_0])
+def test_8bit_formats_special_rows_masks_and_strided_source(fmt):
+    """Zero rows (d = 0 -> codes 0), rows below the scale thresholds, saturating rows, a source
+    whose row stride breaks the 16-byte alignment of the vector load, masks and negative slots."""
+    import gpu_harness as G
+
+    n = 8
+    k = np.zeros((n, 2, 256), dtype=np.float32)
+    rng = np.random.default_rng(1)
+    k[1] = rng.standard_normal((2, 256)) * 1e-12
+    k[2] = rng.standard_normal((2, 256)) * 3e4
+    k[3, :, 7] = 1.0
+    k[4] = 1.0
+    k[5] = rng.standard_normal((2, 256)) * 1e-30
+    k[6] = -rng.random((2, 256))
+    k[7, :, :128] = rng.standard_normal((2, 128)) * 100.0
+    for dt, to_bits in ((DT_BF16, oracle.f32_to_bf16_bits), (DT_F16, lambda a: np.clip(a, -6e4, 6e4).astype(np.float16).view(np.uint16))):
+        kb = to_bits(k)
+        vb = kb[::-1].copy()
+        hpool = oracle.HostPool(2, 2, 256, 16, fmt, XF_IDENTITY)
+        hb = oracle.HostBatch([0, n], [n], np.array([[1, 0]], np.int32), context_lens_before=[0],
+                              write_slot_mapping=oracle.slot_mapping([1, 0], 0, n, 16))
+        oracle.kv_cache_write(hpool, hb, kb, vb, dt)
+        dpool = G.DevPool(hpool)
+        assert G.dev_write(dpool, hb, kb, vb, dt) == 0
+        gk, gv = dpool.download()
+        assert gk.tobytes() == hpool.k.tobytes() and gv.tobytes() == hpool.v.tobytes()
+    hpool, gk, gv = _run_append(fmt, XF_IDENTITY, 16, 50, DT_F16, seed=13, stride=2 * 256 + 4)
+    assert gk.tobytes() == hpool.k.tobytes() and gv.tobytes() == hpool.v.tobytes()
+    tmask = np.ones(24, np.uint8)
+    tmask[[2, 17]] = 0
+    hpool, gk, gv = _run_append(fmt, XF_IDENTITY, 16, 24, DT_BF16, seed=15, tmask=tmask, neg_slots=(0, 9))
+    assert gk.tobytes() == hpool.k.tobytes() and gv.tobytes() == hpool.v.tobytes()
+
+
 def test_write_argument_validation():
     """Error convention of op_kv_cache.cu:836-845,1174-1177."""
     import gpu_harness as G
@@ -134,8 +181,17 @@ def test_write_argument_validation():
     assert l.warp34_kv_cache_write_strided(C.byref(ex), C.byref(L), C.byref(B), G.ptr(k), G.ptr(k), 511, 512) == inval
     B0 = db.struct(total_tokens=0)
     assert l.warp34_kv_cache_write(C.byref(ex), C.byref(L), C.byref(B0), G.ptr(k), G.ptr(k)) == 0
+    # FP8 needs head_dim 256 (op_kv_cache.cu:839-842); 8-bit rows carry fp32 scales: 4-byte aligned
     Lf8 = dpool.layout(fmt=ffi.WARP34_KV_FORMAT_FP8_E4M3)
-    assert l.warp34_kv_cache_write(C.byref(ex), C.byref(Lf8), C.byref(B), G.ptr(k), G.ptr(k)) == nosup
+    Lf8.head_dim = 128
+    assert l.warp34_kv_cache_write(C.byref(ex), C.byref(Lf8), C.byref(B), G.ptr(k), G.ptr(k)) == inval
+    Lf8 = dpool.layout(fmt=ffi.WARP34_KV_FORMAT_FP8_E4M3)
+    Lf8.k_token_stride_bytes = 266
+    assert l.warp34_kv_cache_write(C.byref(ex), C.byref(Lf8), C.byref(B), G.ptr(k), G.ptr(k)) == inval
+    # a TQ4 row needs the WHT256 transform
+    Lt = dpool.layout()
+    Lt.k_transform = ffi.WARP34_KV_TRANSFORM_IDENTITY
+    assert l.warp34_kv_cache_write(C.byref(ex), C.byref(Lt), C.byref(B), G.ptr(k), G.ptr(k)) == nosup
     # bf16 entry points: FP16 storage is rejected like in the reference
     Lh = dpool.layout(fmt=ffi.WARP34_KV_FORMAT_FP16)
     assert l.warp34_kv_cache_write_bf16(C.byref(ex), C.byref(Lh), C.byref(B), G.ptr(k), G.ptr(k)) == inval

@@ -129,6 +129,119 @@ __device__ __forceinline__ void tq4_encode_row(float (&v)[8], int lane, uint8_t*
     }
 }
 
+// fp32 -> OCP FP8 E4M3, round to nearest even, saturating at +-448, NaN -> 0x7f
+// (__nv_cvt_float2_to_fp8x2(.., __NV_SATFINITE, __NV_E4M3) in op_kv_cache.cu:83-86).  Integer
+// arithmetic, so the bits do not depend on a hardware conversion mode.
+__device__ __forceinline__ uint32_t f32_to_e4m3(float f) {
+    const uint32_t u = __float_as_uint(f);
+    const uint32_t sign = (u >> 24) & 0x80u;
+    const uint32_t ax = u & 0x7fffffffu;
+    if (ax > 0x7f800000u) return sign | 0x7fu;
+    const float a = __uint_as_float(ax);
+    if (a >= 448.0f) return sign | 0x7eu;
+    if (a < 0.015625f) return sign | (uint32_t)rintf(a * 512.0f);  // multiples of 2^-9
+    uint32_t r = (ax + 0x7ffffu + ((ax >> 20) & 1u)) >> 20;
+    r -= (127u - 7u) << 3;
+    return sign | (r > 0x7eu ? 0x7eu : r);
+}
+
+// 8-bit rows of a 256-wide head, identity transform; lane l32 holds elements 8 l32 .. 8 l32 + 7.
+//   FP8:  264 B = 256 codes, then fp32 d0 (elements 0..127) and d1; d = amax / 448
+//         (op_kv_cache.cu:104-138)
+//   Q8_0: 272 B = 4 x {fp32 d, 64 int8}; d = amax / 127, q = clamp(roundf(x / d))
+//         (op_kv_cache.cu:32-62)
+// max() is exact and order-free, so only the element-wise arithmetic has to follow the source.
+__device__ __forceinline__ void fp8_encode_row(const float (&v)[8], int lane, uint8_t* row) {
+    const int l32 = lane & 31;
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
+    amax = fmaxf(amax, lane_xor<8>(amax, lane));
+    amax = fmaxf(amax, lane_xor<4>(amax, lane));
+    amax = fmaxf(amax, lane_xor<2>(amax, lane));
+    amax = fmaxf(amax, lane_xor<1>(amax, lane));
+    const float d = amax * (1.0f / 448.0f);
+    const float inv_d = (d > 1e-30f) ? (1.0f / d) : 0.0f;
+    uint32_t w0 = 0, w1 = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        w0 |= f32_to_e4m3(v[j] * inv_d) << (8 * j);
+        w1 |= f32_to_e4m3(v[4 + j] * inv_d) << (8 * j);
+    }
+    *reinterpret_cast<uint2*>(row + 8 * l32) = uint2{w0, w1};
+    if ((l32 & 15) == 0) *reinterpret_cast<float*>(row + 256 + 4 * (l32 >> 4)) = d;
+}
+
+__device__ __forceinline__ void q8_encode_row(const float (&v)[8], int lane, uint8_t* row) {
+    const int l32 = lane & 31;
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
+    amax = fmaxf(amax, lane_xor<4>(amax, lane));
+    amax = fmaxf(amax, lane_xor<2>(amax, lane));
+    amax = fmaxf(amax, lane_xor<1>(amax, lane));
+    const float d = amax / 127.0f;
+    const float inv_d = (d > 1e-12f) ? (1.0f / d) : 0.0f;
+    uint32_t w0 = 0, w1 = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float q0 = fminf(127.0f, fmaxf(-127.0f, roundf(v[j] * inv_d)));
+        const float q1 = fminf(127.0f, fmaxf(-127.0f, roundf(v[4 + j] * inv_d)));
+        w0 |= ((uint32_t)(int)q0 & 0xffu) << (8 * j);
+        w1 |= ((uint32_t)(int)q1 & 0xffu) << (8 * j);
+    }
+    uint8_t* blk = row + 68 * (l32 >> 3);
+    *reinterpret_cast<uint32_t*>(blk + 4 + 8 * (l32 & 7)) = w0;
+    *reinterpret_cast<uint32_t*>(blk + 8 + 8 * (l32 & 7)) = w1;
+    if ((l32 & 7) == 0) *reinterpret_cast<float*>(blk) = d;
+}
+
+// The same two rows from the rotated layout v[j] = y[l32 + 32 j] (y = WHT256(sign * x)), used when
+// an 8-bit layer asks for the WHT256 transform (op_kv_cache.cu:36-44,71-99).
+__device__ __forceinline__ float half_wave_max(float v, int lane) {
+    v = fmaxf(v, lane_xor<16>(v, lane));
+    v = fmaxf(v, lane_xor<8>(v, lane));
+    v = fmaxf(v, lane_xor<4>(v, lane));
+    v = fmaxf(v, lane_xor<2>(v, lane));
+    v = fmaxf(v, lane_xor<1>(v, lane));
+    return v;
+}
+
+__device__ __forceinline__ void fp8_encode_row_rotated(const float (&v)[8], int lane, uint8_t* row) {
+    const int l32 = lane & 31;
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        float amax = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) amax = fmaxf(amax, fabsf(v[4 * b + j]));
+        amax = half_wave_max(amax, lane);
+        const float d = amax * (1.0f / 448.0f);
+        const float inv_d = (d > 1e-30f) ? (1.0f / d) : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            row[l32 + 32 * (4 * b + j)] = (uint8_t)f32_to_e4m3(v[4 * b + j] * inv_d);
+        }
+        if (l32 == 0) *reinterpret_cast<float*>(row + 256 + 4 * b) = d;
+    }
+}
+
+__device__ __forceinline__ void q8_encode_row_rotated(const float (&v)[8], int lane, uint8_t* row) {
+    const int l32 = lane & 31;
+#pragma unroll
+    for (int sb = 0; sb < 4; ++sb) {
+        const float x0 = v[2 * sb], x1 = v[2 * sb + 1];
+        const float amax = half_wave_max(fmaxf(fabsf(x0), fabsf(x1)), lane);
+        const float d = amax / 127.0f;
+        const float inv_d = (d > 1e-12f) ? (1.0f / d) : 0.0f;
+        const float q0 = fminf(127.0f, fmaxf(-127.0f, roundf(x0 * inv_d)));
+        const float q1 = fminf(127.0f, fmaxf(-127.0f, roundf(x1 * inv_d)));
+        uint8_t* blk = row + 68 * sb;
+        blk[4 + l32] = (uint8_t)(int)q0;
+        blk[4 + 32 + l32] = (uint8_t)(int)q1;
+        if (l32 == 0) *reinterpret_cast<float*>(blk) = d;
+    }
+}
+
 // One wave per (token, kv head); lanes 0-31 write K, lanes 32-63 write V.
 template <typename TIn>
 __global__ __launch_bounds__(256) void kv_append_kernel(warp34_kv_layer_layout L,
@@ -165,6 +278,51 @@ __global__ __launch_bounds__(256) void kv_append_kernel(warp34_kv_layer_layout L
                           (size_t)tok * (size_t)(is_v ? v_row_stride : k_row_stride) +
                           (size_t)head * (size_t)L.head_dim;
 
+    __shared__ __align__(8) uint8_t rows[4][2][272];
+    if (format == WARP34_KV_FORMAT_FP8_E4M3 || format == WARP34_KV_FORMAT_Q8_0) {
+        // host side guarantees head_dim == 256 and 4-byte aligned rows
+        float v[8];
+        uint8_t* row = rows[wave][is_v];
+        const int n_dwords = format == WARP34_KV_FORMAT_FP8_E4M3 ? 66 : 68;
+        const uint16_t* src8 = src + 8 * l32;
+        if ((is_v ? L.v_transform : L.k_transform) == WARP34_KV_TRANSFORM_RADEMACHER_WHT256) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = apply_sign(TIn::to_f32(src[l32 + 32 * j]), l32 + 32 * j);
+            wht256_half_wave(v, lane);
+            if (format == WARP34_KV_FORMAT_FP8_E4M3) {
+                fp8_encode_row_rotated(v, lane, row);
+            } else {
+                q8_encode_row_rotated(v, lane, row);
+            }
+        } else {
+        if ((reinterpret_cast<uintptr_t>(src8) & 15u) == 0) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(src8);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v[2 * j] = TIn::to_f32((uint16_t)(w[j] & 0xffffu));
+                v[2 * j + 1] = TIn::to_f32((uint16_t)(w[j] >> 16));
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = TIn::to_f32(src8[j]);
+        }
+        if (format == WARP34_KV_FORMAT_FP8_E4M3) {
+            fp8_encode_row(v, lane, row);
+        } else {
+            q8_encode_row(v, lane, row);
+        }
+        }
+        __atomic_signal_fence(__ATOMIC_SEQ_CST);
+        __builtin_amdgcn_wave_barrier();
+        __atomic_signal_fence(__ATOMIC_SEQ_CST);
+        const uint32_t* r32 = reinterpret_cast<const uint32_t*>(row);
+        uint32_t* d32 = reinterpret_cast<uint32_t*>(dst);
+        d32[l32] = r32[l32];
+        d32[l32 + 32] = r32[l32 + 32];
+        if (l32 + 64 < n_dwords) d32[l32 + 64] = r32[l32 + 64];
+        return;
+    }
     if (format == WARP34_KV_FORMAT_TQ4) {
         // host side guarantees head_dim == 256 and the WHT256 transform for TQ4
         float v[8];
@@ -172,7 +330,6 @@ __global__ __launch_bounds__(256) void kv_append_kernel(warp34_kv_layer_layout L
         for (int j = 0; j < 8; ++j) v[j] = TIn::to_f32(src[l32 + 32 * j]);
         // the row is assembled in LDS and leaves with one 32-bit store per lane (16-bit stores
         // when the destination is only 2-byte aligned, which is all the row format promises)
-        __shared__ __align__(4) uint8_t rows[4][2][136];
         uint8_t* row = rows[wave][is_v];
         tq4_encode_row(v, lane, row);
         __atomic_signal_fence(__ATOMIC_SEQ_CST);
@@ -214,7 +371,31 @@ static bool format_supported_for_write(int format, int transform, int head_dim) 
     if (format == WARP34_KV_FORMAT_TQ4) {
         return head_dim == 256 && transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256;
     }
+    if (format == WARP34_KV_FORMAT_Q8_0 || format == WARP34_KV_FORMAT_FP8_E4M3) {
+        // the tail-anchor layers of the default policy store these un-rotated (cache.rs:87-109);
+        // the rotated variant is what op_kv_cache.cu:36-44,71-99 accepts as well
+        return head_dim == 256 && (transform == WARP34_KV_TRANSFORM_IDENTITY ||
+                                   transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256);
+    }
     return false;
+}
+
+static bool is_8bit_format(int format) {
+    return format == WARP34_KV_FORMAT_Q8_0 || format == WARP34_KV_FORMAT_FP8_E4M3;
+}
+
+// Q8_0 and FP8 rows carry fp32 scales (alignof 4, tq4_kv_common.cuh:28-46) and are stored with
+// 32-bit stores.
+static bool rows_aligned_for_write(const warp34_kv_layer_layout* l) {
+    if (is_8bit_format(l->k_format) &&
+        ((l->k_base | l->k_page_stride_bytes | l->k_head_stride_bytes | l->k_token_stride_bytes) & 3u)) {
+        return false;
+    }
+    if (is_8bit_format(l->v_format) &&
+        ((l->v_base | l->v_page_stride_bytes | l->v_head_stride_bytes | l->v_token_stride_bytes) & 3u)) {
+        return false;
+    }
+    return true;
 }
 
 template <typename TIn>
@@ -245,8 +426,9 @@ extern "C" int warp34_kv_cache_write_strided(const warp34_exec* ex, const warp34
         return (int)hipErrorInvalidValue;
     }
     if (layout->k_format == WARP34_KV_FORMAT_FP8_E4M3 || layout->v_format == WARP34_KV_FORMAT_FP8_E4M3) {
+        // gfx950 always has the FP8 path (the reference gates it on the device generation,
+        // op_kv_cache.cu:839-842)
         if (layout->head_dim != 256) return (int)hipErrorInvalidValue;
-        return (int)hipErrorNotSupported;
     }
     if (batch->total_tokens <= 0 || layout->local_kv_heads <= 0) return 0;
     const int min_stride = layout->local_kv_heads * layout->head_dim;
@@ -259,6 +441,7 @@ extern "C" int warp34_kv_cache_write_strided(const warp34_exec* ex, const warp34
         !format_supported_for_write(layout->v_format, layout->v_transform, layout->head_dim)) {
         return (int)hipErrorNotSupported;
     }
+    if (!rows_aligned_for_write(layout)) return (int)hipErrorInvalidValue;
     return launch_append<F16>(ex, layout, batch, k_in, v_in, k_row_stride, v_row_stride);
 }
 
@@ -272,7 +455,7 @@ extern "C" int warp34_kv_cache_write(const warp34_exec* ex, const warp34_kv_laye
 }
 
 // Layouts the bf16 entry points accept: the reference's BF16 identity layout
-// (op_kv_cache.cu:860-865) plus TQ4 + WHT256 at head_dim 256.
+// (op_kv_cache.cu:860-865) plus, at head_dim 256, TQ4 + WHT256 and the 8-bit row formats.
 static bool valid_bf16_entry_layout(const warp34_kv_layer_layout* l) {
     if (!l || l->local_kv_heads <= 0 || l->block_size <= 0 || l->head_dim <= 0 || l->head_dim > 256 ||
         !l->k_base || !l->v_base) {
@@ -285,7 +468,11 @@ static bool valid_bf16_entry_layout(const warp34_kv_layer_layout* l) {
                      l->v_format == WARP34_KV_FORMAT_TQ4 &&
                      l->k_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 &&
                      l->v_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256;
-    return bf16 || tq4;
+    const bool q8 = l->head_dim == 256 && is_8bit_format(l->k_format) && is_8bit_format(l->v_format) &&
+                    format_supported_for_write(l->k_format, l->k_transform, 256) &&
+                    format_supported_for_write(l->v_format, l->v_transform, 256) &&
+                    rows_aligned_for_write(l);
+    return bf16 || tq4 || q8;
 }
 
 // op_kv_cache.cu:1172-1183

@@ -1027,8 +1027,12 @@ __global__ __launch_bounds__(1024) void split_merge_kernel(const float* part_acc
         const f4 r = s_rec[s];
         if (r[1] > 0.f) m_tot = fmaxf(m_tot, r[0]);
     }
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) m_tot = fmaxf(m_tot, __shfl_xor(m_tot, off, 64));
+    m_tot = fmaxf(m_tot, lane_xor<1>(m_tot, lane));
+    m_tot = fmaxf(m_tot, lane_xor<2>(m_tot, lane));
+    m_tot = fmaxf(m_tot, lane_xor<4>(m_tot, lane));
+    m_tot = fmaxf(m_tot, lane_xor<8>(m_tot, lane));
+    m_tot = fmaxf(m_tot, lane_xor<16>(m_tot, lane));
+    m_tot = fmaxf(m_tot, lane_xor<32>(m_tot, lane));
 
     f4 v = {0.f, 0.f, 0.f, 0.f};
     float l_part = 0.f;
