@@ -25,12 +25,15 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 KV_HEADS, Q_HEADS, HEAD_DIM, BLOCK = 2, 16, 256, 64
-ROW_BYTES = {"tq4": 132, "bf16": 512}
+ROW_BYTES = {"tq4": 132, "bf16": 512, "fp8": 264, "q8_0": 272}
 WORKLOADS = {
     # name: (kv format, context lengths or None for the seeded 32-sequence draw, pool tokens)
     "tq4_decode_b1_ctx131072": ("tq4", [131072], 0),
     "tq4_decode_b32_ctx1k_64k": ("tq4", None, 2 << 20),
     "bf16_decode_b1_ctx32768": ("bf16", [32768], 0),
+    # the un-rotated 8-bit rows the default TQ4 policy keeps for its last four layers
+    "fp8_decode_b1_ctx131072": ("fp8", [131072], 0),
+    "q8_0_decode_b1_ctx131072": ("q8_0", [131072], 0),
     # 8 sequences, 16 384-token TQ4 prefix + 2 048-token bf16 chunk each: append + causal attention
     "tq4_prefill_8x2048_ctx16384": ("tq4", [18432] * 8, 0),
     # 16 sequences of 262 144 tokens that share the pages of a 200 000-token prefix; 4 query tokens each
@@ -84,7 +87,8 @@ class Layer:
         self.page = KV_HEADS * self.head
         self.k = torch.zeros(pool_pages * self.page, dtype=torch.uint8, device=dev)
         self.v = torch.zeros(pool_pages * self.page, dtype=torch.uint8, device=dev)
-        kv_format = ffi.WARP34_KV_FORMAT_TQ4 if fmt == "tq4" else ffi.WARP34_KV_FORMAT_BF16
+        kv_format = {"tq4": ffi.WARP34_KV_FORMAT_TQ4, "bf16": ffi.WARP34_KV_FORMAT_BF16,
+                     "fp8": ffi.WARP34_KV_FORMAT_FP8_E4M3, "q8_0": ffi.WARP34_KV_FORMAT_Q8_0}[fmt]
         xf = ffi.WARP34_KV_TRANSFORM_RADEMACHER_WHT256 if fmt == "tq4" else ffi.WARP34_KV_TRANSFORM_IDENTITY
         self.layout = ffi.Warp34KvLayerLayout(
             self.k.data_ptr(), self.v.data_ptr(), self.page, self.head, self.tok, self.page, self.head, self.tok,
@@ -364,15 +368,17 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f16 MFMA operands (TQ4 codes -> fp16 centroids), f32 accumulate, bf16 Q/out" if fmt == "tq4"
-                 else "bf16 MFMA operands, f32 accumulate, bf16 Q/out",
+        "dtype": {"tq4": "f16 MFMA operands (TQ4 codes -> fp16 centroids), f32 accumulate, bf16 Q/out",
+                  "bf16": "bf16 MFMA operands, f32 accumulate, bf16 Q/out",
+                  "fp8": "f16 MFMA operands (E4M3 codes widened, fp32 block scales), f32 accumulate, bf16 Q/out",
+                  "q8_0": "f16 MFMA operands (int8 codes widened, fp32 block scales), f32 accumulate, bf16 Q/out"}[fmt],
         "data": "synthetic",
         "config": {
             "workload": args.workload,
             "requests": R, "query_tokens_per_request": ql, "shared_prefix_tokens": shared,
             "context_tokens_total": total_tokens_kv,
             "q_heads": Q_HEADS, "kv_heads": KV_HEADS, "head_dim": HEAD_DIM, "page_tokens": BLOCK,
-            "kv_format": "tq4+wht256" if fmt == "tq4" else "bf16", "kv_pools_cycled": n_layers,
+            "kv_format": "tq4+wht256" if fmt == "tq4" else fmt, "kv_pools_cycled": n_layers,
             "pool_pages": pool_pages,
             "kv_bytes_per_step": kv_bytes,
         },
@@ -384,7 +390,7 @@ def main():
             "frac": round(gbs / HBM_PEAK_GBS, 4),
             "traffic": MEASURED_TRAFFIC.get(args.workload),
             "kernel": "paged_attn_%s_kernel (+ split_merge_kernel, both inside the timed launch)"
-                      % ("tq4" if fmt == "tq4" else "kv16"),
+                      % ("tq4" if fmt == "tq4" else "rows"),
             "avg_launch_us": round(ms_per_step * 1e3, 3),
             "host_wall_us_per_step": round(t_wall / args.steps * 1e6, 2),
         },

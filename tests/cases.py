@@ -6,9 +6,10 @@ from oracle import FMT_TQ4, XF_IDENTITY, XF_WHT256
 
 
 def make_case(fmt, block_size, seq_lens, q_lens, seed, dtype, kv_heads=2, q_heads=8, perm_seed=5,
-              extra_pages=3):
+              extra_pages=3, xf=None):
     """Append seq_len tokens per request through the oracle's write, return everything."""
-    xf = XF_WHT256 if fmt == FMT_TQ4 else XF_IDENTITY
+    if xf is None:
+        xf = XF_WHT256 if fmt == FMT_TQ4 else XF_IDENTITY
     pages_per = [(s + block_size - 1) // block_size for s in seq_lens]
     num_pages = sum(pages_per) + extra_pages
     perm = oracle.permutation(num_pages, perm_seed)

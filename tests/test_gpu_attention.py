@@ -12,7 +12,7 @@ import pytest
 
 import oracle
 from cases import make_case
-from oracle import DT_BF16, DT_F16, FMT_BF16, FMT_FP16, FMT_TQ4
+from oracle import DT_BF16, DT_F16, FMT_BF16, FMT_FP8, FMT_FP16, FMT_Q8_0, FMT_TQ4, XF_IDENTITY, XF_WHT256
 
 pytestmark = pytest.mark.gpu
 
@@ -28,11 +28,11 @@ def _dev_pool(pool):
 
 
 def _check(fmt, dtype, block_size, seq_lens, q_lens, seed, scratch=SCRATCH, q_heads=8, kv_heads=2,
-           mask_mode=0, window=0, ctx_null=False, **kw):
+           mask_mode=0, window=0, ctx_null=False, xf=None, **kw):
     import gpu_harness as G
 
     pool, bt, k, v, q, aq, ctx = make_case(fmt, block_size, seq_lens, q_lens, seed, dtype, kv_heads=kv_heads,
-                                           q_heads=q_heads)
+                                           q_heads=q_heads, xf=xf)
     hb = oracle.HostBatch(aq, seq_lens, bt, context_lens_before=None if ctx_null else ctx, mask_mode=mask_mode,
                           sliding_window=window)
     want = oracle.paged_attention(pool, hb, q, dtype, q_heads, n_threads=4)
@@ -212,6 +212,74 @@ def test_kv16_mismatched_query_type_is_refused():
     dpool = _dev_pool(pool)
     rc, got, _ = G.dev_attention(dpool, hb, q, DT_F16, 8)
     assert rc == 801 and (got == 0x5500).all()
+
+
+# ---- 8-bit pages: FP8-E4M3-256 and Q8_0-64 rows (tail layers of the default TQ4 policy) ----
+
+KV8 = [FMT_FP8, FMT_Q8_0]
+
+
+@pytest.mark.parametrize("fmt", KV8)
+@pytest.mark.parametrize("dtype", [DT_F16, DT_BF16])
+@pytest.mark.parametrize("block_size", [16, 64])
+def test_kv8_decode_small_batch(fmt, dtype, block_size):
+    _check(fmt, dtype, block_size, [70, 33, 129, 1, 32], [1, 1, 1, 1, 1], 211)
+
+
+@pytest.mark.parametrize("fmt", KV8)
+@pytest.mark.parametrize("scratch", [0, SCRATCH])
+def test_kv8_decode_gqa8_long(fmt, scratch):
+    _check(fmt, DT_F16, 64, [5000], [1], 221, scratch=scratch, q_heads=16)
+
+
+@pytest.mark.parametrize("fmt", KV8)
+def test_kv8_decode_ctx32k(fmt):
+    _check(fmt, DT_BF16, 64, [32768], [1], 231, scratch=64 << 20, q_heads=16)
+
+
+@pytest.mark.parametrize("fmt", KV8)
+@pytest.mark.parametrize("q_lens", [[4, 4], [2, 3], [16]])
+def test_kv8_verify_multi_token_causal(fmt, q_lens):
+    seq = [300 + 7 * i for i in range(len(q_lens))]
+    _check(fmt, DT_F16, 64, seq, q_lens, 241, q_heads=16)
+    _check(fmt, DT_BF16, 16, seq, q_lens, 242, q_heads=8, scratch=0)
+
+
+@pytest.mark.parametrize("fmt", KV8)
+@pytest.mark.parametrize("mask_mode,window", [(0, 40), (1, 0), (1, 100), (0, 5)])
+def test_kv8_windows(fmt, mask_mode, window):
+    _check(fmt, DT_F16, 16, [333, 90], [3, 2], 251, mask_mode=mask_mode, window=window, ctx_null=True)
+
+
+@pytest.mark.parametrize("fmt", KV8)
+@pytest.mark.parametrize("scratch", [0, SCRATCH])
+def test_kv8_rotated_rows(fmt, scratch):
+    """Rows stored after sign + WHT256 (op_kv_cache.cu:36-44,71-99): the kernel rotates the query
+    rows and rotates the output back."""
+    _check(fmt, DT_F16, 64, [700, 130], [1, 3], 261, scratch=scratch, q_heads=16, xf=XF_WHT256)
+    _check(fmt, DT_BF16, 16, [45], [2], 262, scratch=scratch, xf=XF_WHT256)
+
+
+@pytest.mark.parametrize("fmt", KV8)
+def test_kv8_unwritten_pool_bytes_do_not_leak(fmt):
+    """Rows beyond the sequence hold 0xFF bytes (NaN codes and NaN scales): they must not reach
+    the output."""
+    import gpu_harness as G
+
+    pool, bt, k, v, q, aq, ctx = make_case(fmt, 64, [37, 100], [1, 2], 271, DT_F16)
+    hb = oracle.HostBatch(aq, [37, 100], bt, context_lens_before=ctx)
+    want = oracle.paged_attention(pool, hb, q, DT_F16, 8)
+    kk = pool.k.reshape(-1, pool.kv_heads, pool.block_size, pool.tok)
+    vv = pool.v.reshape(-1, pool.kv_heads, pool.block_size, pool.tok)
+    for r, s in enumerate([37, 100]):
+        last = bt[r, (s - 1) // 64]
+        kk[last, :, s % 64:, :] = 0xFF
+        vv[last, :, s % 64:, :] = 0xFF
+    dpool = _dev_pool(pool)
+    for scratch in (0, SCRATCH):
+        rc, got, _ = G.dev_attention(dpool, hb, q, DT_F16, 8, scratch_bytes=scratch)
+        assert rc == 0
+        G.assert_close(got, DT_F16, want, what="poisoned tail", scale=G.channel_scale(v, DT_F16, hb, 8))
 
 
 # ---- chunked prefill over TQ4 pages (128-row tile kernel) ----

@@ -106,6 +106,8 @@ struct AttnParams {
     int max_chunks;   // cap on chunks per tile (1 = no split, scratch untouched)
     int min_upc;      // minimum units per chunk
     int tiles_by_request;  // 1: blockIdx.z is a request (no request has more than one tile)
+    int rot_q;             // row-format kernel: K rows are stored rotated, rotate the query rows
+    int rot_out;           // row-format kernel: V rows are stored rotated, rotate the output back
 };
 
 // token of k-slot (s, b, i) inside a unit: spreads the four 4-row groups of an MFMA over LDS
@@ -1134,7 +1136,7 @@ __device__ __forceinline__ TileInfo locate_tile(const AttnParams& P, int tile_z,
 
 }  // namespace w34
 
-#include "paged_attn_kv16.h"
+#include "paged_attn_rows.h"
 #include "paged_prefill_tq4.h"
 
 namespace w34 {
@@ -1185,7 +1187,7 @@ template <typename TQ>
 static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
                       const warp34_attention_batch* batch, const void* q, void* out, int num_q_heads,
                       int force_single) {
-    AttnParams P;
+    AttnParams P{};
     P.L = *layout;
     P.B = *batch;
     P.q = (const uint16_t*)q;
@@ -1245,11 +1247,11 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     return rc;
 }
 
-template <typename TQ>
-static int launch_kv16(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
+template <typename TQ, int KVF>
+static int launch_rows(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
                        const warp34_attention_batch* batch, const void* q, void* out, int num_q_heads,
                        int force_single) {
-    AttnParams P;
+    AttnParams P{};
     P.L = *layout;
     P.B = *batch;
     P.q = (const uint16_t*)q;
@@ -1285,17 +1287,19 @@ static int launch_kv16(const warp34_exec* ex, const warp34_kv_layer_layout* layo
         if (bound < grid_x) grid_x = bound < 1 ? 1 : bound;
     }
     P.tiles_by_request = (batch->max_q_len > 0 && batch->max_q_len <= P.tok_tile) ? 1 : 0;
+    P.rot_q = layout->k_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 ? 1 : 0;
+    P.rot_out = layout->v_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 ? 1 : 0;
     const int grid_z = P.tiles_by_request ? batch->num_reqs : batch->total_tokens / P.tok_tile + batch->num_reqs;
     const dim3 grid((unsigned)grid_x, (unsigned)(layout->local_kv_heads * P.q_subgroups), (unsigned)grid_z);
     hipStream_t stream = (hipStream_t)ex->stream;
-    int rc = ensure_dynamic_lds(paged_attn_kv16_kernel<TQ, 1>, kv16_smem_bytes(1));
+    int rc = ensure_dynamic_lds(paged_attn_rows_kernel<TQ, 1, KVF>, kv16_smem_bytes(1));
     if (rc) return rc;
-    hipLaunchKernelGGL((paged_attn_kv16_kernel<TQ, 1>), grid, dim3(kKv16Waves * 64), kv16_smem_bytes(1), stream, P);
+    hipLaunchKernelGGL((paged_attn_rows_kernel<TQ, 1, KVF>), grid, dim3(kKv16Waves * 64), kv16_smem_bytes(1), stream, P);
     rc = (int)hipGetLastError();
     if (rc) return rc;
     if (P.max_chunks > 1) {
         hipLaunchKernelGGL((split_merge_kernel<TQ>), dim3((unsigned)rows), dim3(1024), 0, stream,
-                           (const float*)P.part_acc, (const float*)P.part_ml, P.max_chunks, P, 1.0f, 0);
+                           (const float*)P.part_acc, (const float*)P.part_ml, P.max_chunks, P, 1.0f, P.rot_out);
         rc = (int)hipGetLastError();
     }
     return rc;
@@ -1320,7 +1324,7 @@ static bool prefill_tq4_applicable(const warp34_kv_layer_layout* layout, const w
 template <typename TQ>
 static int launch_prefill_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
                               const warp34_attention_batch* batch, const void* q, void* out, int num_q_heads) {
-    AttnParams P;
+    AttnParams P{};
     P.L = *layout;
     P.B = *batch;
     P.q = (const uint16_t*)q;
@@ -1358,6 +1362,24 @@ static bool is_kv16(const warp34_kv_layer_layout* l, int format) {
 static bool kv16_geometry_ok(const warp34_kv_layer_layout* l, const void* q, const void* out) {
     return l->block_size > 0 && (l->block_size % 16) == 0 && l->k_token_stride_bytes == 512 &&
            l->v_token_stride_bytes == 512 && (l->k_base & 15u) == 0 && (l->v_base & 15u) == 0 &&
+           (l->k_page_stride_bytes & 15u) == 0 && (l->k_head_stride_bytes & 15u) == 0 &&
+           (l->v_page_stride_bytes & 15u) == 0 && (l->v_head_stride_bytes & 15u) == 0 &&
+           (((uintptr_t)q) & 15u) == 0 && (((uintptr_t)out) & 7u) == 0;
+}
+
+// 8-bit rows: both slabs in the same format, each stored plain or rotated
+static bool is_kv8(const warp34_kv_layer_layout* l, int format) {
+    const auto xf_ok = [](int t) {
+        return t == WARP34_KV_TRANSFORM_IDENTITY || t == WARP34_KV_TRANSFORM_RADEMACHER_WHT256;
+    };
+    return l->head_dim == 256 && l->k_format == format && l->v_format == format && xf_ok(l->k_transform) &&
+           xf_ok(l->v_transform);
+}
+
+// 16-token runs must be contiguous and 16-byte aligned for the staging copy
+static bool kv8_geometry_ok(const warp34_kv_layer_layout* l, const void* q, const void* out, unsigned row_bytes) {
+    return l->block_size > 0 && (l->block_size % 16) == 0 && l->k_token_stride_bytes == row_bytes &&
+           l->v_token_stride_bytes == row_bytes && (l->k_base & 15u) == 0 && (l->v_base & 15u) == 0 &&
            (l->k_page_stride_bytes & 15u) == 0 && (l->k_head_stride_bytes & 15u) == 0 &&
            (l->v_page_stride_bytes & 15u) == 0 && (l->v_head_stride_bytes & 15u) == 0 &&
            (((uintptr_t)q) & 15u) == 0 && (((uintptr_t)out) & 7u) == 0;
@@ -1408,7 +1430,16 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
     // point, BF16 pages with the bf16 one, as in the reference)
     if (is_kv16(layout, TQ::kStorageFormat)) {
         if (!kv16_geometry_ok(layout, q, out)) return (int)hipErrorNotSupported;
-        return launch_kv16<TQ>(ex, layout, batch, q, out, num_q_heads, force_single);
+        return launch_rows<TQ, TQ::kStorageFormat>(ex, layout, batch, q, out, num_q_heads, force_single);
+    }
+    // 8-bit pages (the tail layers of the default TQ4 policy, cache.rs:87-109)
+    if (is_kv8(layout, WARP34_KV_FORMAT_FP8_E4M3)) {
+        if (!kv8_geometry_ok(layout, q, out, 264)) return (int)hipErrorNotSupported;
+        return launch_rows<TQ, WARP34_KV_FORMAT_FP8_E4M3>(ex, layout, batch, q, out, num_q_heads, force_single);
+    }
+    if (is_kv8(layout, WARP34_KV_FORMAT_Q8_0)) {
+        if (!kv8_geometry_ok(layout, q, out, 272)) return (int)hipErrorNotSupported;
+        return launch_rows<TQ, WARP34_KV_FORMAT_Q8_0>(ex, layout, batch, q, out, num_q_heads, force_single);
     }
     return (int)hipErrorNotSupported;
 }
@@ -1424,8 +1455,8 @@ extern "C" int warp34_paged_attention_f16(const warp34_exec* ex, const warp34_kv
     const int rc = common_checks(ex, layout, batch, q_in, attn_out, num_q_heads);
     if (rc) return rc;
     if (layout->k_format == WARP34_KV_FORMAT_FP8_E4M3 || layout->v_format == WARP34_KV_FORMAT_FP8_E4M3) {
+        // the reference also asks the device generation here (op_paged_attn.cu:1259); gfx950 has FP8
         if (layout->head_dim != 256) return (int)hipErrorInvalidValue;
-        return (int)hipErrorNotSupported;
     }
     if (batch->total_tokens <= 0 || num_q_heads <= 0) return 0;
     return attention_entry<F16>(ex, layout, batch, q_in, attn_out, num_q_heads, 0);

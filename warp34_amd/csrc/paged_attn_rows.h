@@ -1,18 +1,23 @@
-// Paged GQA decode / verify attention over 16-bit KV pages (FP16 or BF16 storage, identity
-// transform) for gfx950.  Same work decomposition, chunk geometry, wave merge and split-K
-// partial format as the TQ4 kernel in paged_attn.hip (which includes this file); only the
-// per-unit body differs:
+// Paged GQA decode / verify attention over pages whose rows are read as stored: 16-bit rows
+// (FP16 or BF16 storage, identity transform) and the 8-bit rows FP8-E4M3-256 and Q8_0-64, for
+// gfx950.  Same work decomposition, chunk geometry, wave merge and split-K partial format as
+// the TQ4 kernel in paged_attn.hip (which includes this file); only the per-unit body differs:
 //   * a 32-token unit is processed as two 16-token halves; the wave copies the 16 K rows and
-//     16 V rows of a half (512 B each) into its private LDS area with a 528-byte row stride
-//     (132 dwords: the 8 lanes of a 128-bit read pass land on 32 distinct banks);
-//   * S^T = K Q^T: A operand = 16 K rows read straight from LDS (8 x 128-bit reads),
-//     B operand = the query rows, loaded once from global memory in MFMA layout;
+//     16 V rows of a half into its private LDS area.  16-bit rows (512 B) get a 528-byte row
+//     stride (132 dwords: the 8 lanes of a 128-bit read pass land on 32 distinct banks),
+//     8-bit rows (264 B / 272 B, codes and their fp32 block scales) a 272-byte one;
+//   * S^T = K Q^T: A operand = 16 K rows read from LDS, B operand = the query rows, loaded
+//     once in MFMA layout.  8-bit codes are widened to fp16 in registers (exact) and the fp32
+//     block scales are applied to per-block partial scores, so K is never rounded;
 //   * O^T += V^T P^T with 16x16x16 MFMAs: each lane reads the 8-element slice of its 4 tokens
-//     and transposes the 4x8 block of 16-bit values in registers with v_perm_b32;
+//     and transposes the 4x8 block in registers.  8-bit V is dequantised to fp16(d * code)
+//     on the way, which is what the reference stages (op_paged_attn.cu:59-105);
 //   * BF16 storage: P is split into a bf16 high and low part (two MFMAs) so that the 8-bit
-//     mantissa of bf16 does not limit the accuracy of the weighted sum.
-// Replaces paged_attention_gqa_bf16_kernel (op_kv_cache.cu:873-1168) and the FP16 branch of
-// paged_attention_gqa_mma_f16_kernel (op_paged_attn.cu:186-588).
+//     mantissa of bf16 does not limit the accuracy of the weighted sum;
+//   * 8-bit layers may be stored rotated (WHT256 transform): the query rows are then rotated
+//     once per tile and the output is rotated back once (op_kv_cache.cu:443-451,763-783).
+// Replaces paged_attention_gqa_bf16_kernel (op_kv_cache.cu:873-1168) and the FP16, Q8_0 and
+// FP8 branches of paged_attention_gqa_mma_f16_kernel (op_paged_attn.cu:186-588).
 #pragma once
 
 namespace w34 {
@@ -24,6 +29,7 @@ typedef uint32_t u2v __attribute__((ext_vector_type(2)));
 
 constexpr int kKv16Waves = 8;
 constexpr int kKv16RowStride = 528;                      // bytes, 512 + 16 pad
+constexpr int kKv8RowStride = 272;                       // bytes: Q8_0 rows as stored, FP8 rows + 8 pad
 constexpr int kKv16Stage = 2 * 16 * kKv16RowStride;      // K half + V half: 16896 B per wave
 // byte offset of the (m, l) exchange table: behind both the staging areas and the merge regions
 __host__ __device__ constexpr int kv16_ml_offset(int nt) {
@@ -33,6 +39,35 @@ __host__ __device__ constexpr int kv16_ml_offset(int nt) {
 }
 __host__ __device__ constexpr int kv16_smem_bytes(int nt) {
     return kv16_ml_offset(nt) + (kKv16Waves + 1) * nt * 16 * 2 * 4 + 256;
+}
+
+// four E4M3 codes -> four fp16 values (exact)
+__device__ __forceinline__ void fp8x4_to_h4(uint32_t w, uint32_t& lo, uint32_t& hi) {
+    lo = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false));
+    hi = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true));
+}
+// four int8 codes -> four fp16 values (exact): 0x6400 | (q + 128) is 1024 + (q + 128) in fp16
+__device__ __forceinline__ void i8x4_to_h4(uint32_t w, uint32_t& lo, uint32_t& hi) {
+    const uint32_t u = w ^ 0x80808080u;
+    const h2 bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+    const h2 a = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias;
+    const h2 c = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias;
+    lo = __builtin_bit_cast(uint32_t, a);
+    hi = __builtin_bit_cast(uint32_t, c);
+}
+// four 8-bit codes -> fp32
+template <bool FP8>
+__device__ __forceinline__ void codes4_to_f32(uint32_t w, float (&f)[4]) {
+    if constexpr (FP8) {
+        const f2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+        const f2 c = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+        f[0] = a.x, f[1] = a.y, f[2] = c.x, f[3] = c.y;
+    } else {
+        f[0] = (float)(int8_t)(w & 0xFFu);
+        f[1] = (float)(int8_t)((w >> 8) & 0xFFu);
+        f[2] = (float)(int8_t)((w >> 16) & 0xFFu);
+        f[3] = (float)(int8_t)(w >> 24);
+    }
 }
 
 template <bool IS_BF16>
@@ -52,11 +87,19 @@ __device__ __forceinline__ f4 mfma_x16(u2v a, u2v b, f4 c) {
     }
 }
 
-// TQ doubles as the storage type: F16 query/output over FP16 pages, BF16 over BF16 pages.
-template <typename TQ, int NT>
-__global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(const AttnParams P) {
-    constexpr bool IS_BF16 = TQ::kStorageFormat == WARP34_KV_FORMAT_BF16;
+// KVF is the storage format of both slabs.  16-bit pages: TQ doubles as the storage type (F16
+// query/output over FP16 pages, BF16 over BF16 pages).  8-bit pages: the MFMAs run in fp16 and
+// a BF16 query is converted once.
+template <typename TQ, int NT, int KVF>
+__global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_rows_kernel(const AttnParams P) {
+    constexpr bool K8 = KVF == WARP34_KV_FORMAT_FP8_E4M3 || KVF == WARP34_KV_FORMAT_Q8_0;
+    constexpr bool FP8 = KVF == WARP34_KV_FORMAT_FP8_E4M3;
+    static_assert(K8 || KVF == TQ::kStorageFormat, "16-bit pages are read in the query type");
+    constexpr bool IS_BF16 = !K8 && TQ::kStorageFormat == WARP34_KV_FORMAT_BF16;
+    constexpr bool Q_BF16 = TQ::kStorageFormat == WARP34_KV_FORMAT_BF16;
     constexpr int kWaves = kKv16Waves;
+    constexpr int kRowStride = K8 ? kKv8RowStride : kKv16RowStride;  // LDS row stride
+    constexpr int kRowBytes = K8 ? (FP8 ? 264 : 272) : 512;          // row in memory
     extern __shared__ __align__(16) uint8_t smem[];
 
     const int tid = (int)threadIdx.x;
@@ -91,7 +134,38 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
             for (int m = 0; m < 8; ++m) bq[nt][m] = *reinterpret_cast<const u4*>(qrow + 32 * m + 8 * b);
         }
     };
-    load_q(tok_guess);
+    // Rotated K rows: the query rows go through sign + WHT256 first (one row per wave at a time,
+    // element e = 4 lane + k), are staged as fp16 in the still unused staging area and read
+    // back in MFMA layout.
+    constexpr int kQStride = 264;  // halves
+    auto load_q_rotated = [&](int tokbase) {
+        _Float16* qlds = reinterpret_cast<_Float16*>(smem);
+        for (int col = wave; col < 16 * NT; col += kWaves) {
+            const int t = fast_div(col, P.q_group);
+            const int a = col - t * P.q_group;
+            const int tok = min(tokbase + t, B.total_tokens - 1);
+            const uint16_t* qrow = P.q + ((size_t)tok * P.num_q_heads + (size_t)(q_head_base + a)) * kHeadDim;
+            const uint2 raw = *reinterpret_cast<const uint2*>(qrow + 4 * lane);
+            float v[4] = {TQ::to_f32((uint16_t)(raw.x & 0xFFFFu)), TQ::to_f32((uint16_t)(raw.x >> 16)),
+                          TQ::to_f32((uint16_t)(raw.y & 0xFFFFu)), TQ::to_f32((uint16_t)(raw.y >> 16))};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) v[k] = apply_sign(v[k], 4 * lane + k);
+            wht256_wave(v, lane);
+            uint2 packed;
+            packed.x = pack_h2(v[0], v[1]);
+            packed.y = pack_h2(v[2], v[3]);
+            *reinterpret_cast<uint2*>(qlds + col * kQStride + 4 * lane) = packed;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int m = 0; m < 8; ++m)
+                bq[nt][m] = *reinterpret_cast<const u4*>(qlds + (nt * 16 + n) * kQStride + 32 * m + 8 * b);
+        __syncthreads();  // the staging area is reused by the K/V rows
+    };
+    const bool rot_q = K8 && P.rot_q != 0;  // workgroup-uniform
+    if (!rot_q) load_q(tok_guess);
 
     // Speculative block-table load, in flight together with the lookup: it assumes that the
     // request's length is the host's bound max_seq_len.  A wrong guess is fetched again below,
@@ -109,7 +183,22 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
     const int req = ti.req, rq_start = ti.rq_start, rq_end = ti.rq_end;
     const int seq_after = ti.seq_after, ctx_before = ti.ctx_before;
     const int tok0 = rq_start + ti.tile_in_req * P.tok_tile;
-    if (tok0 != tok_guess) load_q(tok0);  // wave-uniform, rare
+    if (rot_q) {
+        load_q_rotated(tok0);  // every wave of the workgroup takes the same path up to here
+    } else {
+        if (tok0 != tok_guess) load_q(tok0);  // wave-uniform, rare
+        if constexpr (K8 && Q_BF16) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int m = 0; m < 8; ++m)
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const uint32_t w = bq[nt][m][k];
+                        bq[nt][m][k] = pack_h2(BF16::to_f32((uint16_t)(w & 0xFFFFu)), BF16::to_f32((uint16_t)(w >> 16)));
+                    }
+        }
+    }
     bool tok_ok[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
@@ -181,7 +270,7 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
                             (size_t)kv_head * L.k_head_stride_bytes;
     const uint8_t* v_base = reinterpret_cast<const uint8_t*>((uintptr_t)L.v_base) +
                             (size_t)kv_head * L.v_head_stride_bytes;
-    uint8_t* stage = smem + wave * kKv16Stage;  // [K rows 0..15][V rows 0..15], 528 B each
+    uint8_t* stage = smem + wave * kKv16Stage;  // [K rows 0..15][V rows 0..15], kRowStride each
     const int32_t* req_blocks = B.block_tables + (size_t)req * B.max_blocks_per_req;
     int slot_base = fast_div(cu_first * kUnit, L.block_size);
     int page_vec;
@@ -190,9 +279,12 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
         page_vec = slot < B.max_blocks_per_req ? req_blocks[slot] : -1;
     };
 
-    // A half = 16 consecutive tokens: 8 KiB of K and 8 KiB of V, each contiguous inside one
-    // page.  Piece c = lane + 64 i (16 B) is element column c % 32 of row c / 32.
-    u4 pf[16];
+    // A half = 16 consecutive tokens: 16 K rows and 16 V rows, each run contiguous inside one
+    // page (8 KiB of 16-bit rows, 4224 B of FP8 rows, 4352 B of Q8_0 rows).  It is fetched as
+    // 16-byte pieces c = lane + 64 i.
+    constexpr int kPieces = 16 * kRowBytes / 16;        // 512, 264 or 272
+    constexpr int kLoads = (kPieces + 63) / 64;         // 8 or 5
+    u4 pf[2 * kLoads];
     auto issue_half = [&](int hidx) {  // hidx = 2 * unit + half
         const int pos = hidx * 16;
         const int page_slot = fast_div(pos, L.block_size);
@@ -208,9 +300,11 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
         const uint8_t* kp = k_base + (live ? (size_t)pg * L.k_page_stride_bytes + (size_t)in_page * L.k_token_stride_bytes : 0);
         const uint8_t* vp = v_base + (live ? (size_t)pg * L.v_page_stride_bytes + (size_t)in_page * L.v_token_stride_bytes : 0);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            pf[i] = *(global_cu4*)(kp + 16 * lane + 1024 * i);
-            pf[8 + i] = *(global_cu4*)(vp + 16 * lane + 1024 * i);
+        for (int i = 0; i < kLoads; ++i) {
+            // pieces beyond the run (last, partial round of the 8-bit formats) re-read piece 0
+            const int c = (kPieces % 64 == 0 || lane + 64 * i < kPieces) ? lane + 64 * i : 0;
+            pf[i] = *(global_cu4*)(kp + 16 * c);
+            pf[kLoads + i] = *(global_cu4*)(vp + 16 * c);
         }
     };
     // rows outside [u_lo, u_hi] are stored as zeros: unwritten pool memory may hold NaN
@@ -218,20 +312,42 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
     auto commit_half = [&](int hidx) {
         const int pos0 = hidx * 16;
         const bool edge = pos0 < u_lo || pos0 + 15 > u_hi;
+        uint8_t* k_rows = stage;
+        uint8_t* v_rows = stage + 16 * kRowStride;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < kLoads; ++i) {
             const int c = lane + 64 * i;
-            const int row = c >> 5;
-            u4 kv = pf[i], vv = pf[8 + i];
-            if (edge) {
-                const bool vis = pos0 + row >= u_lo && pos0 + row <= u_hi;
-                if (!vis) {
-                    kv = u4{0u, 0u, 0u, 0u};
-                    vv = u4{0u, 0u, 0u, 0u};
+            if (kPieces % 64 != 0 && c >= kPieces) break;
+            u4 kv = pf[i], vv = pf[kLoads + i];
+            if constexpr (FP8) {
+                // 264-byte rows: the two 8-byte halves of a piece may belong to different rows
+#pragma unroll
+                for (int hf = 0; hf < 2; ++hf) {
+                    const unsigned sub = 2u * (unsigned)c + hf;
+                    const unsigned row = sub / 33u, col = sub - row * 33u;
+                    u2v k8 = hf ? u2v{kv[2], kv[3]} : u2v{kv[0], kv[1]};
+                    u2v v8 = hf ? u2v{vv[2], vv[3]} : u2v{vv[0], vv[1]};
+                    if (edge && !(pos0 + (int)row >= u_lo && pos0 + (int)row <= u_hi)) {
+                        k8 = u2v{0u, 0u};
+                        v8 = u2v{0u, 0u};
+                    }
+                    *reinterpret_cast<u2v*>(k_rows + row * kRowStride + 8 * col) = k8;
+                    *reinterpret_cast<u2v*>(v_rows + row * kRowStride + 8 * col) = v8;
                 }
+            } else {
+                constexpr int kPiecesPerRow = kRowBytes / 16;  // 32 or 17
+                const int row = (int)((unsigned)c / (unsigned)kPiecesPerRow);
+                const int col = c - row * kPiecesPerRow;
+                if (edge) {
+                    const bool vis = pos0 + row >= u_lo && pos0 + row <= u_hi;
+                    if (!vis) {
+                        kv = u4{0u, 0u, 0u, 0u};
+                        vv = u4{0u, 0u, 0u, 0u};
+                    }
+                }
+                *reinterpret_cast<u4*>(k_rows + row * kRowStride + 16 * col) = kv;
+                *reinterpret_cast<u4*>(v_rows + row * kRowStride + 16 * col) = vv;
             }
-            *reinterpret_cast<u4*>(stage + row * kKv16RowStride + 16 * (c & 31)) = kv;
-            *reinterpret_cast<u4*>(stage + 16 * kKv16RowStride + row * kKv16RowStride + 16 * (c & 31)) = vv;
         }
     };
 
@@ -250,27 +366,105 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
 
     auto process_half = [&](int pos0, const bool MASKED) {
         const uint8_t* k_rows = stage;
-        const uint8_t* v_rows = stage + 16 * kKv16RowStride;
+        const uint8_t* v_rows = stage + 16 * kRowStride;
         // ---- S^T = K Q^T: A row n = token n of the half ----
         f4 s_acc[NT];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) s_acc[nt] = f4{0.f, 0.f, 0.f, 0.f};
-        u4 ka[8];
+        // V operands of the 16 P V MFMAs: a_v[h][j] = element 128 h + 8 n + j of tokens 4b..4b+3
+        u2v a_v[2][8];
+        if constexpr (K8) {
+            // Codes of row n, elements 32 m + 8 b .. + 7, widened to fp16; one partial score per
+            // scale block (FP8: 2 blocks of 128 = m / 4; Q8_0: 4 blocks of 64 = m / 2), combined
+            // with the fp32 scales of this lane's 4 tokens.
+            constexpr int kBlocks = FP8 ? 2 : 4;
+            constexpr int kMPerBlock = 8 / kBlocks;
+            u4 ka[8];
 #pragma unroll
-        for (int m = 0; m < 8; ++m)
-            ka[m] = *reinterpret_cast<const u4*>(k_rows + n * kKv16RowStride + 64 * m + 16 * b);
-#pragma unroll
-        for (int m = 0; m < 8; ++m)
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) s_acc[nt] = mfma_x32<IS_BF16>(ka[m], bq[nt][m], s_acc[nt]);
-
-        // raw V slices of this lane's 4 tokens (rows 4b..4b+3), both halves of the head dim
-        u4 vr[2][4];
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
+            for (int m = 0; m < 8; ++m) {
+                const int off = FP8 ? 32 * m + 8 * b : 68 * (m >> 1) + 4 + 32 * (m & 1) + 8 * b;
+                const uint32_t* src = reinterpret_cast<const uint32_t*>(k_rows + n * kRowStride + off);
+                const uint32_t w0 = src[0], w1 = src[1];
+                uint32_t h0, h1, h2_, h3;
+                if constexpr (FP8) {
+                    fp8x4_to_h4(w0, h0, h1);
+                    fp8x4_to_h4(w1, h2_, h3);
+                } else {
+                    i8x4_to_h4(w0, h0, h1);
+                    i8x4_to_h4(w1, h2_, h3);
+                }
+                ka[m] = u4{h0, h1, h2_, h3};
+            }
+            float dk[4][kBlocks];
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                vr[h][i] = *reinterpret_cast<const u4*>(v_rows + (4 * b + i) * kKv16RowStride + 256 * h + 16 * n);
+#pragma unroll
+                for (int kb = 0; kb < kBlocks; ++kb)
+                    dk[i][kb] = *reinterpret_cast<const float*>(k_rows + (4 * b + i) * kRowStride +
+                                                                (FP8 ? 256 + 4 * kb : 68 * kb));
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                for (int kb = 0; kb < kBlocks; ++kb) {
+                    f4 part = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int mm = 0; mm < kMPerBlock; ++mm)
+                        part = mfma_x32<false>(ka[kb * kMPerBlock + mm], bq[nt][kb * kMPerBlock + mm], part);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) s_acc[nt][i] += dk[i][kb] * part[i];
+                }
+            }
+            // V: fp16(d * code), the value the reference stages (op_paged_attn.cu:59-105)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                float vf[4][8];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint8_t* vrow = v_rows + (4 * b + i) * kRowStride;
+                    const int blk = 2 * h + (n >> 3);  // Q8_0 block of element 128 h + 8 n
+                    const int off = FP8 ? 128 * h + 8 * n : 68 * blk + 4 + 8 * (n & 7);
+                    const uint32_t* src = reinterpret_cast<const uint32_t*>(vrow + off);
+                    const float d = *reinterpret_cast<const float*>(vrow + (FP8 ? 256 + 4 * h : 68 * blk));
+                    float f0[4], f1[4];
+                    codes4_to_f32<FP8>(src[0], f0);
+                    codes4_to_f32<FP8>(src[1], f1);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        vf[i][k] = d * f0[k];
+                        vf[i][4 + k] = d * f1[k];
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    a_v[h][j] = u2v{pack_h2(vf[0][j], vf[1][j]), pack_h2(vf[2][j], vf[3][j])};
+            }
+        } else {
+            u4 ka[8];
+#pragma unroll
+            for (int m = 0; m < 8; ++m)
+                ka[m] = *reinterpret_cast<const u4*>(k_rows + n * kRowStride + 64 * m + 16 * b);
+#pragma unroll
+            for (int m = 0; m < 8; ++m)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) s_acc[nt] = mfma_x32<IS_BF16>(ka[m], bq[nt][m], s_acc[nt]);
+
+            // V slices of this lane's 4 tokens (rows 4b..4b+3), both halves of the head dim; the
+            // 4x8 block of 16-bit values is transposed in registers
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                u4 vr[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    vr[i] = *reinterpret_cast<const u4*>(v_rows + (4 * b + i) * kRowStride + 256 * h + 16 * n);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    // 16-bit element j of the four token slices -> (t0,t1), (t2,t3)
+                    const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+                    a_v[h][j] = u2v{__builtin_amdgcn_perm(vr[1][j >> 1], vr[0][j >> 1], sel),
+                                    __builtin_amdgcn_perm(vr[3][j >> 1], vr[2][j >> 1], sel)};
+                }
+            }
+        }
 
         // ---- online softmax over this lane's 4 tokens ----
         u2v pb_hi[NT], pb_lo[NT];
@@ -326,11 +520,7 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
         for (int h = 0; h < 2; ++h) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                // 16-bit element j of the four token slices -> (t0,t1), (t2,t3)
-                const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
-                u2v a;
-                a[0] = __builtin_amdgcn_perm(vr[h][1][j >> 1], vr[h][0][j >> 1], sel);
-                a[1] = __builtin_amdgcn_perm(vr[h][3][j >> 1], vr[h][2][j >> 1], sel);
+                const u2v a = a_v[h][j];
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
                     o_acc[nt][h][j] = mfma_x16<IS_BF16>(a, pb_hi[nt], o_acc[nt][h][j]);
@@ -447,9 +637,16 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_kv16_kernel(con
             }
         } else {
             const float inv = l_col > 0.f ? 1.0f / l_col : 0.f;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) v[k] *= inv;
+            if (K8 && P.rot_out) {  // rotated V rows: one inverse rotation of the finished row
+                wht256_wave(v, lane);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) v[k] = apply_sign(v[k], 4 * lane + k);
+            }
             uint2 o;
-            o.x = (uint32_t)TQ::from_f32(v[0] * inv) | ((uint32_t)TQ::from_f32(v[1] * inv) << 16);
-            o.y = (uint32_t)TQ::from_f32(v[2] * inv) | ((uint32_t)TQ::from_f32(v[3] * inv) << 16);
+            o.x = (uint32_t)TQ::from_f32(v[0]) | ((uint32_t)TQ::from_f32(v[1]) << 16);
+            o.y = (uint32_t)TQ::from_f32(v[2]) | ((uint32_t)TQ::from_f32(v[3]) << 16);
             *reinterpret_cast<uint2*>(P.out + row * kHeadDim + 4 * lane) = o;
         }
     }
