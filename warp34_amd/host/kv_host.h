@@ -39,6 +39,11 @@ struct LayerFormats {
 // Row bytes of one head in `format`; unknown formats size like 16-bit rows (cache.rs:157-165).
 size_t kv_format_row_bytes(int format, size_t head_dim);
 
+// What DeviceProps::supports_fp8_kv() (model/rank.rs:924-932) answers for the device these kernels
+// are written for: gfx950 converts OCP E4M3 in hardware and the FP8 append and attention
+// kernels are built, so the Tq4 policy's tail layers resolve to FP8.
+constexpr bool kDeviceSupportsFp8Kv = true;
+
 // Tq4: the last four full-attention layers are unrotated 8-bit (FP8 when the device has it,
 // else Q8_0), all earlier ones rotated TQ4 (cache.rs:87-109).
 LayerFormats resolve_layer_with_fp8(KvFormatPolicy policy, size_t full_attn_layer_ordinal,
