@@ -36,6 +36,7 @@ WORKLOADS = {
     "q8_0_decode_b1_ctx131072": ("q8_0", [131072], 0),
     # 8 sequences, 16 384-token TQ4 prefix + 2 048-token bf16 chunk each: append + causal attention
     "tq4_prefill_8x2048_ctx16384": ("tq4", [18432] * 8, 0),
+    "fp8_prefill_8x2048_ctx16384": ("fp8", [18432] * 8, 0),
     # 16 sequences of 262 144 tokens that share the pages of a 200 000-token prefix; 4 query tokens each
     "tq4_verify_16x4_ctx262144_shared200k": ("tq4", [262144] * 16, 0),
 }
@@ -63,7 +64,7 @@ def parse():
                          "FETCH_SIZE / WRITE_SIZE counters of rocprofv3 --pmc)")
     ap.add_argument("--cpu-ctx", type=int, default=32768, help="context length of the CPU-oracle sample")
     args = ap.parse_args()
-    prefill = args.workload.startswith("tq4_prefill")
+    prefill = "_prefill_" in args.workload
     if args.steps <= 0:
         args.steps = 10 if prefill else 200
     if args.warmup < 0:
@@ -181,8 +182,8 @@ def cpu_baseline(ctx_len, threads):
     }
 
 
-def run_prefill(args, torch, lib, ffi, layers, ctx, n_layers, pool_pages):
-    """Chunked prefill: every sequence re-appends its last PREFILL_CHUNK tokens (bf16 -> TQ4)
+def run_prefill(args, torch, lib, ffi, layers, ctx, n_layers, pool_pages, fmt):
+    """Chunked prefill: every sequence re-appends its last PREFILL_CHUNK tokens (bf16 -> TQ4 / FP8)
     and attends causally over prefix + chunk.  One step = append + attention of one layer."""
     dev = "cuda:0"
     R, n = len(ctx), PREFILL_CHUNK
@@ -240,19 +241,23 @@ def run_prefill(args, torch, lib, ffi, layers, ctx, n_layers, pool_pages):
     tf_attn = flops / (ms_attn * 1e-3) / 1e12
     peak = 2500.0
     print(json.dumps({
-        "metric": "chunked prefill over TQ4 pages (append + causal attention): ms/layer + achieved MFMA TFLOP/s",
+        "metric": "chunked prefill over %s pages (append + causal attention): ms/layer + achieved MFMA TFLOP/s"
+                  % fmt.upper(),
         "value": round(tf_step, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "ms_attention_only": round(ms_attn, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16 MFMA operands (TQ4 codes -> fp16 centroids), f32 accumulate, bf16 Q/out",
+        "dtype": "f16 MFMA operands (%s), f32 accumulate, bf16 Q/out"
+                 % ("TQ4 codes -> fp16 centroids" if fmt == "tq4" else "E4M3 codes widened"),
         "data": "synthetic",
         "config": {"workload": args.workload, "requests": R, "chunk_tokens": n, "prefix_tokens": int(ctx[0]) - n,
                    "q_heads": Q_HEADS, "kv_heads": KV_HEADS, "head_dim": HEAD_DIM, "page_tokens": BLOCK,
-                   "kv_format": "tq4+wht256", "kv_pools_cycled": n_layers, "pool_pages": pool_pages,
+                   "kv_format": "tq4+wht256" if fmt == "tq4" else fmt, "kv_pools_cycled": n_layers,
+                   "pool_pages": pool_pages,
                    "attention_flops_per_step": flops, "rows_appended_per_step": N * KV_HEADS * 2},
         "roofline": {"bound": "mfma", "achieved": round(tf_attn, 1), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(tf_attn / peak, 4), "traffic": None,
-                     "kernel": "paged_prefill_tq4_kernel (attention-only launches)",
+                     "kernel": ("paged_prefill_tq4_kernel" if fmt == "tq4" else "paged_attn_rows_kernel") +
+                               " (attention-only launches)",
                      "avg_launch_us": round(ms_attn * 1e3, 1)},
     }))
 
@@ -309,8 +314,8 @@ def main():
     n_layers = args.layers or max(2, -(-(640 << 20) // layer_bytes))
     layers = [Layer(torch, lib, ffi, fmt, ctx, pool_pages, s, shared) for s in range(n_layers)]
 
-    if args.workload.startswith("tq4_prefill"):
-        run_prefill(args, torch, lib, ffi, layers, ctx, n_layers, pool_pages)
+    if "_prefill_" in args.workload:
+        run_prefill(args, torch, lib, ffi, layers, ctx, n_layers, pool_pages, fmt)
         return
 
     R = len(ctx)

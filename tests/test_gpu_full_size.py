@@ -16,7 +16,7 @@ import numpy as np
 import pytest
 
 import oracle
-from oracle import DT_BF16, FMT_TQ4
+from oracle import DT_BF16, FMT_FP8, FMT_Q8_0, FMT_TQ4, XF_IDENTITY, XF_WHT256
 
 pytestmark = pytest.mark.gpu
 
@@ -24,9 +24,10 @@ KV_HEADS, Q_HEADS, D, BS = 2, 16, 256, 64
 
 
 class BigPool:
-    """TQ4 pool on the device, filled request by request through warp34_kv_cache_write_bf16."""
+    """Pool on the device (TQ4 unless told otherwise), filled request by request through
+    warp34_kv_cache_write_bf16."""
 
-    def __init__(self, ctx, num_pages, seed, shared_prefix=0, sample_rows=512):
+    def __init__(self, ctx, num_pages, seed, shared_prefix=0, sample_rows=512, fmt=FMT_TQ4):
         import torch
 
         import gpu_harness as G
@@ -34,7 +35,8 @@ class BigPool:
 
         self.torch, self.G, self.ffi = torch, G, ffi
         self.ctx = [int(c) for c in ctx]
-        self.host = oracle.HostPool(num_pages, KV_HEADS, D, BS, FMT_TQ4, oracle.XF_WHT256)
+        self.fmt = fmt
+        self.host = oracle.HostPool(num_pages, KV_HEADS, D, BS, fmt, XF_WHT256 if fmt == FMT_TQ4 else XF_IDENTITY)
         self.dev = G.DevPool(self.host, fill=0)
         g = torch.Generator(device=G.DEV)
         g.manual_seed(seed)
@@ -106,8 +108,9 @@ class BigPool:
                 for head in range(KV_HEADS):
                     base = page * h.page + head * h.head + off * h.tok
                     for src, slab in ((kk, h.k), (vv, h.v)):
-                        want = oracle.encode_row(oracle.bf16_bits_to_f32(src[i, head]))
-                        assert bytes(slab[base:base + 132]) == bytes(want), "row at slot %d differs" % slot
+                        x = oracle.bf16_bits_to_f32(src[i, head])
+                        want = oracle.encode_row(x) if self.fmt == FMT_TQ4 else oracle.encode_row_fmt(x, self.fmt)
+                        assert bytes(slab[base:base + h.tok]) == bytes(want), "row at slot %d differs" % slot
                         checked += 1
         assert checked >= 256
         return checked
@@ -174,3 +177,25 @@ def test_chunked_prefill_8x2048_on_16k_prefix():
     ob = oracle.HostBatch(np.arange(R + 1) * chunk, pool.ctx, pool.bt, context_lens_before=[prefix] * R,
                           valid_token_mask=mask)
     _attend_and_compare(pool, hb, q, rows=rows, oracle_batch=ob)
+
+
+def test_fp8_decode_131072_tokens():
+    """One sequence of 131 072 tokens over FP8-E4M3 pages (the format of the default policy's last
+    four layers on this device), one query token."""
+    n = 131072
+    pool = BigPool([n], n // BS + 8, seed=431, fmt=FMT_FP8)
+    pool.check_sampled_rows_bit_exact()
+    q = oracle.fill_normal(Q_HEADS * D, 432, DT_BF16).reshape(1, Q_HEADS, D)
+    hb = oracle.HostBatch([0, 1], pool.ctx, pool.bt, context_lens_before=[n - 1])
+    _attend_and_compare(pool, hb, q)
+
+
+def test_q8_0_batched_decode_32_sequences_1k_to_64k():
+    """The batched decode shape over Q8_0 pages."""
+    ctx = np.random.default_rng(0).integers(1024, 65537, size=32)
+    pool = BigPool(ctx, (2 << 20) // BS, seed=441, fmt=FMT_Q8_0)
+    pool.check_sampled_rows_bit_exact()
+    R = len(ctx)
+    q = oracle.fill_normal(R * Q_HEADS * D, 442, DT_BF16).reshape(R, Q_HEADS, D)
+    hb = oracle.HostBatch(np.arange(R + 1), pool.ctx, pool.bt, context_lens_before=[c - 1 for c in pool.ctx])
+    _attend_and_compare(pool, hb, q)
