@@ -77,6 +77,28 @@ def test_tq4_decode_split_vs_single_pass():
     assert small.tobytes() == single.tobytes()
 
 
+@pytest.mark.parametrize("dtype", [DT_BF16, DT_F16])
+def test_tq4_decode_batch_balanced_shares(dtype):
+    """Decode batches whose requests differ widely in length: the work is cut into equal shares
+    of 32-token units across workgroups, so long requests are split over many workgroups and a
+    workgroup may work on several short requests in turn (one of them empty-keyed, one masked)."""
+    import gpu_harness as G
+
+    seq = [5000, 300, 9000, 64, 2500, 33, 1, 7777]
+    _check(FMT_TQ4, dtype, 64, seq, [1] * len(seq), 181, q_heads=16)
+    _check(FMT_TQ4, dtype, 16, seq, [1] * len(seq), 182, q_heads=8, window=0, mask_mode=1)
+    # two query tokens per request (one tile at 8 q heads per kv head), a masked request
+    pool, bt, k, v, q, aq, ctx = make_case(FMT_TQ4, 64, [700, 40, 3000], [2, 2, 2], 183, dtype, q_heads=16)
+    rmask = np.array([1, 0, 1], np.uint8)
+    hb = oracle.HostBatch(aq, [700, 40, 3000], bt, context_lens_before=ctx, valid_req_mask=rmask)
+    want = oracle.paged_attention(pool, hb, q, dtype, 16, n_threads=4)
+    rc, got, _ = G.dev_attention(_dev_pool(pool), hb, q, dtype, 16, scratch_bytes=SCRATCH)
+    assert rc == 0
+    assert (got[2:4] == 0x5500).all()  # rows of the masked request keep the sentinel
+    live = np.array([0, 1, 4, 5])
+    G.assert_close(got[live], dtype, want[live], what="masked request", scale=G.channel_scale(v, dtype, hb, 16)[live])
+
+
 @pytest.mark.parametrize("q_lens", [[4, 4], [2, 3], [16]])
 def test_tq4_verify_multi_token_causal(q_lens):
     seq = [300 + 7 * i for i in range(len(q_lens))]

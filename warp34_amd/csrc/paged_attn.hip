@@ -49,6 +49,7 @@ typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef float f2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u2v __attribute__((ext_vector_type(2)));
 
 // waves per workgroup: 8 for one N tile (<= 256 VGPRs each), 4 for two N tiles (the second
 // tile's accumulators and operands need the full 512-register budget)
@@ -242,13 +243,74 @@ __device__ __forceinline__ constexpr int tq4_pv_elem(int h, int j, int r) {
     return 8 * r - 4 + j;
 }
 
-template <typename TQ, int NT>
-__global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(const AttnParams P) {
+constexpr int kMergeGroups = 16;
+constexpr int kMergeMaxPerGroup = 16;  // at most 256 partials per row
+
+// ---- balanced decode ----------------------------------------------------------------------------
+// A decode batch (at most one tile per request, no window, no token mask) is cut into equal
+// shares of 32-token units, one share per workgroup, whatever the lengths of the requests: the
+// units of all requests are laid end to end and workgroup x owns units [x S, (x + 1) S).  A share
+// that crosses a request boundary is worked off piece by piece.  Piece (x, r) gets partial slot
+// x + r: both grow along the pieces, so the slots are unique and those of one request are
+// consecutive, first_wg(r) + r .. last_wg(r) + r.  The plan is a function of the batch
+// descriptor alone; the merge kernel recomputes it instead of reading it from memory.
+// Starting a piece (table, query rotation, first loads, merge of the waves) costs about as much
+// as kBalPieceCost units of streaming, so every request is charged that many extra units in
+// front of its real ones: a share that contains request boundaries gets fewer keys.
+constexpr int kBalPieceCost = 24;
+__host__ __device__ __forceinline__ size_t bal_partial_row(int slot, int kv_subs, int kv_sub, int col) {
+    return ((size_t)slot * kv_subs + kv_sub) * 16 + col;
+}
+
+struct BalReq {  // request base + lane of a 64-request group
+    int lo, hi, sa, cb, units;
+    int cost;  // units + kBalPieceCost, 0 for a request without work
+};
+__device__ __forceinline__ BalReq bal_load_req(const AttnParams& P, int r) {
+    const warp34_attention_batch& B = P.B;
+    BalReq q{0, 0, 0, 0, 0, 0};
+    if (r >= B.num_reqs) return q;
+    q.lo = B.query_start_loc[r];
+    q.hi = B.query_start_loc[r + 1];
+    q.sa = B.seq_lens_after[r];
+    const int q_len = q.hi - q.lo;
+    q.cb = B.context_lens_before != nullptr ? B.context_lens_before[r] : q.sa - q_len;
+    const bool live = q_len > 0 && (B.valid_req_mask == nullptr || B.valid_req_mask[r] != 0);
+    int last = (B.mask_mode == WARP34_ATTN_MASK_NONCAUSAL_WINDOW) ? q.sa - 1 : q.cb + min(q_len, P.tok_tile) - 1;
+    if (last >= q.sa) last = q.sa - 1;
+    q.units = (live && last >= 0) ? (last >> 5) + 1 : 0;
+    q.cost = q.units > 0 ? q.units + kBalPieceCost : 0;
+    return q;
+}
+__device__ __forceinline__ int wave_incl_scan(int v, int lane) {
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int up = __shfl_up(v, off, 64);
+        if (lane >= off) v += up;
+    }
+    return v;
+}
+// units per share for a batch of `total` units over `groups` workgroups
+__device__ __forceinline__ int bal_share(int total, int groups, int min_share) {
+    int s = (total + groups - 1) / groups;
+    return s < min_share ? min_share : s;
+}
+
+// One piece of work of the balanced decode kernel: units [u_begin, u_end) of request `req`,
+// the piece number `slot` (partials of a request occupy consecutive slots) and the number of
+// pieces the request is cut into.
+struct BalItem {
+    int req, rq_start, rq_end, seq_after, ctx_before;
+    int u_begin, u_end, n_chunks, slot;
+};
+
+// The work of one workgroup on one tile.  BAL = false: the tile and the chunk come from
+// blockIdx (grid = chunks x (kv head, q subgroup) x tiles).  BAL = true: they come from `item`
+// (balanced decode: every workgroup owns an equal share of the batch's units).
+template <typename TQ, int NT, bool BAL>
+__device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, const BalItem& item) {
     constexpr int kWaves = waves_for(NT);
-    extern __shared__ __align__(16) uint8_t smem[];
     uint8_t* stage_all = smem + kLutBytes;  // kWaves * kStageTq4 bytes, reused by prologue/epilogue
-    // lut_read() addresses the table absolutely
-    if ((uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem != 0u) __builtin_trap();
 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
@@ -263,11 +325,11 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
     // every workgroup that is launched has work.  When no request can have more than one tile
     // (max_q_len <= tok_tile, e.g. decode) tile z is request z; otherwise the tile is located
     // with a prefix sum over the requests' tile counts.
-    const int tile_z = (int)blockIdx.z;
+    const int tile_z = BAL ? item.req : (int)blockIdx.z;
     const int kv_sub = (int)blockIdx.y;
     const int kv_head = fast_div(kv_sub, P.q_subgroups);
     const int q_head_base = kv_head * P.gqa + (kv_sub - kv_head * P.q_subgroups) * P.q_group;
-    const int chunk = (int)blockIdx.x;
+    const int chunk = BAL ? 0 : (int)blockIdx.x;
 
     W34_TP(0);
 
@@ -275,7 +337,8 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
     // the raw query rows of this wave's columns and the table.  The first token of the tile is
     // guessed (exact when every request has a whole number of tiles); a wrong guess is
     // corrected after the lookup.
-    const int tok_guess = min(P.tiles_by_request ? tile_z : tile_z * P.tok_tile, B.total_tokens - 1);
+    const int tok_guess = BAL ? item.rq_start
+                              : min(P.tiles_by_request ? tile_z : tile_z * P.tok_tile, B.total_tokens - 1);
     constexpr int kColsPerWave = (16 * NT + kWaves - 1) / kWaves;
     uint2 q_raw[kColsPerWave];
     auto load_q = [&](int tokbase) {
@@ -309,7 +372,14 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
     int req = -1, rq_start = 0, rq_end = 0, seq_after = 0, ctx_before = 0, tile_in_req = 0;
     int spec_slot_base = -1, spec_vec = -1;
     int a_lo = 0, a_hi = 0, a_sa = 0, a_cb = 0, a_rm = 0;
-    if (P.tiles_by_request) {
+    if constexpr (BAL) {
+        req = item.req;
+        rq_start = item.rq_start;
+        rq_end = item.rq_end;
+        seq_after = item.seq_after;
+        ctx_before = item.ctx_before;
+        req_hit = true;
+    } else if (P.tiles_by_request) {
         req = tile_z;  // < num_reqs by the launch geometry
         // Speculative block-table load, in flight together with the request's lengths: it
         // assumes that the request's length is the host's bound max_seq_len.  When the guess is
@@ -378,7 +448,7 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
         for (int k = 0; k < kBytesPerThread / 16; ++k) dst[k] = vv;
     }
 
-    if (P.tiles_by_request) {
+    if (!BAL && P.tiles_by_request) {
         rq_start = __builtin_amdgcn_readfirstlane(a_lo);
         rq_end = __builtin_amdgcn_readfirstlane(a_hi);
         seq_after = __builtin_amdgcn_readfirstlane(a_sa);
@@ -481,11 +551,20 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
     i_lo = __builtin_amdgcn_readfirstlane(i_lo);
     i_hi = __builtin_amdgcn_readfirstlane(i_hi);
 
-    const ChunkGeom g = chunk_geom(u_lo, u_hi, P.max_chunks, P.min_upc);
-    if (chunk >= g.n_chunks) return;
-    const int cu_first = g.u_first + chunk * g.upc;
-    int cu_end = cu_first + g.upc;
-    if (cu_end > g.u_first + g.n_units) cu_end = g.u_first + g.n_units;
+    ChunkGeom g;
+    int cu_first, cu_end;
+    if constexpr (BAL) {
+        // the plan counted the units of [0, u_hi]: the batch has no window and no token mask
+        g = ChunkGeom{0, (u_hi >> 5) + 1, 0, item.n_chunks};
+        cu_first = item.u_begin;
+        cu_end = item.u_end;
+    } else {
+        g = chunk_geom(u_lo, u_hi, P.max_chunks, P.min_upc);
+        if (chunk >= g.n_chunks) return;
+        cu_first = g.u_first + chunk * g.upc;
+        cu_end = cu_first + g.upc;
+        if (cu_end > g.u_first + g.n_units) cu_end = g.u_first + g.n_units;
+    }
     W34_TP(1);
 
     // ---- staging machinery ----------------------------------------------------------------------
@@ -587,23 +666,34 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
     __syncthreads();
     W34_TP(45);
 
-    // B operands of the QK MFMAs: 9 per N tile (5 for the first half-row, 4 for the second)
+    // B operands of the QK MFMAs: 9 per N tile (5 for the first half-row, 4 for the second).
+    // Operand (h, m) of k-block b pairs with row dword D = tq4_qk_dword(h, m, b); its eight
+    // elements (tq4_dword_elem) are contiguous in the query row, so they are fetched with 64-
+    // and 128-bit reads: dword D < 16 covers elements 8 D - 4 .. 8 D + 3 (the first four are
+    // scale nibbles for D = 0), dword 16 elements 124 .. 127 and two scale nibbles' worth of
+    // zeros, dword 17 + k elements 128 + 8 k .. 128 + 8 k + 7.
     h8 bq[NT][9];
+    {
+        const int kb = 8 * (b & 1) + 4 * (b >> 1);  // first dword of this k-block
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
+        for (int nt = 0; nt < NT; ++nt) {
+            const uint8_t* qrow = reinterpret_cast<const uint8_t*>(qlds + (nt * 16 + n) * kQStride);
 #pragma unroll
-        for (int mf = 0; mf < 9; ++mf) {
-            const int h = mf < 5 ? 0 : 1;
-            const int m = mf < 5 ? mf : mf - 5;
-            const int D = tq4_qk_dword(h, m, b);
-            const bool dummy = (h == 0 && m == 4 && b != 0);
-            h8 x;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int e = dummy ? -1 : tq4_dword_elem(D, i);
-                x[i] = e >= 0 ? qlds[(nt * 16 + n) * kQStride + e] : (_Float16)0.0f;
+            for (int m = 0; m < 4; ++m) {
+                const int D = kb + m;
+                u2v lo = *reinterpret_cast<const u2v*>(qrow + (D > 0 ? 16 * D - 8 : 0));
+                if (D == 0) lo = u2v{0u, 0u};
+                const u2v hi = *reinterpret_cast<const u2v*>(qrow + 16 * D);
+                bq[nt][m] = __builtin_bit_cast(h8, u4{lo[0], lo[1], hi[0], hi[1]});
             }
-            bq[nt][mf] = x;
+            {
+                u2v lo = *reinterpret_cast<const u2v*>(qrow + 248);
+                if (b != 0) lo = u2v{0u, 0u};
+                bq[nt][4] = __builtin_bit_cast(h8, u4{lo[0], lo[1], 0u, 0u});
+            }
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+                bq[nt][5 + m] = *reinterpret_cast<const h8*>(qrow + 256 + 16 * (kb + m));
         }
     }
     W34_TP(46);
@@ -928,15 +1018,16 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
         }
         const float m_col = mltot[col * 2 + 0];
         const float l_col = mltot[col * 2 + 1];
-        if (P.max_chunks > 1) {
+        if (BAL ? item.n_chunks > 1 : P.max_chunks > 1) {
             // un-normalised, rotated, still carrying the table gain; the merge kernel finishes
-            float* dst = P.part_acc + (row * P.max_chunks + chunk) * kHeadDim;
+            const size_t prow = BAL ? bal_partial_row(item.slot, (int)gridDim.y, kv_sub, col)
+                                    : row * P.max_chunks + chunk;
+            float* dst = P.part_acc + prow * kHeadDim;
             *reinterpret_cast<f4*>(dst + 4 * lane) = f4{v[0], v[1], v[2], v[3]};
             if (lane == 0) {
                 // (m, l, number of chunks of this row, -): one record per chunk, every record
                 // carries the count so the merge needs no dependent load
-                *reinterpret_cast<f4*>(P.part_ml + (row * P.max_chunks + chunk) * 4) =
-                    f4{m_col, l_col, (float)g.n_chunks, 0.f};
+                *reinterpret_cast<f4*>(P.part_ml + prow * 4) = f4{m_col, l_col, (float)g.n_chunks, 0.f};
             }
         } else {
             const float inv = l_col > 0.f ? kLutInvGain / l_col : 0.f;
@@ -954,6 +1045,196 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
     W34_TP(40);
 }
 
+template <typename TQ, int NT>
+__global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(const AttnParams P) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    // lut_read() addresses the table absolutely
+    if ((uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem != 0u) __builtin_trap();
+    tq4_tile<TQ, NT, false>(P, smem, BalItem{});
+}
+
+// Balanced decode: grid = (groups, kv head x q subgroup).  Every wave computes the plan (the
+// loads are the same addresses in every wave of the chip and stay in cache).
+template <typename TQ>
+__global__ __launch_bounds__(waves_for(1) * 64, 1) void paged_attn_tq4_balanced_kernel(const AttnParams P) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    if ((uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem != 0u) __builtin_trap();
+    const int lane = (int)threadIdx.x & 63;
+#ifdef W34_TRACE
+    const int wave = (int)threadIdx.x >> 6;
+#endif
+    W34_TP(60);
+    const int num_reqs = P.B.num_reqs;
+    int total = 0;
+    for (int base = 0; base < num_reqs; base += 64)
+        total += __builtin_amdgcn_readlane(wave_incl_scan(bal_load_req(P, base + lane).cost, lane), 63);
+    const int share = bal_share(total, (int)gridDim.x, P.min_upc + kBalPieceCost);
+    const int my_begin = (int)blockIdx.x * share;
+    int my_end = my_begin + share;
+    if (my_end > total) my_end = total;
+    if (my_begin >= total) return;
+
+    // The pieces of this share, in order.  Nothing but a few scalars stays live across a tile:
+    // the 64-request group that holds the next piece is loaded and scanned again after each one.
+    int base = 0, before = 0, taken = 0;  // group, units before it, pieces of it already done
+    W34_TP(59);
+#ifdef W34_TRACE
+    int n_items = 0;
+#endif
+    while (base < num_reqs && before < my_end) {
+        BalItem it;
+        bool have = false;
+        int group_units = 0;
+        {
+            const BalReq q = bal_load_req(P, base + lane);
+            const int incl = wave_incl_scan(q.cost, lane);
+            const int start = before + incl - q.units;  // of the real units, behind the charge
+            unsigned long long hits = __ballot(q.units > 0 && start < my_end && start + q.units > my_begin);
+            for (int skip = 0; skip < taken && hits != 0ull; ++skip) hits &= hits - 1ull;
+            group_units = __builtin_amdgcn_readlane(incl, 63);
+            if (hits != 0ull) {
+                const int src = __builtin_ctzll(hits);
+                const int r_start = __builtin_amdgcn_readlane(start, src);
+                const int r_units = __builtin_amdgcn_readlane(q.units, src);
+                it.req = base + src;
+                it.rq_start = __builtin_amdgcn_readlane(q.lo, src);
+                it.rq_end = __builtin_amdgcn_readlane(q.hi, src);
+                it.seq_after = __builtin_amdgcn_readlane(q.sa, src);
+                it.ctx_before = __builtin_amdgcn_readlane(q.cb, src);
+                it.u_begin = max(my_begin, r_start) - r_start;
+                it.u_end = min(my_end, r_start + r_units) - r_start;
+                it.n_chunks = (r_start + r_units - 1) / share - r_start / share + 1;
+                it.slot = (int)blockIdx.x + it.req;
+                have = true;
+            }
+        }
+        if (!have) {
+            before += group_units;
+            base += 64;
+            taken = 0;
+            continue;
+        }
+        ++taken;
+        tq4_tile<TQ, 1, true>(P, smem, it);
+        __syncthreads();  // the tile's merge regions alias the table the next piece rebuilds
+#ifdef W34_TRACE
+        ++n_items;
+        W34_TP(52 + (n_items < 6 ? n_items : 6));
+#endif
+    }
+    W34_TP(61);
+}
+
+// Merge for the balanced decode kernel: one workgroup of 1024 threads per (token, q head) row.
+// Wave 0 recomputes the plan for the row's request; rows whose request was not cut (one piece)
+// were finished by the attention kernel, rows of requests without visible keys are zero.
+template <typename TQ>
+__global__ __launch_bounds__(1024) void balanced_merge_kernel(const AttnParams P, int groups, int kv_subs,
+                                                              float out_scale) {
+    __shared__ f4 s_acc[kMergeGroups][64];
+    __shared__ f4 s_rec[256];
+    __shared__ float s_red[kMergeGroups];
+    __shared__ int s_plan[4];  // valid, first slot, pieces, column
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int grp = tid >> 6;
+    const long long row = (long long)blockIdx.x;
+    const int tok = (int)(row / P.num_q_heads);
+    const int head = (int)(row - (long long)tok * P.num_q_heads);
+    const warp34_attention_batch& B = P.B;
+    if (grp == 0) {
+        int total = 0, r_found = -1, r_start = 0, r_units = 0, r_lo = 0;
+        for (int base = 0; base < B.num_reqs; base += 64) {
+            const BalReq q = bal_load_req(P, base + lane);
+            const int incl = wave_incl_scan(q.cost, lane);
+            const unsigned long long hits = __ballot(base + lane < B.num_reqs && tok >= q.lo && tok < q.hi);
+            if (hits != 0ull && r_found < 0) {
+                const int src = __builtin_ctzll(hits);
+                r_found = base + src;
+                r_start = total + __builtin_amdgcn_readlane(incl - q.units, src);
+                r_units = __builtin_amdgcn_readlane(q.units, src);
+                r_lo = __builtin_amdgcn_readlane(q.lo, src);
+            }
+            total += __builtin_amdgcn_readlane(incl, 63);
+        }
+        const bool req_ok = r_found >= 0 && (B.valid_req_mask == nullptr || B.valid_req_mask[max(r_found, 0)] != 0);
+        const int share = bal_share(total, groups, P.min_upc + kBalPieceCost);
+        const int first_wg = r_start / share;
+        const int pieces = r_units > 0 ? (r_start + r_units - 1) / share - first_wg + 1 : 0;
+        if (lane == 0) {
+            s_plan[0] = req_ok ? 1 : 0;
+            s_plan[1] = first_wg + r_found;
+            s_plan[2] = pieces;
+            s_plan[3] = (tok - r_lo) * P.q_group + head % P.q_group;
+        }
+    }
+    __syncthreads();
+    if (!s_plan[0]) return;  // masked request: output untouched
+    const int n_chunks = s_plan[2];
+    if (n_chunks == 1) return;  // finished by the attention kernel
+    if (n_chunks == 0) {        // no visible key: zeros
+        if (grp == 0) *reinterpret_cast<uint2*>(P.out + (size_t)row * kHeadDim + 4 * lane) = uint2{0u, 0u};
+        return;
+    }
+    const int kv_sub = head / P.q_group;  // = kv_head * q_subgroups + subgroup
+    const size_t prow0 = bal_partial_row(s_plan[1], kv_subs, kv_sub, s_plan[3]);
+    const size_t pstride = (size_t)kv_subs * 16;  // partial rows between consecutive slots
+    if (tid < n_chunks && tid < 256) s_rec[tid] = *reinterpret_cast<const f4*>(P.part_ml + (prow0 + tid * pstride) * 4);
+    f4 a[kMergeMaxPerGroup];
+#pragma unroll
+    for (int k = 0; k < kMergeMaxPerGroup; ++k) {
+        const int s = grp + k * kMergeGroups;
+        a[k] = f4{0.f, 0.f, 0.f, 0.f};
+        if (s < n_chunks) a[k] = *reinterpret_cast<const f4*>(P.part_acc + (prow0 + s * pstride) * kHeadDim + 4 * lane);
+    }
+    __syncthreads();
+    float m_tot = kNegBig;
+    for (int s = lane; s < n_chunks; s += 64) {
+        const f4 r = s_rec[s];
+        if (r[1] > 0.f) m_tot = fmaxf(m_tot, r[0]);
+    }
+    m_tot = fmaxf(m_tot, lane_xor<1>(m_tot, lane));
+    m_tot = fmaxf(m_tot, lane_xor<2>(m_tot, lane));
+    m_tot = fmaxf(m_tot, lane_xor<4>(m_tot, lane));
+    m_tot = fmaxf(m_tot, lane_xor<8>(m_tot, lane));
+    m_tot = fmaxf(m_tot, lane_xor<16>(m_tot, lane));
+    m_tot = fmaxf(m_tot, lane_xor<32>(m_tot, lane));
+    f4 v = {0.f, 0.f, 0.f, 0.f};
+    float l_part = 0.f;
+#pragma unroll
+    for (int k = 0; k < kMergeMaxPerGroup; ++k) {
+        const int s = grp + k * kMergeGroups;
+        if (s < n_chunks) {
+            const f4 r = s_rec[s];
+            if (r[1] > 0.f) {
+                const float w = __builtin_amdgcn_exp2f(r[0] - m_tot);
+                l_part += r[1] * w;
+                v += a[k] * w;
+            }
+        }
+    }
+    s_acc[grp][lane] = v;
+    if (lane == 0) s_red[grp] = l_part;
+    __syncthreads();
+    if (grp != 0) return;
+    float l_tot = 0.f;
+    f4 tot = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k = 0; k < kMergeGroups; ++k) {
+        tot += s_acc[k][lane];
+        l_tot += s_red[k];
+    }
+    const float inv = l_tot > 0.f ? out_scale / l_tot : 0.f;
+    float o[4] = {tot[0] * inv, tot[1] * inv, tot[2] * inv, tot[3] * inv};
+    wht256_wave(o, lane);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) o[k] = apply_sign(o[k], 4 * lane + k);
+    uint2 ob;
+    ob.x = (uint32_t)TQ::from_f32(o[0]) | ((uint32_t)TQ::from_f32(o[1]) << 16);
+    ob.y = (uint32_t)TQ::from_f32(o[2]) | ((uint32_t)TQ::from_f32(o[3]) << 16);
+    *reinterpret_cast<uint2*>(P.out + (size_t)row * kHeadDim + 4 * lane) = ob;
+}
+
 #ifdef W34_TRACE
 extern "C" int warp34_debug_read_trace(unsigned long long* dst) {
     return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_trace), sizeof(unsigned long long) * 64 * 64);
@@ -967,8 +1248,6 @@ extern "C" int warp34_debug_read_trace(unsigned long long* dst) {
 // Everything the row needs (validity, chunk records, accumulators) is requested in ONE memory
 // round trip: records and accumulators of all max_chunks slots are loaded speculatively and
 // the slots beyond the row's chunk count are discarded with selects.
-constexpr int kMergeGroups = 16;
-constexpr int kMergeMaxPerGroup = 16;  // max_chunks <= 256
 template <typename TQ>
 __global__ __launch_bounds__(1024) void split_merge_kernel(const float* part_acc_in, const float* part_ml_in,
                                                            int max_chunks_in, const AttnParams P,
@@ -1145,6 +1424,7 @@ namespace w34 {
 constexpr int kMaxChunksCap = 256;
 constexpr int kMinUnitsPerChunk = 16;  // 512 tokens: two units per wave
 constexpr int kTargetWorkgroupsPerHead = 128;
+constexpr int kBalWorkgroups = 256;  // balanced decode: one workgroup per compute unit
 
 static size_t partial_bytes(long long rows, int max_chunks) {
     return (size_t)rows * (size_t)max_chunks * (kHeadDim + 4) * sizeof(float);
@@ -1231,9 +1511,34 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     // sum_r ceil(q_r / tok_tile) <= total_tokens / tok_tile + num_reqs
     P.tiles_by_request = (batch->max_q_len > 0 && batch->max_q_len <= P.tok_tile) ? 1 : 0;
     const int grid_z = P.tiles_by_request ? batch->num_reqs : batch->total_tokens / P.tok_tile + batch->num_reqs;
-    const dim3 grid((unsigned)grid_x, (unsigned)(layout->local_kv_heads * P.q_subgroups), (unsigned)grid_z);
+    const int kv_subs = layout->local_kv_heads * P.q_subgroups;
+    const dim3 grid((unsigned)grid_x, (unsigned)kv_subs, (unsigned)grid_z);
     hipStream_t stream = (hipStream_t)ex->stream;
     int rc;
+    // Decode batches of several requests: equal shares of the batch's units per workgroup
+    // instead of per-request chunks (the requests' lengths are unknown to the host and differ).
+    if (P.tiles_by_request && batch->num_reqs >= 2 && !force_single && batch->sliding_window <= 0 &&
+        batch->valid_token_mask == nullptr && ex->scratch_ptr != 0 && (ex->scratch_ptr & 15u) == 0u) {
+        static const int bal_wg_env = getenv("W34_BAL_WG") ? atoi(getenv("W34_BAL_WG")) : kBalWorkgroups;
+        int groups = bal_wg_env / kv_subs;
+        if (groups > kMergeGroups * kMergeMaxPerGroup - 1) groups = kMergeGroups * kMergeMaxPerGroup - 1;
+        if (groups < 1) groups = 1;
+        const size_t prows = bal_partial_row(groups + batch->num_reqs, kv_subs, 0, 0);
+        if (partial_bytes((long long)prows, 1) <= ex->scratch_size) {
+            P.part_acc = reinterpret_cast<float*>((uintptr_t)ex->scratch_ptr);
+            P.part_ml = P.part_acc + prows * kHeadDim;
+            P.max_chunks = groups + 1;
+            rc = ensure_dynamic_lds(paged_attn_tq4_balanced_kernel<TQ>, smem_bytes_for(1));
+            if (rc) return rc;
+            hipLaunchKernelGGL((paged_attn_tq4_balanced_kernel<TQ>), dim3((unsigned)groups, (unsigned)kv_subs),
+                               dim3(waves_for(1) * 64), smem_bytes_for(1), stream, P);
+            rc = (int)hipGetLastError();
+            if (rc) return rc;
+            hipLaunchKernelGGL((balanced_merge_kernel<TQ>), dim3((unsigned)rows), dim3(1024), 0, stream, P, groups,
+                               kv_subs, kLutInvGain);
+            return (int)hipGetLastError();
+        }
+    }
     rc = ensure_dynamic_lds(paged_attn_tq4_kernel<TQ, 1>, smem_bytes_for(1));
     if (rc) return rc;
     hipLaunchKernelGGL((paged_attn_tq4_kernel<TQ, 1>), grid, dim3(waves_for(1) * 64), smem_bytes_for(1), stream, P);
@@ -1490,5 +1795,10 @@ extern "C" size_t warp34_paged_attention_scratch_bytes(int total_tokens, int num
     int want = kTargetWorkgroupsPerHead / total_tokens;
     if (want > kMaxChunksCap) want = kMaxChunksCap;
     if (want < 2) want = 2;
-    return partial_bytes((long long)total_tokens * num_q_heads, want);
+    size_t bytes = partial_bytes((long long)total_tokens * num_q_heads, want);
+    // balanced decode: (workgroups + requests) partial slots of 16 columns per (kv head, q subgroup);
+    // requests <= total_tokens and subgroups <= num_q_heads bound it without the layout
+    const size_t bal = partial_bytes(((long long)kBalWorkgroups + (long long)total_tokens * num_q_heads) * 16, 1);
+    if (total_tokens >= 2 && bal > bytes) bytes = bal;
+    return bytes;
 }

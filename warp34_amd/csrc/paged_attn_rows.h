@@ -25,7 +25,6 @@ namespace w34 {
 typedef _Float16 h4 __attribute__((ext_vector_type(4)));
 typedef short s4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
-typedef uint32_t u2v __attribute__((ext_vector_type(2)));
 
 constexpr int kKv16Waves = 8;
 constexpr int kKv16RowStride = 528;                      // bytes, 512 + 16 pad
