@@ -34,6 +34,7 @@ WORKLOADS = {
     # the un-rotated 8-bit rows the default TQ4 policy keeps for its last four layers
     "fp8_decode_b1_ctx131072": ("fp8", [131072], 0),
     "q8_0_decode_b1_ctx131072": ("q8_0", [131072], 0),
+    "fp8_decode_b32_ctx1k_64k": ("fp8", None, 2 << 20),
     # 8 sequences, 16 384-token TQ4 prefix + 2 048-token bf16 chunk each: append + causal attention
     "tq4_prefill_8x2048_ctx16384": ("tq4", [18432] * 8, 0),
     "fp8_prefill_8x2048_ctx16384": ("fp8", [18432] * 8, 0),

@@ -273,6 +273,17 @@ def test_kv8_windows(fmt, mask_mode, window):
     _check(fmt, DT_F16, 16, [333, 90], [3, 2], 251, mask_mode=mask_mode, window=window, ctx_null=True)
 
 
+@pytest.mark.parametrize("fmt,dtype,xf", [(FMT_FP8, DT_BF16, XF_IDENTITY), (FMT_Q8_0, DT_F16, XF_WHT256),
+                                          (FMT_BF16, DT_BF16, XF_IDENTITY), (FMT_FP16, DT_F16, XF_IDENTITY)])
+def test_rows_decode_batch_balanced_shares(fmt, dtype, xf):
+    """Decode batches with very different request lengths over 16-bit and 8-bit pages: equal
+    shares of units per workgroup, long requests cut into many pieces, several short requests
+    worked off by one workgroup."""
+    seq = [5000, 300, 9000, 64, 2500, 33, 1, 7777]
+    _check(fmt, dtype, 64, seq, [1] * len(seq), 281, q_heads=16, xf=xf)
+    _check(fmt, dtype, 16, seq[:5], [2, 1, 2, 1, 2], 282, q_heads=8, xf=xf)
+
+
 @pytest.mark.parametrize("fmt", KV8)
 @pytest.mark.parametrize("scratch", [0, SCRATCH])
 def test_kv8_rotated_rows(fmt, scratch):

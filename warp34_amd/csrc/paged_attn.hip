@@ -257,7 +257,7 @@ constexpr int kMergeMaxPerGroup = 16;  // at most 256 partials per row
 // Starting a piece (table, query rotation, first loads, merge of the waves) costs about as much
 // as kBalPieceCost units of streaming, so every request is charged that many extra units in
 // front of its real ones: a share that contains request boundaries gets fewer keys.
-constexpr int kBalPieceCost = 24;
+constexpr int kBalPieceCost = 32;
 __host__ __device__ __forceinline__ size_t bal_partial_row(int slot, int kv_subs, int kv_sub, int col) {
     return ((size_t)slot * kv_subs + kv_sub) * 16 + col;
 }
@@ -1054,11 +1054,10 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
 }
 
 // Balanced decode: grid = (groups, kv head x q subgroup).  Every wave computes the plan (the
-// loads are the same addresses in every wave of the chip and stay in cache).
-template <typename TQ>
-__global__ __launch_bounds__(waves_for(1) * 64, 1) void paged_attn_tq4_balanced_kernel(const AttnParams P) {
-    extern __shared__ __align__(16) uint8_t smem[];
-    if ((uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem != 0u) __builtin_trap();
+// loads are the same addresses in every wave of the chip and stay in cache) and calls
+// tile(piece) for the pieces of its workgroup's share, in order.
+template <typename TileFn>
+__device__ __forceinline__ void bal_for_each_piece(const AttnParams& P, TileFn&& tile) {
     const int lane = (int)threadIdx.x & 63;
 #ifdef W34_TRACE
     const int wave = (int)threadIdx.x >> 6;
@@ -1078,13 +1077,10 @@ __global__ __launch_bounds__(waves_for(1) * 64, 1) void paged_attn_tq4_balanced_
     // the 64-request group that holds the next piece is loaded and scanned again after each one.
     int base = 0, before = 0, taken = 0;  // group, units before it, pieces of it already done
     W34_TP(59);
-#ifdef W34_TRACE
-    int n_items = 0;
-#endif
     while (base < num_reqs && before < my_end) {
         BalItem it;
         bool have = false;
-        int group_units = 0;
+        int group_units = 0, piece_end = 0;
         {
             const BalReq q = bal_load_req(P, base + lane);
             const int incl = wave_incl_scan(q.cost, lane);
@@ -1105,6 +1101,7 @@ __global__ __launch_bounds__(waves_for(1) * 64, 1) void paged_attn_tq4_balanced_
                 it.u_end = min(my_end, r_start + r_units) - r_start;
                 it.n_chunks = (r_start + r_units - 1) / share - r_start / share + 1;
                 it.slot = (int)blockIdx.x + it.req;
+                piece_end = r_start + it.u_end;
                 have = true;
             }
         }
@@ -1115,14 +1112,18 @@ __global__ __launch_bounds__(waves_for(1) * 64, 1) void paged_attn_tq4_balanced_
             continue;
         }
         ++taken;
-        tq4_tile<TQ, 1, true>(P, smem, it);
-        __syncthreads();  // the tile's merge regions alias the table the next piece rebuilds
-#ifdef W34_TRACE
-        ++n_items;
-        W34_TP(52 + (n_items < 6 ? n_items : 6));
-#endif
+        tile(it);
+        if (piece_end >= my_end) break;  // the share ends with this piece
+        __syncthreads();  // the tile's merge regions alias what the next piece sets up
     }
     W34_TP(61);
+}
+
+template <typename TQ>
+__global__ __launch_bounds__(waves_for(1) * 64, 1) void paged_attn_tq4_balanced_kernel(const AttnParams P) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    if ((uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem != 0u) __builtin_trap();
+    bal_for_each_piece(P, [&](const BalItem& it) { tq4_tile<TQ, 1, true>(P, smem, it); });
 }
 
 // Merge for the balanced decode kernel: one workgroup of 1024 threads per (token, q head) row.
@@ -1130,7 +1131,7 @@ __global__ __launch_bounds__(waves_for(1) * 64, 1) void paged_attn_tq4_balanced_
 // were finished by the attention kernel, rows of requests without visible keys are zero.
 template <typename TQ>
 __global__ __launch_bounds__(1024) void balanced_merge_kernel(const AttnParams P, int groups, int kv_subs,
-                                                              float out_scale) {
+                                                              float out_scale, int rotate) {
     __shared__ f4 s_acc[kMergeGroups][64];
     __shared__ f4 s_rec[256];
     __shared__ float s_red[kMergeGroups];
@@ -1226,9 +1227,11 @@ __global__ __launch_bounds__(1024) void balanced_merge_kernel(const AttnParams P
     }
     const float inv = l_tot > 0.f ? out_scale / l_tot : 0.f;
     float o[4] = {tot[0] * inv, tot[1] * inv, tot[2] * inv, tot[3] * inv};
-    wht256_wave(o, lane);
+    if (rotate) {
+        wht256_wave(o, lane);
 #pragma unroll
-    for (int k = 0; k < 4; ++k) o[k] = apply_sign(o[k], 4 * lane + k);
+        for (int k = 0; k < 4; ++k) o[k] = apply_sign(o[k], 4 * lane + k);
+    }
     uint2 ob;
     ob.x = (uint32_t)TQ::from_f32(o[0]) | ((uint32_t)TQ::from_f32(o[1]) << 16);
     ob.y = (uint32_t)TQ::from_f32(o[2]) | ((uint32_t)TQ::from_f32(o[3]) << 16);
@@ -1463,6 +1466,19 @@ static int ensure_dynamic_lds(KernelT kernel, int bytes) {
     return 0;
 }
 
+// Decode batches of several requests take the balanced path: no request has more than one
+// tile, no window, no token mask (the plan counts units of [0, last key]), usable scratch.
+static bool balanced_decode_applicable(const warp34_exec* ex, const warp34_attention_batch* batch,
+                                       int tiles_by_request, int force_single) {
+    return tiles_by_request && batch->num_reqs >= 2 && !force_single && batch->sliding_window <= 0 &&
+           batch->valid_token_mask == nullptr && ex->scratch_ptr != 0 && (ex->scratch_ptr & 15u) == 0u;
+}
+static int balanced_groups(int kv_subs) {
+    int groups = kBalWorkgroups / kv_subs;
+    if (groups > kMergeGroups * kMergeMaxPerGroup - 1) groups = kMergeGroups * kMergeMaxPerGroup - 1;
+    return groups < 1 ? 1 : groups;
+}
+
 template <typename TQ>
 static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
                       const warp34_attention_batch* batch, const void* q, void* out, int num_q_heads,
@@ -1517,12 +1533,8 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     int rc;
     // Decode batches of several requests: equal shares of the batch's units per workgroup
     // instead of per-request chunks (the requests' lengths are unknown to the host and differ).
-    if (P.tiles_by_request && batch->num_reqs >= 2 && !force_single && batch->sliding_window <= 0 &&
-        batch->valid_token_mask == nullptr && ex->scratch_ptr != 0 && (ex->scratch_ptr & 15u) == 0u) {
-        static const int bal_wg_env = getenv("W34_BAL_WG") ? atoi(getenv("W34_BAL_WG")) : kBalWorkgroups;
-        int groups = bal_wg_env / kv_subs;
-        if (groups > kMergeGroups * kMergeMaxPerGroup - 1) groups = kMergeGroups * kMergeMaxPerGroup - 1;
-        if (groups < 1) groups = 1;
+    if (balanced_decode_applicable(ex, batch, P.tiles_by_request, force_single)) {
+        const int groups = balanced_groups(kv_subs);
         const size_t prows = bal_partial_row(groups + batch->num_reqs, kv_subs, 0, 0);
         if (partial_bytes((long long)prows, 1) <= ex->scratch_size) {
             P.part_acc = reinterpret_cast<float*>((uintptr_t)ex->scratch_ptr);
@@ -1535,7 +1547,7 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
             rc = (int)hipGetLastError();
             if (rc) return rc;
             hipLaunchKernelGGL((balanced_merge_kernel<TQ>), dim3((unsigned)rows), dim3(1024), 0, stream, P, groups,
-                               kv_subs, kLutInvGain);
+                               kv_subs, kLutInvGain, 1);
             return (int)hipGetLastError();
         }
     }
@@ -1595,9 +1607,29 @@ static int launch_rows(const warp34_exec* ex, const warp34_kv_layer_layout* layo
     P.rot_q = layout->k_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 ? 1 : 0;
     P.rot_out = layout->v_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 ? 1 : 0;
     const int grid_z = P.tiles_by_request ? batch->num_reqs : batch->total_tokens / P.tok_tile + batch->num_reqs;
-    const dim3 grid((unsigned)grid_x, (unsigned)(layout->local_kv_heads * P.q_subgroups), (unsigned)grid_z);
+    const int kv_subs = layout->local_kv_heads * P.q_subgroups;
+    const dim3 grid((unsigned)grid_x, (unsigned)kv_subs, (unsigned)grid_z);
     hipStream_t stream = (hipStream_t)ex->stream;
-    int rc = ensure_dynamic_lds(paged_attn_rows_kernel<TQ, 1, KVF>, kv16_smem_bytes(1));
+    int rc;
+    if (balanced_decode_applicable(ex, batch, P.tiles_by_request, force_single)) {
+        const int groups = balanced_groups(kv_subs);
+        const size_t prows = bal_partial_row(groups + batch->num_reqs, kv_subs, 0, 0);
+        if (partial_bytes((long long)prows, 1) <= ex->scratch_size) {
+            P.part_acc = reinterpret_cast<float*>((uintptr_t)ex->scratch_ptr);
+            P.part_ml = P.part_acc + prows * kHeadDim;
+            P.max_chunks = groups + 1;
+            rc = ensure_dynamic_lds(paged_attn_rows_balanced_kernel<TQ, KVF>, kv16_smem_bytes(1));
+            if (rc) return rc;
+            hipLaunchKernelGGL((paged_attn_rows_balanced_kernel<TQ, KVF>), dim3((unsigned)groups, (unsigned)kv_subs),
+                               dim3(kKv16Waves * 64), kv16_smem_bytes(1), stream, P);
+            rc = (int)hipGetLastError();
+            if (rc) return rc;
+            hipLaunchKernelGGL((balanced_merge_kernel<TQ>), dim3((unsigned)rows), dim3(1024), 0, stream, P, groups,
+                               kv_subs, 1.0f, P.rot_out);
+            return (int)hipGetLastError();
+        }
+    }
+    rc = ensure_dynamic_lds(paged_attn_rows_kernel<TQ, 1, KVF>, kv16_smem_bytes(1));
     if (rc) return rc;
     hipLaunchKernelGGL((paged_attn_rows_kernel<TQ, 1, KVF>), grid, dim3(kKv16Waves * 64), kv16_smem_bytes(1), stream, P);
     rc = (int)hipGetLastError();

@@ -89,8 +89,10 @@ __device__ __forceinline__ f4 mfma_x16(u2v a, u2v b, f4 c) {
 // KVF is the storage format of both slabs.  16-bit pages: TQ doubles as the storage type (F16
 // query/output over FP16 pages, BF16 over BF16 pages).  8-bit pages: the MFMAs run in fp16 and
 // a BF16 query is converted once.
-template <typename TQ, int NT, int KVF>
-__global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_rows_kernel(const AttnParams P) {
+// BAL: the tile and its unit range come from `item` (balanced decode, see bal_for_each_piece)
+// instead of blockIdx.
+template <typename TQ, int NT, int KVF, bool BAL>
+__device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, const BalItem& item) {
     constexpr bool K8 = KVF == WARP34_KV_FORMAT_FP8_E4M3 || KVF == WARP34_KV_FORMAT_Q8_0;
     constexpr bool FP8 = KVF == WARP34_KV_FORMAT_FP8_E4M3;
     static_assert(K8 || KVF == TQ::kStorageFormat, "16-bit pages are read in the query type");
@@ -99,7 +101,6 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_rows_kernel(con
     constexpr int kWaves = kKv16Waves;
     constexpr int kRowStride = K8 ? kKv8RowStride : kKv16RowStride;  // LDS row stride
     constexpr int kRowBytes = K8 ? (FP8 ? 264 : 272) : 512;          // row in memory
-    extern __shared__ __align__(16) uint8_t smem[];
 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
@@ -109,17 +110,18 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_rows_kernel(con
     const warp34_kv_layer_layout& L = P.L;
     const warp34_attention_batch& B = P.B;
 
-    const int tile_z = (int)blockIdx.z;  // tile index (see locate_tile)
+    const int tile_z = BAL ? item.req : (int)blockIdx.z;  // tile index (see locate_tile)
     const int kv_sub = (int)blockIdx.y;
     const int kv_head = fast_div(kv_sub, P.q_subgroups);
     const int q_head_base = kv_head * P.gqa + (kv_sub - kv_head * P.q_subgroups) * P.q_group;
-    const int chunk = (int)blockIdx.x;
+    const int chunk = BAL ? 0 : (int)blockIdx.x;
 
     // query rows in MFMA B layout straight from global memory: lane (n, b) holds
     // Q[column n][32 m + 8 b .. + 7] for m = 0..7 (dead columns are zeroed below).  The first
     // token of the tile is guessed so that these loads overlap the lookup; a wrong guess is
     // corrected after it.
-    const int tok_guess = min(P.tiles_by_request ? tile_z : tile_z * P.tok_tile, B.total_tokens - 1);
+    const int tok_guess = BAL ? item.rq_start
+                              : min(P.tiles_by_request ? tile_z : tile_z * P.tok_tile, B.total_tokens - 1);
     u4 bq[NT][8];
     auto load_q = [&](int tokbase) {
 #pragma unroll
@@ -170,14 +172,19 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_rows_kernel(con
     // request's length is the host's bound max_seq_len.  A wrong guess is fetched again below,
     // so it changes the latency only, never the result.
     int spec_slot_base = -1, spec_vec = -1;
-    if (P.tiles_by_request && B.sliding_window <= 0 && B.max_seq_len > 0) {
+    if (!BAL && P.tiles_by_request && B.sliding_window <= 0 && B.max_seq_len > 0) {
         const ChunkGeom sg = chunk_geom(0, B.max_seq_len - 1, P.max_chunks, P.min_upc);
         spec_slot_base = fast_div((sg.u_first + chunk * sg.upc) * kUnit, L.block_size);
         const int slot = spec_slot_base + lane;
         if (slot < B.max_blocks_per_req)
             spec_vec = B.block_tables[(size_t)tile_z * B.max_blocks_per_req + slot];
     }
-    const TileInfo ti = locate_tile(P, tile_z, lane);
+    TileInfo ti;
+    if constexpr (BAL) {
+        ti = TileInfo{true, item.req, item.rq_start, item.rq_end, item.seq_after, item.ctx_before, 0};
+    } else {
+        ti = locate_tile(P, tile_z, lane);
+    }
     if (!ti.hit) return;  // no such tile, empty or masked request: outputs untouched
     const int req = ti.req, rq_start = ti.rq_start, rq_end = ti.rq_end;
     const int seq_after = ti.seq_after, ctx_before = ti.ctx_before;
@@ -259,11 +266,20 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_rows_kernel(con
     i_lo = __builtin_amdgcn_readfirstlane(i_lo);
     i_hi = __builtin_amdgcn_readfirstlane(i_hi);
 
-    const ChunkGeom g = chunk_geom(u_lo, u_hi, P.max_chunks, P.min_upc);
-    if (chunk >= g.n_chunks) return;
-    const int cu_first = g.u_first + chunk * g.upc;
-    int cu_end = cu_first + g.upc;
-    if (cu_end > g.u_first + g.n_units) cu_end = g.u_first + g.n_units;
+    ChunkGeom g;
+    int cu_first, cu_end;
+    if constexpr (BAL) {
+        // the plan counted the units of [0, u_hi]: the batch has no window and no token mask
+        g = ChunkGeom{0, (u_hi >> 5) + 1, 0, item.n_chunks};
+        cu_first = item.u_begin;
+        cu_end = item.u_end;
+    } else {
+        g = chunk_geom(u_lo, u_hi, P.max_chunks, P.min_upc);
+        if (chunk >= g.n_chunks) return;
+        cu_first = g.u_first + chunk * g.upc;
+        cu_end = cu_first + g.upc;
+        if (cu_end > g.u_first + g.n_units) cu_end = g.u_first + g.n_units;
+    }
 
     const uint8_t* k_base = reinterpret_cast<const uint8_t*>((uintptr_t)L.k_base) +
                             (size_t)kv_head * L.k_head_stride_bytes;
@@ -627,12 +643,13 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_rows_kernel(con
         }
         const float m_col = mltot[col * 2 + 0];
         const float l_col = mltot[col * 2 + 1];
-        if (P.max_chunks > 1) {
-            float* dst = P.part_acc + (row * P.max_chunks + chunk) * kHeadDim;
+        if (BAL ? item.n_chunks > 1 : P.max_chunks > 1) {
+            const size_t prow = BAL ? bal_partial_row(item.slot, (int)gridDim.y, kv_sub, col)
+                                    : row * P.max_chunks + chunk;
+            float* dst = P.part_acc + prow * kHeadDim;
             *reinterpret_cast<f4*>(dst + 4 * lane) = f4{v[0], v[1], v[2], v[3]};
             if (lane == 0) {
-                *reinterpret_cast<f4*>(P.part_ml + (row * P.max_chunks + chunk) * 4) =
-                    f4{m_col, l_col, (float)g.n_chunks, 0.f};
+                *reinterpret_cast<f4*>(P.part_ml + prow * 4) = f4{m_col, l_col, (float)g.n_chunks, 0.f};
             }
         } else {
             const float inv = l_col > 0.f ? 1.0f / l_col : 0.f;
@@ -649,6 +666,18 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_rows_kernel(con
             *reinterpret_cast<uint2*>(P.out + row * kHeadDim + 4 * lane) = o;
         }
     }
+}
+
+template <typename TQ, int NT, int KVF>
+__global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_rows_kernel(const AttnParams P) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    rows_tile<TQ, NT, KVF, false>(P, smem, BalItem{});
+}
+
+template <typename TQ, int KVF>
+__global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_rows_balanced_kernel(const AttnParams P) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    bal_for_each_piece(P, [&](const BalItem& it) { rows_tile<TQ, 1, KVF, true>(P, smem, it); });
 }
 
 }  // namespace w34
