@@ -185,6 +185,44 @@ int warp34_paged_attention_f16_force_kernel_for_test(
     const warp34_attention_batch* batch,
     const void* q_in, void* attn_out, int num_q_heads, int use_64q);
 
+/* ------------------------------------------------------------------------------------
+ * Producer side of the path: per-head RMSNorm + RoPE over packed bf16 rows
+ * [rows, (q_heads + 2 kv_heads) * dim] (replaces ops/op_dflash2.cu:338-418,1251-1410).
+ *
+ * For each Q and K head: y = bf16(x * rsqrt(mean(x^2) + eps) * w), then the pairs
+ * (c, c + dim/2) are rotated with cos = table[pos][c], sin = table[pos][dim/2 + c]
+ * (table: [table_rows, dim], bf16 for the first entry point, fp32 for the others).  Rows
+ * whose position is outside [0, table_rows) are skipped.  Q goes to q_out
+ * [rows, q_heads * dim] when q_out != NULL, otherwise it is rotated in place; V is never
+ * modified.  dim <= 256 and even, q_heads % kv_heads == 0, eps > 0 and finite, q_out != qkv.
+ *
+ * _kv_write_: rows with write_slot_mapping[row] >= 0 store the rotated K and the V row in
+ * the paged cache (same addressing as the append entry points) and leave the packed K as it
+ * was; rows with a negative slot are rotated in place.  The reference accepts BF16 pages
+ * only (op_dflash2.cu:1326-1333); this library also takes TQ4 + WHT256, FP8_E4M3 and Q8_0
+ * pages at dim 256 (K and V in the same format and transform), written with the encoders
+ * of the append entry points: a fused call equals operator + append bit for bit.
+ * ------------------------------------------------------------------------------------ */
+int warp34_dflash_qk_norm_rope_bf16(const warp34_exec* ex, void* qkv, const int32_t* positions,
+                                    const void* qw, const void* kw, const void* table,
+                                    int rows, int q_heads, int kv_heads, int dim,
+                                    int table_rows, float eps);               /* warp34_cuda.h:635-637 */
+int warp34_dflash_qk_norm_rope_bf16_f32_table(const warp34_exec* ex, void* qkv,
+                                              const int32_t* positions, const void* qw,
+                                              const void* kw, const void* table,
+                                              int rows, int q_heads, int kv_heads, int dim,
+                                              int table_rows, float eps);     /* warp34_cuda.h:619-621 */
+int warp34_dflash_qk_norm_rope_bf16_f32_table_qout(const warp34_exec* ex, void* qkv, void* q_out,
+                                                   const int32_t* positions, const void* qw,
+                                                   const void* kw, const void* table,
+                                                   int rows, int q_heads, int kv_heads, int dim,
+                                                   int table_rows, float eps); /* warp34_cuda.h:622-624 */
+int warp34_dflash_qk_norm_rope_kv_write_bf16_f32_table(
+    const warp34_exec* ex, void* qkv, void* q_out, const int32_t* positions,
+    const void* qw, const void* kw, const void* table,
+    const warp34_kv_layer_layout* kv_layout, const int32_t* write_slot_mapping,
+    int rows, int q_heads, int kv_heads, int dim, int table_rows, float eps);  /* warp34_cuda.h:625-628 */
+
 /* Bytes of scratch the attention entry points can make use of for a batch of this shape
  * (split-K partials).  No counterpart in the reference, whose engine simply guarantees
  * >= 8 MiB (op_paged_attn.cu:1301-1304); provided so a host can size ex->scratch. */

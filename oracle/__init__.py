@@ -87,6 +87,10 @@ def lib():
         L.tq4o_paged_attention_split.restype = C.c_int
         L.tq4o_paged_attention_split.argtypes = [C.POINTER(Layout), C.POINTER(Batch), C.c_void_p, C.c_int,
                                                  C.c_void_p, C.c_int, C.c_int]
+        L.tq4o_qk_norm_rope_bf16.restype = C.c_int
+        L.tq4o_qk_norm_rope_bf16.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                             C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float,
+                                             C.POINTER(Layout), C.c_void_p]
         L.tq4o_fill_normal.argtypes = [C.c_void_p, C.c_size_t, C.c_uint64, C.c_int]
         L.tq4o_fill_kv_rows.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_uint64, C.c_int, C.c_int]
         L.tq4o_permutation.argtypes = [C.c_void_p, C.c_int, C.c_uint64]
@@ -304,6 +308,30 @@ def paged_attention(pool, batch, q_bits, q_dtype, num_q_heads, n_threads=1, out=
     if rc:
         raise RuntimeError("oracle paged_attention: unsupported shape")
     return out
+
+
+def qk_norm_rope_bf16(qkv, positions, qw, kw, table, q_heads, kv_heads, dim, eps, q_out=None, pool=None,
+                      write_slot_mapping=None):
+    """ops/op_dflash2.cu:338-418.  qkv: uint16 [rows, (q_heads + 2 kv_heads) * dim], modified in
+    place; table: float32 or uint16 (bf16 bits) [table_rows, dim]; with pool + write_slot_mapping the
+    rotated K and the V rows go to the pool instead.  Returns (qkv, q_out)."""
+    assert qkv.dtype == np.uint16 and qkv.flags.c_contiguous
+    rows = qkv.shape[0]
+    positions = np.ascontiguousarray(positions, dtype=np.int32)
+    qw = np.ascontiguousarray(qw, dtype=np.uint16)
+    kw = np.ascontiguousarray(kw, dtype=np.uint16)
+    table = np.ascontiguousarray(table)
+    assert table.dtype in (np.float32, np.uint16)
+    slots = None if write_slot_mapping is None else np.ascontiguousarray(write_slot_mapping, dtype=np.int32)
+    L = pool.layout() if pool is not None else None
+    rc = lib().tq4o_qk_norm_rope_bf16(qkv.ctypes.data, None if q_out is None else q_out.ctypes.data,
+                                      positions.ctypes.data, qw.ctypes.data, kw.ctypes.data, table.ctypes.data,
+                                      1 if table.dtype == np.float32 else 0, rows, q_heads, kv_heads, dim,
+                                      table.shape[0], eps, None if L is None else C.byref(L),
+                                      None if slots is None else slots.ctypes.data)
+    if rc:
+        raise RuntimeError("oracle qk_norm_rope_bf16: rc=%d" % rc)
+    return qkv, q_out
 
 
 def slot_mapping(block_table, ctx_before, n_tokens, block_size):

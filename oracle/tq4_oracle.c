@@ -324,6 +324,91 @@ static int write_row(uint8_t* dst, int format, int transform, const uint16_t* sr
     return -1;
 }
 
+/* ---- QK RMSNorm + RoPE over packed bf16 rows, optionally with the K/V rows written into the
+ * paged cache: qk_norm_rope_bf16_warp, ops/op_dflash2.cu:338-418 ----
+ * Declared numerics: fp32 in source order without contraction; the sum of squares in the order
+ * of reduce_sum256_exact_warp (op_dflash2.cu:30-39: per lane ((v0+v128)+(v64+v192)) +
+ * ((v32+v160)+(v96+v224)), then the 32-lane xor butterfly 16,8,4,2,1); rsqrt(x) :=
+ * fl32(1/sqrt(x) in fp64); bf16 round-to-nearest-even. */
+static float sum256_warp_order(const float* sq) { /* sq[c], c = lane + 32 k */
+    float lane_sum[32];
+    for (int lane = 0; lane < 32; ++lane) {
+        const float v0 = sq[lane], v32 = sq[lane + 32], v64 = sq[lane + 64], v96 = sq[lane + 96];
+        const float v128 = sq[lane + 128], v160 = sq[lane + 160], v192 = sq[lane + 192], v224 = sq[lane + 224];
+        lane_sum[lane] = ((v0 + v128) + (v64 + v192)) + ((v32 + v160) + (v96 + v224));
+    }
+    for (int mask = 16; mask >= 1; mask >>= 1) {
+        float next[32];
+        for (int lane = 0; lane < 32; ++lane) next[lane] = lane_sum[lane] + lane_sum[lane ^ mask];
+        memcpy(lane_sum, next, sizeof(next));
+    }
+    return lane_sum[0];
+}
+
+int tq4o_qk_norm_rope_bf16(uint16_t* qkv, uint16_t* q_out, const int32_t* positions, const uint16_t* qw,
+                           const uint16_t* kw, const void* table, int table_is_f32, int rows, int q_heads,
+                           int kv_heads, int dim, int table_rows, float eps, const tq4o_layout* L,
+                           const int32_t* write_slot_mapping) {
+    if (!qkv || !positions || !qw || !kw || !table || rows < 0 || q_heads < 0 || kv_heads <= 0 || dim <= 0 ||
+        dim > 256 || (dim & 1) || table_rows <= 0 || !(eps > 0.0f)) {
+        return -1;
+    }
+    const int half = dim / 2;
+    const size_t row_elems = (size_t)(q_heads + 2 * kv_heads) * dim;
+    for (int row = 0; row < rows; ++row) {
+        const int pos = positions[row];
+        if (pos < 0 || pos >= table_rows) continue; /* :356 */
+        for (int head = 0; head < q_heads + kv_heads; ++head) {
+            uint16_t* src = qkv + (size_t)row * row_elems + (size_t)head * dim;
+            const uint16_t* w = head < q_heads ? qw : kw;
+            float sq[256];
+            for (int c = 0; c < 256; ++c) {
+                const float x = c < dim ? tq4o_bf16_to_f32(src[c]) : 0.0f;
+                sq[c] = x * x;
+            }
+            const float sum_sq = sum256_warp_order(sq);
+            const float mean = sum_sq / (float)dim + eps;
+            const float inv = (float)(1.0 / sqrt((double)mean));
+            uint16_t out[256];
+            for (int c = 0; c < half; ++c) {
+                const float a = tq4o_bf16_to_f32(tq4o_f32_to_bf16(tq4o_bf16_to_f32(src[c]) * inv * tq4o_bf16_to_f32(w[c])));
+                const float b = tq4o_bf16_to_f32(
+                    tq4o_f32_to_bf16(tq4o_bf16_to_f32(src[half + c]) * inv * tq4o_bf16_to_f32(w[half + c])));
+                float cosine, sine;
+                if (table_is_f32) {
+                    const float* t = (const float*)table + (size_t)pos * dim;
+                    cosine = t[c];
+                    sine = t[half + c];
+                } else {
+                    const uint16_t* t = (const uint16_t*)table + (size_t)pos * dim;
+                    cosine = tq4o_bf16_to_f32(t[c]);
+                    sine = tq4o_bf16_to_f32(t[half + c]);
+                }
+                const float ac = a * cosine, bs = b * sine, bc = b * cosine, as = a * sine;
+                out[c] = tq4o_f32_to_bf16(ac - bs);
+                out[half + c] = tq4o_f32_to_bf16(bc + as);
+            }
+            uint16_t* dst = (q_out != NULL && head < q_heads) ? q_out + ((size_t)row * q_heads + head) * dim : src;
+            if (write_slot_mapping != NULL && L != NULL && head >= q_heads && write_slot_mapping[row] >= 0) {
+                /* rotated K and the untouched V go to the cache, the packed row keeps its K (:387-403) */
+                const int slot = write_slot_mapping[row];
+                const int kv_head = head - q_heads;
+                const int page = slot / L->block_size, off = slot % L->block_size;
+                uint8_t* k_dst = L->k_base + (size_t)page * L->k_page_stride + (size_t)kv_head * L->k_head_stride +
+                                 (size_t)off * L->k_token_stride;
+                uint8_t* v_dst = L->v_base + (size_t)page * L->v_page_stride + (size_t)kv_head * L->v_head_stride +
+                                 (size_t)off * L->v_token_stride;
+                const uint16_t* v_src = src + (size_t)kv_heads * dim;
+                if (write_row(k_dst, L->k_format, L->k_transform, out, dim, TQ4O_DT_BF16) != 0) return -2;
+                if (write_row(v_dst, L->v_format, L->v_transform, v_src, dim, TQ4O_DT_BF16) != 0) return -2;
+            } else {
+                memcpy(dst, out, (size_t)dim * sizeof(uint16_t));
+            }
+        }
+    }
+    return 0;
+}
+
 /* ---- paged append: op_kv_cache.cu:325-368 ---- */
 int tq4o_kv_cache_write(const tq4o_layout* L, const tq4o_batch* B, const uint16_t* k_in,
                         const uint16_t* v_in, int k_row_stride, int v_row_stride, int in_dtype) {

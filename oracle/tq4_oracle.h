@@ -35,6 +35,11 @@
  *                     round trip error bounds, layout pins (264 B: codes then two fp32 scales;
  *                     272 B: four {fp32 scale, 64 int8}) -- exact BYTES for general inputs are
  *                     pinned by no reference-held vector: "parity unpinned" beyond that
+ *   tq4o_qk_norm_rope independent fp64 restatement (RMS norm, weight, rotation of the (c, c + dim/2)
+ *                     pairs) within one bf16 ulp; identity rotation at cos = 1, sin = 0; pair norms
+ *                     preserved; V bit-identical; cache rows = append of the rotated K.  The
+ *                     reference's golden tensors for this operator are not in its tree (LFS
+ *                     pointers only), so exact bf16 bits are "parity unpinned"
  */
 #ifndef TQ4_ORACLE_H
 #define TQ4_ORACLE_H
@@ -123,6 +128,16 @@ int tq4o_kv_cache_write(const tq4o_layout* L, const tq4o_batch* B,
  * time.  q is 16-bit of dtype q_dtype; out is fp32 [total_tokens, num_q_heads, head_dim];
  * rows that the reference leaves untouched are left untouched here too.
  * n_threads > 1 spreads rows over pthreads (results do not depend on it). --- */
+/* ops/op_dflash2.cu:338-418,1251-1410: RMSNorm over each Q and K head of packed bf16 rows
+ * [rows, (q_heads + 2 kv_heads) * dim], RoPE with a [table_rows, dim] cos|sin table (fp32 or bf16),
+ * Q to q_out (or in place), K in place -- or, with a layout and a slot mapping, K (rotated) and V
+ * (as it is) into the paged cache in the layout's formats.  Rows whose position is outside the
+ * table are skipped. */
+int tq4o_qk_norm_rope_bf16(uint16_t* qkv, uint16_t* q_out, const int32_t* positions, const uint16_t* qw,
+                           const uint16_t* kw, const void* table, int table_is_f32, int rows, int q_heads,
+                           int kv_heads, int dim, int table_rows, float eps, const tq4o_layout* L,
+                           const int32_t* write_slot_mapping);
+
 int tq4o_paged_attention(const tq4o_layout* L, const tq4o_batch* B,
                          const uint16_t* q, int q_dtype, float* out, int num_q_heads,
                          int n_threads);

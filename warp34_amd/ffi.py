@@ -104,6 +104,19 @@ SIGNATURES = {
     "warp34_paged_attention_f16_force_kernel_for_test":
         (C.c_int, [_EX, _LAY, _BAT, C.c_void_p, C.c_void_p, C.c_int, C.c_int]),
     "warp34_paged_attention_scratch_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int]),
+    # QK RMSNorm + RoPE on packed bf16 rows, optionally fused with the paged KV write
+    "warp34_dflash_qk_norm_rope_bf16":
+        (C.c_int, [_EX, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                   C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float]),
+    "warp34_dflash_qk_norm_rope_bf16_f32_table":
+        (C.c_int, [_EX, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                   C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float]),
+    "warp34_dflash_qk_norm_rope_bf16_f32_table_qout":
+        (C.c_int, [_EX, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                   C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float]),
+    "warp34_dflash_qk_norm_rope_kv_write_bf16_f32_table":
+        (C.c_int, [_EX, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, _LAY, C.c_void_p,
+                   C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float]),
     "warp34_cuda_error_string": (C.c_char_p, [C.c_int]),
     "warp34_get_device_count": (C.c_int, [C.POINTER(C.c_int)]),
     "warp34_set_device": (C.c_int, [C.c_int]),
