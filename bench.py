@@ -39,6 +39,8 @@ WORKLOADS = {
     # 8 sequences, 16 384-token TQ4 prefix + 2 048-token bf16 chunk each: append + causal attention
     "tq4_prefill_8x2048_ctx16384": ("tq4", [18432] * 8, 0),
     "fp8_prefill_8x2048_ctx16384": ("fp8", [18432] * 8, 0),
+    # producer side: QK RMSNorm + RoPE fused with the TQ4 append of an 8 192-token chunk
+    "tq4_norm_rope_append_8192": ("tq4", [8192], 0),
     # 16 sequences of 262 144 tokens that share the pages of a 200 000-token prefix; 4 query tokens each
     "tq4_verify_16x4_ctx262144_shared200k": ("tq4", [262144] * 16, 0),
 }
@@ -266,6 +268,91 @@ def run_prefill(args, torch, lib, ffi, layers, ctx, n_layers, pool_pages, fmt):
     }))
 
 
+def run_producer(args, torch, lib, ffi, layers, n, n_layers, fmt):
+    """QK RMSNorm + RoPE over packed bf16 [n, (16 + 2 * 2) * 256] rows with the K / V rows written
+    into TQ4 pages: the fused entry point against the two-call sequence (operator in place, then
+    the strided append).  One step = one layer's producer work for an n-token chunk."""
+    dev = "cuda:0"
+    g = torch.Generator(device=dev)
+    g.manual_seed(11)
+    row = (Q_HEADS + 2 * KV_HEADS) * HEAD_DIM
+    qkv0 = torch.randn((n, row), generator=g, device=dev).to(torch.bfloat16)
+    qkv = qkv0.clone()
+    q_out = torch.empty((n, Q_HEADS * HEAD_DIM), dtype=torch.bfloat16, device=dev)
+    qw = (1.0 + 0.1 * torch.randn(HEAD_DIM, generator=g, device=dev)).to(torch.bfloat16)
+    kw = (1.0 + 0.1 * torch.randn(HEAD_DIM, generator=g, device=dev)).to(torch.bfloat16)
+    half = HEAD_DIM // 2
+    inv_freq = 1.0 / (10000.0 ** (torch.arange(half, device=dev) / half))
+    ang = torch.arange(n, device=dev)[:, None] * inv_freq[None, :]
+    table = torch.cat([torch.cos(ang), torch.sin(ang)], dim=1).float().contiguous()
+    pos = torch.arange(n, dtype=torch.int32, device=dev)
+    ex = ffi.Warp34Exec(torch.cuda.current_stream().cuda_stream, 0, 0, 0)
+    per_layer = []
+    for L in layers:
+        slots = torch.cat(L.tail_slots) if len(L.tail_slots) > 1 else L.tail_slots[0]
+        posn = torch.arange(0, n, device=dev)
+        slots = (L.block_tables[0, (posn // BLOCK)].to(torch.int64) * BLOCK + posn % BLOCK).to(torch.int32)
+        qsl = torch.tensor([0, n], dtype=torch.int32, device=dev)
+        seq = torch.tensor([n], dtype=torch.int32, device=dev)
+        batch = ffi.Warp34AttentionBatch(qsl.data_ptr(), None, seq.data_ptr(), L.block_tables.data_ptr(),
+                                         slots.data_ptr(), None, None, 1, n, L.max_blocks, n, n, 0, 0, 0.0625, 0)
+        per_layer.append((L, slots, batch, qsl, seq))
+    vp = lambda t: C.c_void_p(t.data_ptr())
+
+    def fused(i):
+        L, slots, batch, _, _ = per_layer[i % n_layers]
+        rc = lib.warp34_dflash_qk_norm_rope_kv_write_bf16_f32_table(
+            C.byref(ex), vp(qkv), vp(q_out), vp(pos), vp(qw), vp(kw), vp(table), C.byref(L.layout), vp(slots),
+            n, Q_HEADS, KV_HEADS, HEAD_DIM, n, 1e-6)
+        if rc:
+            raise RuntimeError("fused producer rc=%d" % rc)
+
+    def two_calls(i):
+        L, slots, batch, _, _ = per_layer[i % n_layers]
+        rc = lib.warp34_dflash_qk_norm_rope_bf16_f32_table_qout(
+            C.byref(ex), vp(qkv), vp(q_out), vp(pos), vp(qw), vp(kw), vp(table), n, Q_HEADS, KV_HEADS, HEAD_DIM, n, 1e-6)
+        k_cols = C.c_void_p(qkv.data_ptr() + 2 * Q_HEADS * HEAD_DIM)
+        v_cols = C.c_void_p(qkv.data_ptr() + 2 * (Q_HEADS + KV_HEADS) * HEAD_DIM)
+        rc = rc or lib.warp34_kv_cache_write_strided_bf16(C.byref(ex), C.byref(L.layout), C.byref(batch), k_cols,
+                                                          v_cols, row)
+        if rc:
+            raise RuntimeError("operator + append rc=%d" % rc)
+
+    def timed(step):
+        for i in range(args.warmup):
+            step(i)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(args.steps):
+            step(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    ms_fused = timed(fused)
+    ms_two = timed(two_calls)
+    # algorithmic bytes: the packed row is read once, Q is written once, one K and one V row per kv head
+    bytes_step = n * (row * 2 + Q_HEADS * HEAD_DIM * 2 + 2 * KV_HEADS * ROW_BYTES[fmt]) + n * HEAD_DIM * 4
+    gbs = bytes_step / (ms_fused * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "QK RMSNorm + RoPE fused with the %s append: us/layer + achieved HBM GB/s" % fmt.upper(),
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_fused, 6), "us_per_layer": round(ms_fused * 1e3, 2),
+        "us_per_layer_operator_then_append": round(ms_two * 1e3, 2),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32 arithmetic on bf16 rows, %s rows written" % fmt.upper(), "data": "synthetic",
+        "config": {"workload": args.workload, "tokens": n, "q_heads": Q_HEADS, "kv_heads": KV_HEADS,
+                   "head_dim": HEAD_DIM, "page_tokens": BLOCK, "kv_format": "tq4+wht256" if fmt == "tq4" else fmt,
+                   "kv_pools_cycled": n_layers, "bytes_per_step": bytes_step},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "qk_norm_rope_kernel<true, true> (fused cache write)",
+                     "avg_launch_us": round(ms_fused * 1e3, 2)},
+    }))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -345,6 +432,9 @@ def run_workload(args, torch, lib, ffi, dev):
 
     if "_prefill_" in args.workload:
         run_prefill(args, torch, lib, ffi, layers, ctx, n_layers, pool_pages, fmt)
+        return None
+    if "_norm_rope_append_" in args.workload:
+        run_producer(args, torch, lib, ffi, layers, int(ctx[0]), n_layers, fmt)
         return None
 
     R = len(ctx)

@@ -32,7 +32,9 @@ struct NormRopeParams {
     float eps;
 };
 
-template <bool TABLE_F32>
+// D256: head size 256 known at compile time (no bounds tests, the second pass reuses the
+// values of the first instead of loading them again).
+template <bool TABLE_F32, bool D256>
 __global__ __launch_bounds__(256) void qk_norm_rope_kernel(const NormRopeParams P) {
     __shared__ __align__(8) uint8_t rows_lds[4][2][272];
     const int wave = (int)(threadIdx.x >> 6);
@@ -48,7 +50,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(const NormRopeParams 
     const int pos = P.positions[row];
     if (pos < 0 || pos >= P.table_rows) return;  // op_dflash2.cu:356
 
-    const int dim = P.dim, half = dim >> 1;
+    const int dim = D256 ? 256 : P.dim, half = dim >> 1;
     const size_t row_elems = (size_t)(P.q_heads + 2 * P.kv_heads) * dim;
     uint16_t* row_base = P.qkv + (size_t)row * row_elems;
 
@@ -74,7 +76,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(const NormRopeParams 
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
         const int c = l32 + 32 * k;
-        raw[k] = c < dim ? BF16::to_f32(src[c]) : 0.0f;
+        raw[k] = (D256 || c < dim) ? BF16::to_f32(src[c]) : 0.0f;
         sq[k] = raw[k] * raw[k];
     }
     float s = ((sq[0] + sq[4]) + (sq[2] + sq[6])) + ((sq[1] + sq[5]) + (sq[3] + sq[7]));
@@ -88,10 +90,11 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(const NormRopeParams 
     for (int k = 0; k < 4; ++k) {
         const int c = l32 + 32 * k;
         lo[k] = hi[k] = 0.0f;
-        if (c < half) {
-            const float a = BF16::to_f32(BF16::from_f32(BF16::to_f32(src[c]) * inv * BF16::to_f32(w[c])));
-            const float b =
-                BF16::to_f32(BF16::from_f32(BF16::to_f32(src[half + c]) * inv * BF16::to_f32(w[half + c])));
+        if (D256 || c < half) {
+            const float x_lo = D256 ? raw[k] : BF16::to_f32(src[c]);
+            const float x_hi = D256 ? raw[k + 4] : BF16::to_f32(src[half + c]);
+            const float a = BF16::to_f32(BF16::from_f32(x_lo * inv * BF16::to_f32(w[c])));
+            const float b = BF16::to_f32(BF16::from_f32(x_hi * inv * BF16::to_f32(w[half + c])));
             float cosine, sine;
             if constexpr (TABLE_F32) {
                 const float* t = reinterpret_cast<const float*>(P.table) + (size_t)pos * dim;
@@ -126,7 +129,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(const NormRopeParams 
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const int c = l32 + 32 * k;
-                    if (c < half) {
+                    if (D256 || c < half) {
                         d16[c] = BF16::from_f32(lo[k]);
                         d16[half + c] = BF16::from_f32(hi[k]);
                     }
@@ -148,7 +151,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(const NormRopeParams 
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const int c = l32 + 32 * k;
-        if (c < half) {
+        if (D256 || c < half) {
             dst[c] = BF16::from_f32(lo[k]);
             dst[half + c] = BF16::from_f32(hi[k]);
         }
@@ -185,7 +188,11 @@ static int launch_norm_rope(const warp34_exec* ex, void* qkv, void* q_out, const
     P.eps = eps;
     const long long items = (long long)rows * ((q_heads + 1) / 2 + kv_heads);
     const unsigned grid = (unsigned)((items + 3) / 4);
-    hipLaunchKernelGGL((qk_norm_rope_kernel<TABLE_F32>), dim3(grid), dim3(256), 0, (hipStream_t)ex->stream, P);
+    if (dim == 256) {
+        hipLaunchKernelGGL((qk_norm_rope_kernel<TABLE_F32, true>), dim3(grid), dim3(256), 0, (hipStream_t)ex->stream, P);
+    } else {
+        hipLaunchKernelGGL((qk_norm_rope_kernel<TABLE_F32, false>), dim3(grid), dim3(256), 0, (hipStream_t)ex->stream, P);
+    }
     return (int)hipGetLastError();
 }
 
