@@ -59,11 +59,10 @@ struct BF16 {
     __device__ static __forceinline__ float to_f32(uint16_t b) {
         return __uint_as_float((uint32_t)b << 16);
     }
-    __device__ static __forceinline__ uint16_t from_f32(float f) {  // round to nearest even
-        uint32_t x = __float_as_uint(f);
-        if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((x >> 16) | 0x40u);
-        x += 0x7FFFu + ((x >> 16) & 1u);
-        return (uint16_t)(x >> 16);
+    // round to nearest even: gfx950 converts in hardware (v_cvt_pk_bf16_f32); a NaN comes out
+    // as a quiet NaN whose payload is the hardware's choice
+    __device__ static __forceinline__ uint16_t from_f32(float f) {
+        return __builtin_bit_cast(uint16_t, (__bf16)f);
     }
 };
 

@@ -41,11 +41,20 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(const NormRopeParams 
     const int lane = lane_id();
     const int half_id = lane >> 5;
     const int l32 = lane & 31;
+    // Items are ordered KV items of all rows first, then the Q items: the long items (norm +
+    // two row encodes) start first and every workgroup holds items of one kind.
     const int q_items = (P.q_heads + 1) >> 1;
-    const int items_per_row = q_items + P.kv_heads;
     const long long item = (long long)blockIdx.x * 4 + wave;
-    const int row = (int)(item / items_per_row);
-    const int it = (int)(item - (long long)row * items_per_row);
+    const long long n_kv_items = (long long)P.rows * P.kv_heads;
+    int row, it;
+    if (item < n_kv_items) {
+        row = (int)(item / P.kv_heads);
+        it = q_items + (int)(item - (long long)row * P.kv_heads);
+    } else {
+        const long long qi = item - n_kv_items;
+        row = q_items > 0 ? (int)(qi / q_items) : P.rows;
+        it = q_items > 0 ? (int)(qi - (long long)row * q_items) : 0;
+    }
     if (row >= P.rows) return;
     const int pos = P.positions[row];
     if (pos < 0 || pos >= P.table_rows) return;  // op_dflash2.cu:356
