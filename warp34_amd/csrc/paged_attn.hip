@@ -379,6 +379,11 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         seq_after = item.seq_after;
         ctx_before = item.ctx_before;
         req_hit = true;
+        // the piece's first unit is known: its block-table slice is requested together with the
+        // query rows
+        spec_slot_base = fast_div(item.u_begin * kUnit, L.block_size);
+        const int slot = spec_slot_base + lane;
+        if (slot < B.max_blocks_per_req) spec_vec = B.block_tables[(size_t)req * B.max_blocks_per_req + slot];
     } else if (P.tiles_by_request) {
         req = tile_z;  // < num_reqs by the launch geometry
         // Speculative block-table load, in flight together with the request's lengths: it
@@ -907,18 +912,37 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
     };
 
 
-    for (; unit < cu_end; unit += kWaves) {
+    // Units are dealt to the waves by a fixed rule, never handed out dynamically: which wave
+    // sums which keys decides the floating-point result, and the output has to be the same bits
+    // on every run and under every page permutation.  The rule is round robin with one extra
+    // unit for waves 0-3 after every eight rounds (68 units: nine each for waves 0-3, eight each
+    // for waves 4-7): the SIMD serves its older wave first, which makes waves 0-3 about 10 %
+    // faster per unit, and an even deal leaves them waiting at the merge.
+    auto nth_unit = [&](int j) -> int {  // j-th unit of this wave
+        if constexpr (kWaves == 8) {
+            if (wave < 4) {
+                const int g = j / 9, k = j - 9 * g;
+                return cu_first + 68 * g + (k < 8 ? 8 * k + wave : 64 + wave);
+            }
+            return cu_first + 68 * (j >> 3) + 8 * (j & 7) + wave;
+        } else {
+            return cu_first + j * kWaves + wave;
+        }
+    };
+    for (int j = 0; unit < cu_end; ++j) {
         commit_loads();
 #ifdef W34_TRACE
         if (trace_it < 8) W34_TP(4 + 4 * trace_it);
 #endif
-        if (unit + kWaves < cu_end) issue_loads(unit + kWaves);
+        const int next_unit = nth_unit(j + 1);
+        if (next_unit < cu_end) issue_loads(next_unit);
         const int t0 = unit * kUnit;
         process_unit(t0, !(t0 >= i_lo && t0 + kUnit - 1 <= i_hi));
 #ifdef W34_TRACE
         if (trace_it < 8) W34_TP(4 + 4 * trace_it + 3);
         ++trace_it;
 #endif
+        unit = next_unit;
     }
     W34_TP(36);
 
