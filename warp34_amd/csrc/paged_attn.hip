@@ -1088,8 +1088,12 @@ __device__ __forceinline__ void bal_for_each_piece(const AttnParams& P, TileFn&&
 #endif
     W34_TP(60);
     const int num_reqs = P.B.num_reqs;
-    int total = 0;
-    for (int base = 0; base < num_reqs; base += 64)
+    // the first 64 requests are loaded once: their lane values serve the total and the search for
+    // the first piece (most workgroups have exactly one piece, most batches at most 64 requests)
+    const BalReq q0 = bal_load_req(P, lane);
+    const int incl0 = wave_incl_scan(q0.cost, lane);
+    int total = __builtin_amdgcn_readlane(incl0, 63);
+    for (int base = 64; base < num_reqs; base += 64)
         total += __builtin_amdgcn_readlane(wave_incl_scan(bal_load_req(P, base + lane).cost, lane), 63);
     const int share = bal_share(total, (int)gridDim.x, P.min_upc + kBalPieceCost);
     const int my_begin = (int)blockIdx.x * share;
@@ -1100,45 +1104,50 @@ __device__ __forceinline__ void bal_for_each_piece(const AttnParams& P, TileFn&&
     // The pieces of this share, in order.  Nothing but a few scalars stays live across a tile:
     // the 64-request group that holds the next piece is loaded and scanned again after each one.
     int base = 0, before = 0, taken = 0;  // group, units before it, pieces of it already done
+    BalItem it{};
+    int piece_end = 0;
     W34_TP(59);
-    while (base < num_reqs && before < my_end) {
-        BalItem it;
-        bool have = false;
-        int group_units = 0, piece_end = 0;
-        {
-            const BalReq q = bal_load_req(P, base + lane);
-            const int incl = wave_incl_scan(q.cost, lane);
-            const int start = before + incl - q.units;  // of the real units, behind the charge
-            unsigned long long hits = __ballot(q.units > 0 && start < my_end && start + q.units > my_begin);
-            for (int skip = 0; skip < taken && hits != 0ull; ++skip) hits &= hits - 1ull;
-            group_units = __builtin_amdgcn_readlane(incl, 63);
-            if (hits != 0ull) {
-                const int src = __builtin_ctzll(hits);
-                const int r_start = __builtin_amdgcn_readlane(start, src);
-                const int r_units = __builtin_amdgcn_readlane(q.units, src);
-                it.req = base + src;
-                it.rq_start = __builtin_amdgcn_readlane(q.lo, src);
-                it.rq_end = __builtin_amdgcn_readlane(q.hi, src);
-                it.seq_after = __builtin_amdgcn_readlane(q.sa, src);
-                it.ctx_before = __builtin_amdgcn_readlane(q.cb, src);
-                it.u_begin = max(my_begin, r_start) - r_start;
-                it.u_end = min(my_end, r_start + r_units) - r_start;
-                it.n_chunks = (r_start + r_units - 1) / share - r_start / share + 1;
-                it.slot = (int)blockIdx.x + it.req;
-                piece_end = r_start + it.u_end;
-                have = true;
-            }
-        }
-        if (!have) {
-            before += group_units;
+    // next piece inside the group whose lane values are (q, incl); false: the group has none left
+    auto scan_group = [&](const BalReq& q, int incl) -> bool {
+        const int start = before + incl - q.units;  // of the real units, behind the charge
+        unsigned long long hits = __ballot(q.units > 0 && start < my_end && start + q.units > my_begin);
+        for (int skip = 0; skip < taken && hits != 0ull; ++skip) hits &= hits - 1ull;
+        if (hits == 0ull) {
+            before += __builtin_amdgcn_readlane(incl, 63);
             base += 64;
             taken = 0;
-            continue;
+            return false;
         }
+        const int src = __builtin_ctzll(hits);
+        const int r_start = __builtin_amdgcn_readlane(start, src);
+        const int r_units = __builtin_amdgcn_readlane(q.units, src);
+        it.req = base + src;
+        it.rq_start = __builtin_amdgcn_readlane(q.lo, src);
+        it.rq_end = __builtin_amdgcn_readlane(q.hi, src);
+        it.seq_after = __builtin_amdgcn_readlane(q.sa, src);
+        it.ctx_before = __builtin_amdgcn_readlane(q.cb, src);
+        it.u_begin = max(my_begin, r_start) - r_start;
+        it.u_end = min(my_end, r_start + r_units) - r_start;
+        it.n_chunks = (r_start + r_units - 1) / share - r_start / share + 1;
+        it.slot = (int)blockIdx.x + it.req;
+        piece_end = r_start + it.u_end;
         ++taken;
+        return true;
+    };
+    auto find_next = [&]() -> bool {
+        while (base < num_reqs && before < my_end) {
+            const BalReq q = bal_load_req(P, base + lane);
+            if (scan_group(q, wave_incl_scan(q.cost, lane))) return true;
+        }
+        return false;
+    };
+    bool have = scan_group(q0, incl0);
+    if (!have) have = find_next();
+    while (have) {
         tile(it);
         if (piece_end >= my_end) break;  // the share ends with this piece
         __syncthreads();  // the tile's merge regions alias what the next piece sets up
+        have = find_next();
     }
     W34_TP(61);
 }
