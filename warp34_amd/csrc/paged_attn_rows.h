@@ -172,7 +172,12 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
     // request's length is the host's bound max_seq_len.  A wrong guess is fetched again below,
     // so it changes the latency only, never the result.
     int spec_slot_base = -1, spec_vec = -1;
-    if (!BAL && P.tiles_by_request && B.sliding_window <= 0 && B.max_seq_len > 0) {
+    if constexpr (BAL) {
+        // the piece's first unit is known: its block-table slice is requested with the query rows
+        spec_slot_base = fast_div(item.u_begin * kUnit, L.block_size);
+        const int slot = spec_slot_base + lane;
+        if (slot < B.max_blocks_per_req) spec_vec = B.block_tables[(size_t)tile_z * B.max_blocks_per_req + slot];
+    } else if (P.tiles_by_request && B.sliding_window <= 0 && B.max_seq_len > 0) {
         const ChunkGeom sg = chunk_geom(0, B.max_seq_len - 1, P.max_chunks, P.min_upc);
         spec_slot_base = fast_div((sg.u_first + chunk * sg.upc) * kUnit, L.block_size);
         const int slot = spec_slot_base + lane;
@@ -552,7 +557,18 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
     } else {
         load_page_vec();
     }
-    int hidx = 2 * unit;
+    // Units are dealt by a fixed rule (the result must not depend on timing): round robin with
+    // one extra unit for waves 0-3 after every eight rounds, because each SIMD serves its older
+    // wave first (see the TQ4 kernel).
+    auto nth_unit = [&](int j) -> int {
+        if (wave < 4) {
+            const int g = j / 9, k = j - 9 * g;
+            return cu_first + 68 * g + (k < 8 ? 8 * k + wave : 64 + wave);
+        }
+        return cu_first + 68 * (j >> 3) + 8 * (j & 7) + wave;
+    };
+    static_assert(kWaves == 8, "unit deal assumes two waves per SIMD");
+    int hidx = 2 * unit, unit_no = 0;
     issue_half(hidx);
     while (unit < cu_end) {
         commit_half(hidx);
@@ -560,7 +576,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
         if (next_h & 1) {
             // second half of the same unit
         } else {
-            next_unit = unit + kWaves;
+            next_unit = nth_unit(++unit_no);
             next_h = 2 * next_unit;
         }
         if (next_unit < cu_end) issue_half(next_h);
