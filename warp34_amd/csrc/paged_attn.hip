@@ -109,6 +109,7 @@ struct AttnParams {
     int tiles_by_request;  // 1: blockIdx.z is a request (no request has more than one tile)
     int rot_q;             // row-format kernel: K rows are stored rotated, rotate the query rows
     int rot_out;           // row-format kernel: V rows are stored rotated, rotate the output back
+    int32_t* bal_table;    // balanced decode: per query token {first partial slot, pieces, token of the tile, -}
 };
 
 // token of k-slot (s, b, i) inside a unit: spreads the four 4-row groups of an MFMA over LDS
@@ -252,8 +253,11 @@ constexpr int kMergeMaxPerGroup = 16;  // at most 256 partials per row
 // units of all requests are laid end to end and workgroup x owns units [x S, (x + 1) S).  A share
 // that crosses a request boundary is worked off piece by piece.  Piece (x, r) gets partial slot
 // x + r: both grow along the pieces, so the slots are unique and those of one request are
-// consecutive, first_wg(r) + r .. last_wg(r) + r.  The plan is a function of the batch
-// descriptor alone; the merge kernel recomputes it instead of reading it from memory.
+// consecutive, first_wg(r) + r .. last_wg(r) + r.  The workgroup that owns a request's first
+// piece records {first slot, number of pieces, token of the tile} for each of the request's
+// query tokens in a per-token table for the merge kernel; the tokens of requests without work
+// are recorded by workgroup (0, 0): pieces = 0 for a live request without visible keys (output
+// zeros), -1 for a masked one and for tokens behind the last request (output untouched).
 // Starting a piece (table, query rotation, first loads, merge of the waves) costs about as much
 // as kBalPieceCost units of streaming, so every request is charged that many extra units in
 // front of its real ones: a share that contains request boundaries gets fewer keys.
@@ -265,10 +269,11 @@ __host__ __device__ __forceinline__ size_t bal_partial_row(int slot, int kv_subs
 struct BalReq {  // request base + lane of a 64-request group
     int lo, hi, sa, cb, units;
     int cost;  // units + kBalPieceCost, 0 for a request without work
+    int live;  // has query tokens and is not masked
 };
 __device__ __forceinline__ BalReq bal_load_req(const AttnParams& P, int r) {
     const warp34_attention_batch& B = P.B;
-    BalReq q{0, 0, 0, 0, 0, 0};
+    BalReq q{0, 0, 0, 0, 0, 0, 0};
     if (r >= B.num_reqs) return q;
     q.lo = B.query_start_loc[r];
     q.hi = B.query_start_loc[r + 1];
@@ -280,6 +285,7 @@ __device__ __forceinline__ BalReq bal_load_req(const AttnParams& P, int r) {
     if (last >= q.sa) last = q.sa - 1;
     q.units = (live && last >= 0) ? (last >> 5) + 1 : 0;
     q.cost = q.units > 0 ? q.units + kBalPieceCost : 0;
+    q.live = live ? 1 : 0;
     return q;
 }
 __device__ __forceinline__ int wave_incl_scan(int v, int lane) {
@@ -1093,8 +1099,25 @@ __device__ __forceinline__ void bal_for_each_piece(const AttnParams& P, TileFn&&
     const BalReq q0 = bal_load_req(P, lane);
     const int incl0 = wave_incl_scan(q0.cost, lane);
     int total = __builtin_amdgcn_readlane(incl0, 63);
-    for (int base = 64; base < num_reqs; base += 64)
-        total += __builtin_amdgcn_readlane(wave_incl_scan(bal_load_req(P, base + lane).cost, lane), 63);
+    // wave 0 of workgroup (0, 0) records the requests no workgroup will work on
+    const bool recorder = blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x < 64;
+    auto record_idle = [&](const BalReq& q, int r) {
+        if (!recorder || r >= num_reqs) return;
+        if (q.units == 0) {
+            for (int t = q.lo; t < q.hi && t < P.B.total_tokens; ++t)
+                *reinterpret_cast<int4*>(P.bal_table + 4 * (size_t)t) = int4{0, q.live ? 0 : -1, t - q.lo, 0};
+        }
+        if (r == num_reqs - 1) {
+            for (int t = max(q.hi, 0); t < P.B.total_tokens; ++t)
+                *reinterpret_cast<int4*>(P.bal_table + 4 * (size_t)t) = int4{0, -1, 0, 0};
+        }
+    };
+    record_idle(q0, lane);
+    for (int base = 64; base < num_reqs; base += 64) {
+        const BalReq q = bal_load_req(P, base + lane);
+        record_idle(q, base + lane);
+        total += __builtin_amdgcn_readlane(wave_incl_scan(q.cost, lane), 63);
+    }
     const int share = bal_share(total, (int)gridDim.x, P.min_upc + kBalPieceCost);
     const int my_begin = (int)blockIdx.x * share;
     int my_end = my_begin + share;
@@ -1131,6 +1154,11 @@ __device__ __forceinline__ void bal_for_each_piece(const AttnParams& P, TileFn&&
         it.n_chunks = (r_start + r_units - 1) / share - r_start / share + 1;
         it.slot = (int)blockIdx.x + it.req;
         piece_end = r_start + it.u_end;
+        if (it.u_begin == 0 && blockIdx.y == 0 && (int)threadIdx.x < it.rq_end - it.rq_start &&
+            it.rq_start + (int)threadIdx.x < P.B.total_tokens) {  // first piece: one entry per query token
+            *reinterpret_cast<int4*>(P.bal_table + 4 * (size_t)(it.rq_start + (int)threadIdx.x)) =
+                int4{it.slot, it.n_chunks, (int)threadIdx.x, 0};
+        }
         ++taken;
         return true;
     };
@@ -1160,58 +1188,31 @@ __global__ __launch_bounds__(waves_for(1) * 64, 1) void paged_attn_tq4_balanced_
 }
 
 // Merge for the balanced decode kernel: one workgroup of 1024 threads per (token, q head) row.
-// Wave 0 recomputes the plan for the row's request; rows whose request was not cut (one piece)
-// were finished by the attention kernel, rows of requests without visible keys are zero.
+// The token's table entry says where its partials are; rows whose request was not cut (one
+// piece) were finished by the attention kernel, rows of live requests without visible keys are
+// zero, rows of masked requests stay untouched.
 template <typename TQ>
-__global__ __launch_bounds__(1024) void balanced_merge_kernel(const AttnParams P, int groups, int kv_subs,
-                                                              float out_scale, int rotate) {
+__global__ __launch_bounds__(1024) void balanced_merge_kernel(const AttnParams P, int kv_subs, float out_scale,
+                                                              int rotate) {
     __shared__ f4 s_acc[kMergeGroups][64];
     __shared__ f4 s_rec[256];
     __shared__ float s_red[kMergeGroups];
-    __shared__ int s_plan[4];  // valid, first slot, pieces, column
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
     const int grp = tid >> 6;
     const long long row = (long long)blockIdx.x;
     const int tok = (int)(row / P.num_q_heads);
     const int head = (int)(row - (long long)tok * P.num_q_heads);
-    const warp34_attention_batch& B = P.B;
-    if (grp == 0) {
-        int total = 0, r_found = -1, r_start = 0, r_units = 0, r_lo = 0;
-        for (int base = 0; base < B.num_reqs; base += 64) {
-            const BalReq q = bal_load_req(P, base + lane);
-            const int incl = wave_incl_scan(q.cost, lane);
-            const unsigned long long hits = __ballot(base + lane < B.num_reqs && tok >= q.lo && tok < q.hi);
-            if (hits != 0ull && r_found < 0) {
-                const int src = __builtin_ctzll(hits);
-                r_found = base + src;
-                r_start = total + __builtin_amdgcn_readlane(incl - q.units, src);
-                r_units = __builtin_amdgcn_readlane(q.units, src);
-                r_lo = __builtin_amdgcn_readlane(q.lo, src);
-            }
-            total += __builtin_amdgcn_readlane(incl, 63);
-        }
-        const bool req_ok = r_found >= 0 && (B.valid_req_mask == nullptr || B.valid_req_mask[max(r_found, 0)] != 0);
-        const int share = bal_share(total, groups, P.min_upc + kBalPieceCost);
-        const int first_wg = r_start / share;
-        const int pieces = r_units > 0 ? (r_start + r_units - 1) / share - first_wg + 1 : 0;
-        if (lane == 0) {
-            s_plan[0] = req_ok ? 1 : 0;
-            s_plan[1] = first_wg + r_found;
-            s_plan[2] = pieces;
-            s_plan[3] = (tok - r_lo) * P.q_group + head % P.q_group;
-        }
-    }
-    __syncthreads();
-    if (!s_plan[0]) return;  // masked request: output untouched
-    const int n_chunks = s_plan[2];
-    if (n_chunks == 1) return;  // finished by the attention kernel
-    if (n_chunks == 0) {        // no visible key: zeros
+    const int4 entry = *reinterpret_cast<const int4*>(P.bal_table + 4 * (size_t)tok);  // same address in every lane
+    const int n_chunks = entry.y;
+    if (n_chunks < 0 || n_chunks == 1) return;  // masked, or finished by the attention kernel
+    if (n_chunks == 0) {                        // no visible key: zeros
         if (grp == 0) *reinterpret_cast<uint2*>(P.out + (size_t)row * kHeadDim + 4 * lane) = uint2{0u, 0u};
         return;
     }
+    const int col = entry.z * P.q_group + head % P.q_group;
     const int kv_sub = head / P.q_group;  // = kv_head * q_subgroups + subgroup
-    const size_t prow0 = bal_partial_row(s_plan[1], kv_subs, kv_sub, s_plan[3]);
+    const size_t prow0 = bal_partial_row(entry.x, kv_subs, kv_sub, col);
     const size_t pstride = (size_t)kv_subs * 16;  // partial rows between consecutive slots
     if (tid < n_chunks && tid < 256) s_rec[tid] = *reinterpret_cast<const f4*>(P.part_ml + (prow0 + tid * pstride) * 4);
     f4 a[kMergeMaxPerGroup];
@@ -1569,9 +1570,10 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     if (balanced_decode_applicable(ex, batch, P.tiles_by_request, force_single)) {
         const int groups = balanced_groups(kv_subs);
         const size_t prows = bal_partial_row(groups + batch->num_reqs, kv_subs, 0, 0);
-        if (partial_bytes((long long)prows, 1) <= ex->scratch_size) {
+        if (partial_bytes((long long)prows, 1) + (size_t)batch->total_tokens * 16 <= ex->scratch_size) {
             P.part_acc = reinterpret_cast<float*>((uintptr_t)ex->scratch_ptr);
             P.part_ml = P.part_acc + prows * kHeadDim;
+            P.bal_table = reinterpret_cast<int32_t*>(P.part_ml + prows * 4);
             P.max_chunks = groups + 1;
             rc = ensure_dynamic_lds(paged_attn_tq4_balanced_kernel<TQ>, smem_bytes_for(1));
             if (rc) return rc;
@@ -1579,7 +1581,8 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
                                dim3(waves_for(1) * 64), smem_bytes_for(1), stream, P);
             rc = (int)hipGetLastError();
             if (rc) return rc;
-            hipLaunchKernelGGL((balanced_merge_kernel<TQ>), dim3((unsigned)rows), dim3(1024), 0, stream, P, groups,
+            hipLaunchKernelGGL((balanced_merge_kernel<TQ>),
+                               dim3((unsigned)rows), dim3(1024), 0, stream, P,
                                kv_subs, kLutInvGain, 1);
             return (int)hipGetLastError();
         }
@@ -1647,9 +1650,10 @@ static int launch_rows(const warp34_exec* ex, const warp34_kv_layer_layout* layo
     if (balanced_decode_applicable(ex, batch, P.tiles_by_request, force_single)) {
         const int groups = balanced_groups(kv_subs);
         const size_t prows = bal_partial_row(groups + batch->num_reqs, kv_subs, 0, 0);
-        if (partial_bytes((long long)prows, 1) <= ex->scratch_size) {
+        if (partial_bytes((long long)prows, 1) + (size_t)batch->total_tokens * 16 <= ex->scratch_size) {
             P.part_acc = reinterpret_cast<float*>((uintptr_t)ex->scratch_ptr);
             P.part_ml = P.part_acc + prows * kHeadDim;
+            P.bal_table = reinterpret_cast<int32_t*>(P.part_ml + prows * 4);
             P.max_chunks = groups + 1;
             rc = ensure_dynamic_lds(paged_attn_rows_balanced_kernel<TQ, KVF>, kv16_smem_bytes(1));
             if (rc) return rc;
@@ -1657,7 +1661,8 @@ static int launch_rows(const warp34_exec* ex, const warp34_kv_layer_layout* layo
                                dim3(kKv16Waves * 64), kv16_smem_bytes(1), stream, P);
             rc = (int)hipGetLastError();
             if (rc) return rc;
-            hipLaunchKernelGGL((balanced_merge_kernel<TQ>), dim3((unsigned)rows), dim3(1024), 0, stream, P, groups,
+            hipLaunchKernelGGL((balanced_merge_kernel<TQ>),
+                               dim3((unsigned)rows), dim3(1024), 0, stream, P,
                                kv_subs, 1.0f, P.rot_out);
             return (int)hipGetLastError();
         }
@@ -1863,7 +1868,8 @@ extern "C" size_t warp34_paged_attention_scratch_bytes(int total_tokens, int num
     size_t bytes = partial_bytes((long long)total_tokens * num_q_heads, want);
     // balanced decode: (workgroups + requests) partial slots of 16 columns per (kv head, q subgroup);
     // requests <= total_tokens and subgroups <= num_q_heads bound it without the layout
-    const size_t bal = partial_bytes(((long long)kBalWorkgroups + (long long)total_tokens * num_q_heads) * 16, 1);
+    const size_t bal = partial_bytes(((long long)kBalWorkgroups + (long long)total_tokens * num_q_heads) * 16, 1) +
+                       (size_t)total_tokens * 16;  // + the per-token table
     if (total_tokens >= 2 && bal > bytes) bytes = bal;
     return bytes;
 }
