@@ -41,6 +41,8 @@ WORKLOADS = {
     "fp8_prefill_8x2048_ctx16384": ("fp8", [18432] * 8, 0),
     # producer side: QK RMSNorm + RoPE fused with the TQ4 append of an 8 192-token chunk
     "tq4_norm_rope_append_8192": ("tq4", [8192], 0),
+    # consumer side: out = attn_out * sigmoid(gate) over the rows of a 16 384-token prefill step
+    "attn_output_gate_16384x4096": ("tq4", [64], 0),
     # 16 sequences of 262 144 tokens that share the pages of a 200 000-token prefix; 4 query tokens each
     "tq4_verify_16x4_ctx262144_shared200k": ("tq4", [262144] * 16, 0),
 }
@@ -268,6 +270,49 @@ def run_prefill(args, torch, lib, ffi, layers, ctx, n_layers, pool_pages, fmt):
     }))
 
 
+def run_gate(args, torch, lib, ffi):
+    """out = attn_out * sigmoid(gate) on fp16 [16 384, 4 096] (16 q heads x 256): three buffer sets
+    are cycled so that the 403 MB of a step do not come out of the Infinity Cache."""
+    dev = "cuda:0"
+    n, dim, sets = 16384, Q_HEADS * HEAD_DIM, 3
+    g = torch.Generator(device=dev)
+    g.manual_seed(5)
+    bufs = [tuple(torch.randn((n, dim), generator=g, device=dev).to(torch.float16) for _ in range(2)) +
+            (torch.empty((n, dim), dtype=torch.float16, device=dev),) for _ in range(sets)]
+    ex = ffi.Warp34Exec(torch.cuda.current_stream().cuda_stream, 0, 0, 0)
+
+    def step(i):
+        a, gt, o = bufs[i % sets]
+        rc = lib.warp34_apply_attn_output_gate_f16(C.byref(ex), C.c_void_p(a.data_ptr()), C.c_void_p(gt.data_ptr()),
+                                                   C.c_void_p(o.data_ptr()), None, n, dim)
+        if rc:
+            raise RuntimeError("warp34_apply_attn_output_gate_f16 rc=%d" % rc)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(args.steps):
+        step(i)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / args.steps
+    nbytes = 3 * n * dim * 2
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "attention output gate: us/step + achieved HBM GB/s", "value": round(gbs, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 6),
+        "us_per_layer": round(ms * 1e3, 2), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32 arithmetic on f16 rows", "data": "synthetic",
+        "config": {"workload": args.workload, "tokens": n, "total_dim": dim, "bytes_per_step": nbytes},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "attn_output_gate_kernel<true>",
+                     "avg_launch_us": round(ms * 1e3, 2)},
+    }))
+
+
 def run_producer(args, torch, lib, ffi, layers, n, n_layers, fmt):
     """QK RMSNorm + RoPE over packed bf16 [n, (16 + 2 * 2) * 256] rows with the K / V rows written
     into TQ4 pages: the fused entry point against the two-call sequence (operator in place, then
@@ -432,6 +477,9 @@ def run_workload(args, torch, lib, ffi, dev):
 
     if "_prefill_" in args.workload:
         run_prefill(args, torch, lib, ffi, layers, ctx, n_layers, pool_pages, fmt)
+        return None
+    if args.workload.startswith("attn_output_gate"):
+        run_gate(args, torch, lib, ffi)
         return None
     if "_norm_rope_append_" in args.workload:
         run_producer(args, torch, lib, ffi, layers, int(ctx[0]), n_layers, fmt)

@@ -223,6 +223,14 @@ int warp34_dflash_qk_norm_rope_kv_write_bf16_f32_table(
     const warp34_kv_layer_layout* kv_layout, const int32_t* write_slot_mapping,
     int rows, int q_heads, int kv_heads, int dim, int table_rows, float eps);  /* warp34_cuda.h:625-628 */
 
+/* Consumer side of the path: out = attn_out * sigmoid(gate) over fp16 [num_tokens, total_dim]
+ * (replaces ops/op_norms_rope_act.cu:742-759,1329-1344; called right after
+ * warp34_paged_attention_f16 in the gated layers, model/forward.rs:1192-1211).  Rows whose
+ * valid_token_mask byte is 0 are left untouched; the mask may be NULL. */
+int warp34_apply_attn_output_gate_f16(const warp34_exec* ex, const void* attn_out, const void* gate,
+                                      void* out, const uint8_t* valid_token_mask,
+                                      int num_tokens, int total_dim);             /* warp34_cuda.h:297-300 */
+
 /* Bytes of scratch the attention entry points can make use of for a batch of this shape
  * (split-K partials).  No counterpart in the reference, whose engine simply guarantees
  * >= 8 MiB (op_paged_attn.cu:1301-1304); provided so a host can size ex->scratch. */

@@ -334,6 +334,23 @@ def qk_norm_rope_bf16(qkv, positions, qw, kw, table, q_heads, kv_heads, dim, eps
     return qkv, q_out
 
 
+def apply_attn_output_gate_f16(attn_out, gate, out=None, valid_token_mask=None):
+    """ops/op_norms_rope_act.cu:742-759 on uint16 (fp16 bits) [num_tokens, total_dim] arrays."""
+    attn_out = np.ascontiguousarray(attn_out, dtype=np.uint16)
+    gate = np.ascontiguousarray(gate, dtype=np.uint16)
+    if out is None:
+        out = np.zeros_like(attn_out)
+    mask = None if valid_token_mask is None else np.ascontiguousarray(valid_token_mask, dtype=np.uint8)
+    fn = lib().tq4o_apply_attn_output_gate_f16
+    fn.restype = C.c_int
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int]
+    rc = fn(attn_out.ctypes.data, gate.ctypes.data, out.ctypes.data, None if mask is None else mask.ctypes.data,
+            attn_out.shape[0], attn_out.shape[1])
+    if rc:
+        raise RuntimeError("oracle apply_attn_output_gate_f16: rc=%d" % rc)
+    return out
+
+
 def slot_mapping(block_table, ctx_before, n_tokens, block_size):
     """crates/warp34-host/src/model/execution.rs:382-388"""
     pos = np.arange(ctx_before, ctx_before + n_tokens)

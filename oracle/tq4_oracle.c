@@ -409,6 +409,24 @@ int tq4o_qk_norm_rope_bf16(uint16_t* qkv, uint16_t* q_out, const int32_t* positi
     return 0;
 }
 
+/* ---- output gate: apply_attn_output_gate_f16_kernel, ops/op_norms_rope_act.cu:742-759 ----
+ * out = fp16(a * (1 / (1 + expf(-g)))) in fp32, source order. */
+int tq4o_apply_attn_output_gate_f16(const uint16_t* attn_out, const uint16_t* gate, uint16_t* out,
+                                    const uint8_t* valid_token_mask, int num_tokens, int total_dim) {
+    if (!attn_out || !gate || !out) return -1;
+    for (int tok = 0; tok < num_tokens; ++tok) {
+        if (valid_token_mask != NULL && valid_token_mask[tok] == 0) continue;
+        for (int col = 0; col < total_dim; ++col) {
+            const size_t idx = (size_t)tok * total_dim + col;
+            const float a = tq4o_f16_to_f32(attn_out[idx]);
+            const float g = tq4o_f16_to_f32(gate[idx]);
+            const float sig = 1.0f / (1.0f + expf(-g));
+            out[idx] = tq4o_f32_to_f16(a * sig);
+        }
+    }
+    return 0;
+}
+
 /* ---- paged append: op_kv_cache.cu:325-368 ---- */
 int tq4o_kv_cache_write(const tq4o_layout* L, const tq4o_batch* B, const uint16_t* k_in,
                         const uint16_t* v_in, int k_row_stride, int v_row_stride, int in_dtype) {

@@ -138,6 +138,12 @@ int tq4o_qk_norm_rope_bf16(uint16_t* qkv, uint16_t* q_out, const int32_t* positi
                            int kv_heads, int dim, int table_rows, float eps, const tq4o_layout* L,
                            const int32_t* write_slot_mapping);
 
+/* ops/op_norms_rope_act.cu:742-759: out = attn_out * sigmoid(gate), fp16 [num_tokens, total_dim];
+ * rows with a zero mask byte are skipped.  Pinned by the float64 sigmoid within one fp16 ulp,
+ * g = 0 -> a / 2 exactly, saturation at large |g|. */
+int tq4o_apply_attn_output_gate_f16(const uint16_t* attn_out, const uint16_t* gate, uint16_t* out,
+                                    const uint8_t* valid_token_mask, int num_tokens, int total_dim);
+
 int tq4o_paged_attention(const tq4o_layout* L, const tq4o_batch* B,
                          const uint16_t* q, int q_dtype, float* out, int num_q_heads,
                          int n_threads);

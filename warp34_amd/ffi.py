@@ -117,6 +117,8 @@ SIGNATURES = {
     "warp34_dflash_qk_norm_rope_kv_write_bf16_f32_table":
         (C.c_int, [_EX, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, _LAY, C.c_void_p,
                    C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float]),
+    "warp34_apply_attn_output_gate_f16":
+        (C.c_int, [_EX, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int]),
     "warp34_cuda_error_string": (C.c_char_p, [C.c_int]),
     "warp34_get_device_count": (C.c_int, [C.POINTER(C.c_int)]),
     "warp34_set_device": (C.c_int, [C.c_int]),
