@@ -443,7 +443,7 @@ def main():
         import copy
 
         sub = copy.copy(args)
-        sub.workload, sub.steps, sub.warmup = "tq4_decode_b8_ctx131072", 50, 5
+        sub.workload, sub.steps, sub.warmup = "tq4_decode_b8_ctx131072", 200, 20
         torch.cuda.empty_cache()
         r8 = run_workload(sub, torch, lib, ffi, dev)
         result["batch_point"] = {"workload": sub.workload, "us_per_layer": r8["us_per_layer"],
