@@ -793,19 +793,20 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
             // rows 4b+i of the result are tokens unit_token(s, b, i); apply the K scales
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int trow = unit_token(s, b, i);
                 const float d0 = half_lo_to_f32(ks0[s][i]);
                 const float d1 = half_hi_to_f32(ks16[s][i]);
 #pragma unroll
+                for (int nt = 0; nt < NT; ++nt) sc[nt][4 * s + i] = d0 * s_acc[nt][0][i] + d1 * s_acc[nt][1][i];
+            }
+        }
+        if (MASKED) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const int pos = t0 + unit_token(t >> 2, b, t & 3);
+#pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
-                    const float v = d0 * s_acc[nt][0][i] + d1 * s_acc[nt][1][i];
-                    if (MASKED) {
-                        const int pos = t0 + trow;
-                        const bool vis = col_ok[nt] && pos >= col_lo[nt] && pos <= col_hi[nt];
-                        sc[nt][4 * s + i] = vis ? v : kNegBig;
-                    } else {
-                        sc[nt][4 * s + i] = v;
-                    }
+                    const bool vis = col_ok[nt] && pos >= col_lo[nt] && pos <= col_hi[nt];
+                    sc[nt][t] = vis ? sc[nt][t] : kNegBig;
                 }
             }
         }
@@ -834,15 +835,16 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
             m_run[nt] = m_new;
             float p[8];
             float psum = 0.f;
+            // (the MASKED tests sit outside the unrolled loops: one wave-uniform branch per block
+            // instead of one per element, and the eight exponentials can overlap)
 #pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                if (MASKED) {
-                    p[t] = sc[nt][t] > 0.5f * kNegBig ? __builtin_amdgcn_exp2f(sc[nt][t] - m_new) : 0.f;
-                } else {
-                    p[t] = __builtin_amdgcn_exp2f(sc[nt][t] - m_new);
-                }
-                psum += p[t];
+            for (int t = 0; t < 8; ++t) p[t] = __builtin_amdgcn_exp2f(sc[nt][t] - m_new);
+            if (MASKED) {
+#pragma unroll
+                for (int t = 0; t < 8; ++t) p[t] = sc[nt][t] > 0.5f * kNegBig ? p[t] : 0.f;
             }
+#pragma unroll
+            for (int t = 0; t < 8; ++t) psum += p[t];
             l_run[nt] = l_run[nt] * alpha + psum;
             if (__ballot(alpha != 1.0f) != 0ull) {
 #pragma unroll
@@ -850,23 +852,25 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
 #pragma unroll
                     for (int j = 0; j < 8; ++j) o_acc[nt][h][j] *= alpha;
             }
+            float w0[8], w1[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                w0[t] = p[t] * half_lo_to_f32(vd0[t]);
+                w1[t] = p[t] * half_hi_to_f32(vd16[t]);
+            }
+            if (MASKED) {
+                // masked tokens have p == 0; select instead of multiply so that a garbage scale
+                // (rows beyond the sequence end) cannot inject NaN
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    w0[t] = p[t] > 0.f ? w0[t] : 0.f;
+                    w1[t] = p[t] > 0.f ? w1[t] : 0.f;
+                }
+            }
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                const float d0a = half_lo_to_f32(vd0[2 * k]);
-                const float d0b = half_lo_to_f32(vd0[2 * k + 1]);
-                const float d1a = half_hi_to_f32(vd16[2 * k]);
-                const float d1b = half_hi_to_f32(vd16[2 * k + 1]);
-                if (MASKED) {
-                    // masked tokens have p == 0; select instead of multiply so that a garbage
-                    // scale (rows beyond the sequence end) cannot inject NaN
-                    pb[nt][0][k] = pack_h2(p[2 * k] > 0.f ? p[2 * k] * d0a : 0.f,
-                                           p[2 * k + 1] > 0.f ? p[2 * k + 1] * d0b : 0.f);
-                    pb[nt][1][k] = pack_h2(p[2 * k] > 0.f ? p[2 * k] * d1a : 0.f,
-                                           p[2 * k + 1] > 0.f ? p[2 * k + 1] * d1b : 0.f);
-                } else {
-                    pb[nt][0][k] = pack_h2(p[2 * k] * d0a, p[2 * k + 1] * d0b);
-                    pb[nt][1][k] = pack_h2(p[2 * k] * d1a, p[2 * k + 1] * d1b);
-                }
+                pb[nt][0][k] = pack_h2(w0[2 * k], w0[2 * k + 1]);
+                pb[nt][1][k] = pack_h2(w1[2 * k], w1[2 * k + 1]);
             }
         }
 
