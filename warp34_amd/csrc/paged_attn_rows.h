@@ -490,11 +490,13 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
         u2v pb_hi[NT], pb_lo[NT];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
+            // (the MASKED tests sit outside the unrolled loops: one wave-uniform branch per block)
             float sc[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                sc[i] = s_acc[nt][i] * score_scale;
-                if (MASKED) {
+            for (int i = 0; i < 4; ++i) sc[i] = s_acc[nt][i] * score_scale;
+            if (MASKED) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
                     const int pos = pos0 + 4 * b + i;
                     const bool vis = col_ok[nt] && pos >= col_lo[nt] && pos <= col_hi[nt];
                     sc[i] = vis ? sc[i] : kNegBig;
@@ -508,11 +510,13 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
             float p[4];
             float psum = 0.f;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                p[i] = __builtin_amdgcn_exp2f(sc[i] - m_new);
-                if (MASKED) p[i] = sc[i] > 0.5f * kNegBig ? p[i] : 0.f;
-                psum += p[i];
+            for (int i = 0; i < 4; ++i) p[i] = __builtin_amdgcn_exp2f(sc[i] - m_new);
+            if (MASKED) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) p[i] = sc[i] > 0.5f * kNegBig ? p[i] : 0.f;
             }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) psum += p[i];
             l_run[nt] = l_run[nt] * alpha + psum;
             if (__ballot(alpha != 1.0f) != 0ull) {
 #pragma unroll

@@ -335,14 +335,14 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
                 for (int h = 0; h < 2; ++h)
                     s_acc[h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[h][m], bq[h][m], s_acc[h], 0, 0, 0);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const float v = kd0[i] * s_acc[0][i] + kd1[i] * s_acc[1][i];
-                if (MASKED) {
-                    const int pos = t0 + 16 * s + 4 * b + i;
-                    score[4 * s + i] = (col_ok && pos >= col_lo && pos <= col_hi) ? v : kNegBig;
-                } else {
-                    score[4 * s + i] = v;
-                }
+            for (int i = 0; i < 4; ++i) score[4 * s + i] = kd0[i] * s_acc[0][i] + kd1[i] * s_acc[1][i];
+        }
+        // (the MASKED tests sit outside the unrolled loops: one wave-uniform branch per block)
+        if (MASKED) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const int pos = t0 + 16 * (t >> 2) + 4 * b + (t & 3);
+                score[t] = (col_ok && pos >= col_lo && pos <= col_hi) ? score[t] : kNegBig;
             }
         }
         // online softmax, log2 domain; key slot j of this lane = token 16 (j >> 2) + 4 b + (j & 3)
@@ -355,11 +355,13 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         float p[8];
         float psum = 0.f;
 #pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            p[t] = __builtin_amdgcn_exp2f(score[t] - m_new);
-            if (MASKED) p[t] = score[t] > 0.5f * kNegBig ? p[t] : 0.f;
-            psum += p[t];
+        for (int t = 0; t < 8; ++t) p[t] = __builtin_amdgcn_exp2f(score[t] - m_new);
+        if (MASKED) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) p[t] = score[t] > 0.5f * kNegBig ? p[t] : 0.f;
         }
+#pragma unroll
+        for (int t = 0; t < 8; ++t) psum += p[t];
         l_run = l_run * alpha + psum;
         if (__ballot(alpha != 1.0f) != 0ull) {
 #pragma unroll
@@ -374,10 +376,11 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             const f4 db = *reinterpret_cast<const f4*>(sc + 64 + 32 * h + 16 + 4 * b);
             float w[8];
 #pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                const float d = t < 4 ? da[t] : db[t - 4];
+            for (int t = 0; t < 8; ++t) w[t] = p[t] * (t < 4 ? da[t] : db[t - 4]);
+            if (MASKED) {
                 // select, not multiply: a garbage scale of a row beyond the sequence must not make NaN
-                w[t] = MASKED ? (p[t] > 0.f ? p[t] * d : 0.f) : p[t] * d;
+#pragma unroll
+                for (int t = 0; t < 8; ++t) w[t] = p[t] > 0.f ? w[t] : 0.f;
             }
             pb[h] = u4{pack_h2(w[0], w[1]), pack_h2(w[2], w[3]), pack_h2(w[4], w[5]), pack_h2(w[6], w[7])};
         }
