@@ -110,6 +110,7 @@ struct AttnParams {
     int rot_q;             // row-format kernel: K rows are stored rotated, rotate the query rows
     int rot_out;           // row-format kernel: V rows are stored rotated, rotate the output back
     int32_t* bal_table;    // balanced decode: per query token {first partial slot, pieces, token of the tile, -}
+    uint32_t block_magic;  // floor(2^32 / block_size), see div_block
 };
 
 // token of k-slot (s, b, i) inside a unit: spreads the four 4-row groups of an MFMA over LDS
@@ -130,6 +131,18 @@ __device__ __forceinline__ int fast_div(int a, int b) {
     q += r >= b ? 1 : 0;
     q -= r < 0 ? 1 : 0;
     return q;
+}
+
+// pos / block_size for 0 <= pos < 2^31 without a branch: the high word of pos * floor(2^32 / b)
+// is the quotient or one less, one compare settles it.  The inner loops divide a token position
+// by the page size for every group of 16 keys.
+__device__ __forceinline__ int div_block(int pos, const AttnParams& P) {
+    int q = (int)__umulhi((uint32_t)pos, P.block_magic);
+    q += (pos - q * P.L.block_size >= P.L.block_size) ? 1 : 0;
+    return q;
+}
+__host__ inline uint32_t block_magic_for(int block_size) {
+    return block_size <= 1 ? 0xFFFFFFFFu : (uint32_t)((1ull << 32) / (uint32_t)block_size);
 }
 
 struct ChunkGeom {
@@ -609,7 +622,7 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
 #pragma unroll
         for (int gidx = 0; gidx < 2; ++gidx) {
             const int pos = unit * kUnit + 16 * gidx;
-            const int page_slot = fast_div(pos, L.block_size);
+            const int page_slot = div_block(pos, P);
             const int in_page = pos - page_slot * L.block_size;
             int rel = page_slot - slot_base;
             if (rel >= 64) {  // wave-uniform, at most once per 64 slots
@@ -1524,6 +1537,7 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     AttnParams P{};
     P.L = *layout;
     P.B = *batch;
+    P.block_magic = block_magic_for(layout->block_size);
     P.q = (const uint16_t*)q;
     P.out = (uint16_t*)out;
     P.num_q_heads = num_q_heads;
@@ -1611,6 +1625,7 @@ static int launch_rows(const warp34_exec* ex, const warp34_kv_layer_layout* layo
     AttnParams P{};
     P.L = *layout;
     P.B = *batch;
+    P.block_magic = block_magic_for(layout->block_size);
     P.q = (const uint16_t*)q;
     P.out = (uint16_t*)out;
     P.num_q_heads = num_q_heads;
@@ -1706,6 +1721,7 @@ static int launch_prefill_tq4(const warp34_exec* ex, const warp34_kv_layer_layou
     AttnParams P{};
     P.L = *layout;
     P.B = *batch;
+    P.block_magic = block_magic_for(layout->block_size);
     P.q = (const uint16_t*)q;
     P.out = (uint16_t*)out;
     P.part_acc = nullptr;

@@ -307,7 +307,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
     u4 pf[2 * kLoads];
     auto issue_half = [&](int hidx) {  // hidx = 2 * unit + half
         const int pos = hidx * 16;
-        const int page_slot = fast_div(pos, L.block_size);
+        const int page_slot = div_block(pos, P);
         const int in_page = pos - page_slot * L.block_size;
         int rel = page_slot - slot_base;
         if (rel >= 64) {

@@ -177,7 +177,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     // the request's pages are unspecified.
     auto load_page = [&](int k) -> int32_t {
         const int pos = (u_first + k) * kUnit + 16 * (ld_run & 1);
-        const int slot = __builtin_amdgcn_readfirstlane(fast_div(pos, L.block_size));
+        const int slot = __builtin_amdgcn_readfirstlane(div_block(pos, P));
         const bool live = k < n_units && pos <= hi_all && pos + 15 >= lo_all && slot < B.max_blocks_per_req;
         int32_t pg = -1;
         if (live) pg = req_blocks[slot];
@@ -185,7 +185,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     };
     auto issue_loads = [&](int k, int32_t pg) {
         const int pos = (u_first + k) * kUnit + 16 * (ld_run & 1);
-        const int slot = __builtin_amdgcn_readfirstlane(fast_div(pos, L.block_size));
+        const int slot = __builtin_amdgcn_readfirstlane(div_block(pos, P));
         const int in_page = pos - slot * L.block_size;
         size_t off = 0;  // missing page: rows of page 0, every one of them is masked
         if (pg >= 0) off = (size_t)pg * ld_page_stride + (size_t)in_page * ld_tok_stride;
