@@ -263,53 +263,69 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
 #pragma unroll
         for (int j = 0; j < 8; ++j) o_acc[h][j] = f4{0.f, 0.f, 0.f, 0.f};
 
+    // Three phases, each a batch of independent LDS operations: all raw reads, all table reads,
+    // all writes.  (Written item by item, every item's reads would have to wait for the previous
+    // item's writes: the compiler cannot prove that they do not alias.)
     auto dequant_unit = [&](int rawbuf, int deqbuf) {
         const uint32_t raw = (uint32_t)(kPfRawBase + rawbuf * kPfRawBytes);
         const uint32_t deq = (uint32_t)(kPfDeqBase + deqbuf * kPfDeqBytes);
-        // K
+        // ---- phase 1: raw dwords ----
+        uint32_t kw0[2], kw1[2];
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
-            const uint32_t w0 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + k_src[it][0]));
-            const uint32_t w1 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + k_src[it][1]));
-            const uint32_t word = __builtin_amdgcn_alignbit(w1, w0, k_shift[it]);
-            uint2 lo, hi;
-            lo.x = lut_read(word, lut_lane, 0x0c0c0400u);
-            lo.y = lut_read(word, lut_lane, 0x0c0c0500u);
-            hi.x = lut_read(word, lut_lane, 0x0c0c0600u);
-            hi.y = lut_read(word, lut_lane, 0x0c0c0700u);
-            *reinterpret_cast<uint2*>(smem + deq + k_dst[it][0]) = lo;
-            *reinterpret_cast<uint2*>(smem + deq + k_dst[it][1]) = hi;
+            kw0[it] = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + k_src[it][0]));
+            kw1[it] = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + k_src[it][1]));
         }
-        // V
-        {
-            const uint32_t a0 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[0]));
-            const uint32_t a1 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[1]));
-            const uint32_t b0 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[0] + kTq4RowBytes));
-            const uint32_t b1 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[1] + kTq4RowBytes));
-            const uint32_t wa = __builtin_amdgcn_alignbit(a1, a0, v_shift);
-            const uint32_t wb = __builtin_amdgcn_alignbit(b1, b0, v_shift);
-            // byte q of ev / od = (even / odd element of token 2p) | (same of token 2p+1) << 4
-            const uint32_t ev = (wa & 0x0F0F0F0Fu) | ((wb << 4) & 0xF0F0F0F0u);
-            const uint32_t od = ((wa >> 4) & 0x0F0F0F0Fu) | (wb & 0xF0F0F0F0u);
-            const uint32_t first = nibsel ? od : ev;   // elements of parity nibsel, stored at v_dst
-            const uint32_t second = nibsel ? ev : od;  // the other parity, one V^T row (64 B) away
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const uint32_t sel = 0x0c0c0400u + ((uint32_t)q << 8);
-                const uint32_t x0 = lut_read(first, lut_lane, sel);
-                const uint32_t x1 = lut_read(second, lut_lane, sel);
-                const uint32_t addr = deq + v_dst[q];
-                *reinterpret_cast<uint32_t*>(smem + addr) = x0;
-                *reinterpret_cast<uint32_t*>(smem + (addr ^ 64u)) = x1;
-            }
-        }
+        const uint32_t a0 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[0]));
+        const uint32_t a1 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[1]));
+        const uint32_t b0 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[0] + kTq4RowBytes));
+        const uint32_t b1 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[1] + kTq4RowBytes));
         // scales: thread x * 32 + r (x = 0: K d0, 1: K d1, 2: V d0, 3: V d1) of waves 0 and 1
+        uint16_t scale_bits = 0;
         if (tid < 128) {
             const int x = tid >> 5, r = tid & 31;
-            const uint8_t* src = smem + raw + (x >> 1) * (kPfRawBytes / 2) + r * kTq4RowBytes + (x & 1) * 66;
-            const uint16_t bits = *reinterpret_cast<const uint16_t*>(src);
+            scale_bits = *reinterpret_cast<const uint16_t*>(smem + raw + (x >> 1) * (kPfRawBytes / 2) +
+                                                            r * kTq4RowBytes + (x & 1) * 66);
+        }
+        // ---- phase 2: table reads ----
+        uint2 k_lo[2], k_hi[2];
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const uint32_t word = __builtin_amdgcn_alignbit(kw1[it], kw0[it], k_shift[it]);
+            k_lo[it].x = lut_read(word, lut_lane, 0x0c0c0400u);
+            k_lo[it].y = lut_read(word, lut_lane, 0x0c0c0500u);
+            k_hi[it].x = lut_read(word, lut_lane, 0x0c0c0600u);
+            k_hi[it].y = lut_read(word, lut_lane, 0x0c0c0700u);
+        }
+        const uint32_t wa = __builtin_amdgcn_alignbit(a1, a0, v_shift);
+        const uint32_t wb = __builtin_amdgcn_alignbit(b1, b0, v_shift);
+        // byte q of ev / od = (even / odd element of token 2p) | (same of token 2p+1) << 4
+        const uint32_t ev = (wa & 0x0F0F0F0Fu) | ((wb << 4) & 0xF0F0F0F0u);
+        const uint32_t od = ((wa >> 4) & 0x0F0F0F0Fu) | (wb & 0xF0F0F0F0u);
+        const uint32_t first = nibsel ? od : ev;   // elements of parity nibsel, stored at v_dst
+        const uint32_t second = nibsel ? ev : od;  // the other parity, one V^T row (64 B) away
+        uint32_t vx0[4], vx1[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t sel = 0x0c0c0400u + ((uint32_t)q << 8);
+            vx0[q] = lut_read(first, lut_lane, sel);
+            vx1[q] = lut_read(second, lut_lane, sel);
+        }
+        // ---- phase 3: writes ----
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            *reinterpret_cast<uint2*>(smem + deq + k_dst[it][0]) = k_lo[it];
+            *reinterpret_cast<uint2*>(smem + deq + k_dst[it][1]) = k_hi[it];
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t addr = deq + v_dst[q];
+            *reinterpret_cast<uint32_t*>(smem + addr) = vx0[q];
+            *reinterpret_cast<uint32_t*>(smem + (addr ^ 64u)) = vx1[q];
+        }
+        if (tid < 128) {
             *reinterpret_cast<float*>(smem + deq + kPfKBytes + kPfVBytes + 4 * tid) =
-                (float)__builtin_bit_cast(_Float16, bits);
+                (float)__builtin_bit_cast(_Float16, scale_bits);
         }
     };
 
