@@ -264,7 +264,7 @@ def run_prefill(args, torch, lib, ffi, layers, ctx, n_layers, pool_pages, fmt):
                    "attention_flops_per_step": flops, "rows_appended_per_step": N * KV_HEADS * 2},
         "roofline": {"bound": "mfma", "achieved": round(tf_attn, 1), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(tf_attn / peak, 4), "traffic": None,
-                     "kernel": ("paged_prefill_tq4_kernel" if fmt == "tq4" else "paged_attn_rows_kernel") +
+                     "kernel": "paged_prefill_tq4_kernel" +
                                " (attention-only launches)",
                      "avg_launch_us": round(ms_attn * 1e3, 1)},
     }))

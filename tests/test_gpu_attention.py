@@ -317,11 +317,12 @@ def test_kv8_unwritten_pool_bytes_do_not_leak(fmt):
 
 # ---- chunked prefill over TQ4 pages (128-row tile kernel) ----
 
-def _prefill_case(dtype, block_size, seq_lens, q_lens, seed, q_heads=16, force=None, **kw):
+def _prefill_case(dtype, block_size, seq_lens, q_lens, seed, q_heads=16, force=None, fmt=FMT_TQ4, xf=None,
+                  mask_mode=0, window=0, **kw):
     import gpu_harness as G
 
-    pool, bt, k, v, q, aq, ctx = make_case(FMT_TQ4, block_size, seq_lens, q_lens, seed, dtype, q_heads=q_heads)
-    hb = oracle.HostBatch(aq, seq_lens, bt, context_lens_before=ctx, **kw)
+    pool, bt, k, v, q, aq, ctx = make_case(fmt, block_size, seq_lens, q_lens, seed, dtype, q_heads=q_heads, xf=xf)
+    hb = oracle.HostBatch(aq, seq_lens, bt, context_lens_before=ctx, mask_mode=mask_mode, sliding_window=window, **kw)
     want = oracle.paged_attention(pool, hb, q, dtype, q_heads, n_threads=8)
     dpool = _dev_pool(pool)
     rc, got, _ = G.dev_attention(dpool, hb, q, dtype, q_heads, scratch_bytes=SCRATCH, force_kernel=force)
@@ -347,7 +348,40 @@ def test_prefill_tile_kernel_auto_dispatch(dtype):
 
 @pytest.mark.parametrize("mask_mode,window", [(0, 100), (1, 0), (1, 64)])
 def test_prefill_tile_kernel_windows(mask_mode, window):
-    _prefill_case(DT_F16, 16, [400, 130], [90, 130], 221, force=0, mask_mode=mask_mode, sliding_window=window)
+    _prefill_case(DT_F16, 16, [400, 130], [90, 130], 221, force=0, mask_mode=mask_mode, window=window)
+
+
+@pytest.mark.parametrize("xf", [XF_IDENTITY, XF_WHT256])
+@pytest.mark.parametrize("dtype", [DT_BF16, DT_F16])
+def test_prefill_tile_kernel_fp8_pages(xf, dtype):
+    """The tile kernel over FP8-E4M3 pages (same row shape as TQ4: two scale blocks of 128), plain
+    and rotated, through the automatic dispatch and the test selector."""
+    _prefill_case(dtype, 64, [1500, 900], [1100, 650], 331, fmt=FMT_FP8, xf=xf)
+    if dtype == DT_F16:  # the test selector is an f16 entry point
+        _prefill_case(dtype, 16, [300, 77], [130, 40], 332, fmt=FMT_FP8, xf=xf, force=1)
+        _prefill_case(dtype, 64, [700], [333], 333, fmt=FMT_FP8, xf=xf, mask_mode=1, window=64, force=1)
+
+
+def test_prefill_tile_kernel_fp8_unwritten_rows_do_not_leak():
+    """Rows beyond the sequence hold 0xFF bytes (NaN codes, NaN scales) in the last page of each
+    request: the tile kernel must keep them out of the P V product."""
+    import gpu_harness as G
+
+    seq_lens, q_lens = [1500, 901], [1100, 650]
+    pool, bt, k, v, q, aq, ctx = make_case(FMT_FP8, 64, seq_lens, q_lens, 341, DT_F16, q_heads=16)
+    hb = oracle.HostBatch(aq, seq_lens, bt, context_lens_before=ctx)
+    want = oracle.paged_attention(pool, hb, q, DT_F16, 16, n_threads=8)
+    kk = pool.k.reshape(-1, pool.kv_heads, pool.block_size, pool.tok)
+    vv = pool.v.reshape(-1, pool.kv_heads, pool.block_size, pool.tok)
+    for r, s in enumerate(seq_lens):
+        last = bt[r, (s - 1) // 64]
+        kk[last, :, s % 64:, :] = 0xFF
+        vv[last, :, s % 64:, :] = 0xFF
+    dpool = _dev_pool(pool)
+    for force in (None, 1):
+        rc, got, _ = G.dev_attention(dpool, hb, q, DT_F16, 16, scratch_bytes=SCRATCH, force_kernel=force)
+        assert rc == 0
+        G.assert_close(got, DT_F16, want, what="poisoned tail, tile kernel", scale=G.channel_scale(v, DT_F16, hb, 16))
 
 
 def test_prefill_tile_kernel_masks_and_page_permutation():

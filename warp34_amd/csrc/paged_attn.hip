@@ -1715,7 +1715,7 @@ static bool prefill_tq4_applicable(const warp34_kv_layer_layout* layout, const w
     return q_group > 0 && (q_group & (q_group - 1)) == 0 && batch->max_q_len > 0;
 }
 
-template <typename TQ>
+template <typename TQ, int KVF>
 static int launch_prefill_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
                               const warp34_attention_batch* batch, const void* q, void* out, int num_q_heads) {
     AttnParams P{};
@@ -1743,9 +1743,12 @@ static int launch_prefill_tq4(const warp34_exec* ex, const warp34_kv_layer_layou
     P.min_upc = kMinUnitsPerChunk;
     const int tiles = (batch->max_q_len + P.tok_tile - 1) / P.tok_tile;
     const dim3 grid((unsigned)tiles, (unsigned)(layout->local_kv_heads * P.q_subgroups), (unsigned)batch->num_reqs);
-    int rc = ensure_dynamic_lds(paged_prefill_tq4_kernel<TQ>, kPfSmem);
+    P.rot_q = layout->k_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 ? 1 : 0;
+    P.rot_out = layout->v_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 ? 1 : 0;
+    int rc = ensure_dynamic_lds(paged_prefill_tq4_kernel<TQ, KVF>, PfLds<KVF>::kSmem);
     if (rc) return rc;
-    hipLaunchKernelGGL((paged_prefill_tq4_kernel<TQ>), grid, dim3(kPfWaves * 64), kPfSmem, (hipStream_t)ex->stream, P);
+    hipLaunchKernelGGL((paged_prefill_tq4_kernel<TQ, KVF>), grid, dim3(kPfWaves * 64), PfLds<KVF>::kSmem,
+                       (hipStream_t)ex->stream, P);
     return (int)hipGetLastError();
 }
 
@@ -1818,7 +1821,7 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
         const bool many_rows = batch->max_q_len >= 32 &&
                                (long long)batch->total_tokens * num_q_heads >= 128ll * kPfRows;
         if ((force_single || many_rows) && prefill_tq4_applicable(layout, batch, num_q_heads))
-            return launch_prefill_tq4<TQ>(ex, layout, batch, q, out, num_q_heads);
+            return launch_prefill_tq4<TQ, WARP34_KV_FORMAT_TQ4>(ex, layout, batch, q, out, num_q_heads);
         return launch_tq4<TQ>(ex, layout, batch, q, out, num_q_heads, force_single);
     }
     // 16-bit pages: the storage type must be the query type (FP16 pages with the f16 entry
@@ -1830,6 +1833,11 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
     // 8-bit pages (the tail layers of the default TQ4 policy, cache.rs:87-109)
     if (is_kv8(layout, WARP34_KV_FORMAT_FP8_E4M3)) {
         if (!kv8_geometry_ok(layout, q, out, 264)) return (int)hipErrorNotSupported;
+        // many query rows per request: the tile kernel (FP8 rows have the shape of TQ4 rows)
+        const bool many_rows = batch->max_q_len >= 32 &&
+                               (long long)batch->total_tokens * num_q_heads >= 128ll * kPfRows;
+        if ((force_single || many_rows) && prefill_tq4_applicable(layout, batch, num_q_heads))
+            return launch_prefill_tq4<TQ, WARP34_KV_FORMAT_FP8_E4M3>(ex, layout, batch, q, out, num_q_heads);
         return launch_rows<TQ, WARP34_KV_FORMAT_FP8_E4M3>(ex, layout, batch, q, out, num_q_heads, force_single);
     }
     if (is_kv8(layout, WARP34_KV_FORMAT_Q8_0)) {

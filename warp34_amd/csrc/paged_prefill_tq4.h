@@ -1,5 +1,8 @@
-// Chunked-prefill attention over TQ4 pages for gfx950: many query rows per workgroup, every
-// K/V unit dequantised ONCE per workgroup and shared by all waves through LDS.
+// Chunked-prefill attention over TQ4 or FP8-E4M3 pages for gfx950: many query rows per workgroup,
+// every K/V unit dequantised ONCE per workgroup and shared by all waves through LDS.  (FP8 rows
+// have the same shape as TQ4 rows -- two scale blocks of 128 elements -- so only the loader and
+// the dequantiser differ: codes are widened with v_cvt_scalef32_pk_f16_fp8 instead of the table,
+// there is no table in LDS and, for un-rotated layers, no rotation.)
 // Replaces paged_attention_prefill_mma_f16_kernel + launch_prefill
 // (op_paged_attn.cu:594-1128,1220-1259).  Included by paged_attn.hip.
 //
@@ -27,18 +30,31 @@ constexpr int kPfKBytes = 32 * kPfKStride;                    // 16896
 constexpr int kPfVBytes = 256 * 64;                           // V^T: 256 rows x 32 halves
 constexpr int kPfScaleBytes = 4 * 32 * 4;                     // K d0, K d1, V d0, V d1 per token
 constexpr int kPfDeqBytes = kPfKBytes + kPfVBytes + kPfScaleBytes;
-constexpr int kPfRawBytes = kStageTq4;                        // 64 raw rows of 132 B
-constexpr int kPfDeqBase = kLutBytes;
-constexpr int kPfRawBase = kPfDeqBase + 2 * kPfDeqBytes;
-constexpr int kPfSmem = kPfRawBase + 2 * kPfRawBytes + 256;
-static_assert(kPfSmem <= 160 * 1024, "prefill LDS budget");
-static_assert(kPfWaves * 16 * 260 * 4 <= kPfSmem, "epilogue regions must fit");
+// LDS map per page format: [table (TQ4 only)] [2 dequantised units] [2 raw units]
+template <int KVF>
+struct PfLds {
+    static constexpr bool kFp8 = KVF == WARP34_KV_FORMAT_FP8_E4M3;
+    static constexpr int kRowBytes = kFp8 ? 264 : kTq4RowBytes;
+    static constexpr int kRun = 16 * kRowBytes;                // 16 rows: 2112 B / 4224 B
+    static constexpr int kRaw = 4 * kRun;                      // K rows 0-31, V rows 0-31
+    static constexpr int kDeqBase = kFp8 ? 0 : kLutBytes;
+    static constexpr int kRawBase = kDeqBase + 2 * kPfDeqBytes;
+    static constexpr int kLoop = kRawBase + 2 * kRaw + 256;
+    static constexpr int kEpilogue = kPfWaves * 16 * 260 * 4;  // the output transpose regions
+    static constexpr int kSmem = kLoop > kEpilogue ? kLoop : kEpilogue;
+    static_assert(kSmem <= 160 * 1024, "prefill LDS budget");
+};
+static_assert(PfLds<WARP34_KV_FORMAT_TQ4>::kRaw == kStageTq4, "TQ4 raw unit");
 static_assert(kPfWaves * 16 * 264 * 2 <= 2 * kPfDeqBytes, "query staging must fit in the dequant buffers");
 
 typedef __attribute__((address_space(3))) uint32_t lds_u32;
 
-template <typename TQ>
+template <typename TQ, int KVF>
 __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(const AttnParams P) {
+    using M = PfLds<KVF>;
+    constexpr bool FP8 = M::kFp8;
+    constexpr int kPfDeqBase = M::kDeqBase, kPfRawBase = M::kRawBase, kPfRawBytes = M::kRaw;
+    constexpr int kRowB = M::kRowBytes, kRunB = M::kRun;
     extern __shared__ __align__(16) uint8_t smem[];
     if ((uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem != 0u) __builtin_trap();
 
@@ -70,7 +86,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     if (tile_tokens > B.total_tokens - tok0) tile_tokens = B.total_tokens - tok0;
 
     // ---- the pair table (64 lane replicas, as in the decode kernel) ----
-    {
+    if constexpr (!FP8) {
         const int e = tid >> 1;
         const uint32_t v = pack_h2(kLutGain * centroid_of_code(e & 15), kLutGain * centroid_of_code(e >> 4));
         u4 vv = {v, v, v, v};
@@ -113,7 +129,9 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     // ---- rotated, scaled queries of this wave's 16 columns -> LDS -> MFMA B operands ----
     constexpr int kQStride = 264;
     _Float16* qbuf = reinterpret_cast<_Float16*>(smem + kPfDeqBase) + wave * 16 * kQStride;
-    const float q_scale = B.sm_scale * kLog2e * kLutInvGain;
+    const float q_scale = B.sm_scale * kLog2e * (FP8 ? 1.0f : kLutInvGain);
+    const bool rot_q = !FP8 || P.rot_q != 0;
+    const bool rot_out = !FP8 || P.rot_out != 0;
     {
         uint2 q_raw[16];
 #pragma unroll
@@ -132,9 +150,11 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             v[1] = TQ::to_f32((uint16_t)(q_raw[c].x >> 16));
             v[2] = TQ::to_f32((uint16_t)(q_raw[c].y & 0xFFFFu));
             v[3] = TQ::to_f32((uint16_t)(q_raw[c].y >> 16));
+            if (rot_q) {  // keys stored rotated: rotate the query rows
 #pragma unroll
-            for (int k = 0; k < 4; ++k) v[k] = apply_sign(v[k], 4 * lane + k);
-            wht256_wave(v, lane);
+                for (int k = 0; k < 4; ++k) v[k] = apply_sign(v[k], 4 * lane + k);
+                wht256_wave(v, lane);
+            }
             uint2 packed = {0u, 0u};  // dead columns: zero query
             if ((ok_mask >> c) & 1u) {
                 packed.x = pack_h2(v[0] * q_scale, v[1] * q_scale);
@@ -154,9 +174,11 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             bq[h][m] = *reinterpret_cast<const h8*>(qbuf + n * kQStride + 128 * h + 32 * m + 8 * b);
 
     // ---- loader ----
-    // A unit is four runs of 16 rows (2112 B = 132 16-byte pieces): K rows 0-15, K rows 16-31,
-    // V rows 0-15, V rows 16-31.  Waves 2r and 2r+1 load pieces 0-127 of run r (one piece per
-    // lane, wave-uniform base); lanes 0-3 of wave 2r also carry the tail pieces 128-131.
+    // A unit is four runs of 16 rows: K rows 0-15, K rows 16-31, V rows 0-15, V rows 16-31.
+    // TQ4: a run is 2112 B = 132 16-byte pieces; waves 2r and 2r+1 load pieces 0-127 of run r
+    // (one piece per lane, wave-uniform base), lanes 0-3 of wave 2r also carry the tail pieces
+    // 128-131.  FP8: a run is 4224 B = 264 pieces; each wave of the pair loads 132 of them
+    // (two per lane and a four-lane tail).
     const uint8_t* k_base = reinterpret_cast<const uint8_t*>((uintptr_t)L.k_base) +
                             (size_t)kv_head * L.k_head_stride_bytes;
     const uint8_t* v_base = reinterpret_cast<const uint8_t*>((uintptr_t)L.v_base) +
@@ -164,14 +186,15 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     const int32_t* req_blocks = B.block_tables + (size_t)req * B.max_blocks_per_req;
     const int ld_run = wave >> 1;
     const bool ld_is_v = ld_run >= 2;
-    const bool ld_tail = (wave & 1) == 0;  // wave-uniform
+    const bool ld_tail = FP8 || (wave & 1) == 0;  // wave-uniform
     const uint8_t* ld_base = ld_is_v ? v_base : k_base;
     const uint64_t ld_page_stride = ld_is_v ? L.v_page_stride_bytes : L.k_page_stride_bytes;
     const uint64_t ld_tok_stride = ld_is_v ? L.v_token_stride_bytes : L.k_token_stride_bytes;
-    const uint32_t ld_lane_off = (uint32_t)((wave & 1) * 1024 + 16 * lane);
-    const uint32_t ld_commit0 = (uint32_t)(ld_run * kRunBytes) + ld_lane_off;
-    const uint32_t ld_commit1 = (uint32_t)(ld_run * kRunBytes + 2048 + 16 * (lane & 3));
-    u4 pf[2];
+    const uint32_t ld_lane_off = (uint32_t)((wave & 1) * (FP8 ? 2112 : 1024) + 16 * lane);
+    const uint32_t ld_tail_off = (uint32_t)((FP8 ? (wave & 1) * 2112 : 0) + 2048 + 16 * (lane & 3));
+    const uint32_t ld_commit0 = (uint32_t)(ld_run * kRunB) + ld_lane_off;
+    const uint32_t ld_commit1 = (uint32_t)(ld_run * kRunB) + ld_tail_off;
+    u4 pf[FP8 ? 3 : 2];
     // page id of unit k (relative to u_first) for this wave's run; -1 = nothing to fetch.
     // Only groups that overlap the visible key range are fetched: block-table entries beyond
     // the request's pages are unspecified.
@@ -191,12 +214,14 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         if (pg >= 0) off = (size_t)pg * ld_page_stride + (size_t)in_page * ld_tok_stride;
         const uint8_t* src = ld_base + off;
         pf[0] = *(global_cu4*)(src + ld_lane_off);
-        if (ld_tail) pf[1] = *(global_cu4*)(src + 2048 + 16 * (lane & 3));
+        if (ld_tail) pf[1] = *(global_cu4*)(src + ld_tail_off);
+        if constexpr (FP8) pf[2] = *(global_cu4*)(src + ld_lane_off + 1024);
     };
     auto commit_loads = [&](int buf) {
         uint8_t* raw = smem + kPfRawBase + buf * kPfRawBytes;
         *reinterpret_cast<u4*>(raw + ld_commit0) = pf[0];
         if (ld_tail && lane < 4) *reinterpret_cast<u4*>(raw + ld_commit1) = pf[1];
+        if constexpr (FP8) *reinterpret_cast<u4*>(raw + ld_commit0 + 1024) = pf[2];
     };
 
     // ---- dequantiser ----
@@ -329,6 +354,75 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         }
     };
 
+    // FP8 rows: 256 E4M3 codes, then fp32 d0, d1.  Same three phases.  K: thread (row r = tid / 16,
+    // segment g = tid % 16) widens codes 16 g .. 16 g + 15 into the row-major fp16 tile (exact; the
+    // scores take the fp32 scales).  V: thread (token pair p = tid % 16, group j = tid / 16) turns
+    // dims 8 j .. 8 j + 7 of tokens 2p, 2p + 1 into fp16(d * code), each element rounded on its own
+    // (a scale folded into the probabilities would round all 128 elements of a half the same way,
+    // and the inverse rotation of rotated pages gathers such an error into a single channel), and
+    // stores them as (token 2p, token 2p + 1) pairs into the transposed tile, same slots and
+    // swizzle as the TQ4 path.  Value rows outside the visible key range become zeros: unwritten
+    // pool memory may hold NaN codes, and 0 * NaN would poison the P V product.
+    auto dequant_unit_fp8 = [&](int rawbuf, int deqbuf, int t0) {
+        const uint8_t* raw = smem + kPfRawBase + rawbuf * kPfRawBytes;
+        uint8_t* deq = smem + kPfDeqBase + deqbuf * kPfDeqBytes;
+        const int kr = tid >> 4, kg = tid & 15;
+        const int vp = tid & 15, vj = tid >> 4;
+        // ---- phase 1: raw codes and scales ----
+        const u2v kc0 = *reinterpret_cast<const u2v*>(raw + kr * kRowB + 16 * kg);
+        const u2v kc1 = *reinterpret_cast<const u2v*>(raw + kr * kRowB + 16 * kg + 8);
+        u2v va = *reinterpret_cast<const u2v*>(raw + kPfRawBytes / 2 + (2 * vp) * kRowB + 8 * vj);
+        u2v vb = *reinterpret_cast<const u2v*>(raw + kPfRawBytes / 2 + (2 * vp + 1) * kRowB + 8 * vj);
+        float da = *reinterpret_cast<const float*>(raw + kPfRawBytes / 2 + (2 * vp) * kRowB + 256 + 4 * (vj >> 4));
+        float db = *reinterpret_cast<const float*>(raw + kPfRawBytes / 2 + (2 * vp + 1) * kRowB + 256 + 4 * (vj >> 4));
+        float scale = 0.f;
+        if (tid < 64) {
+            const int x = tid >> 5, r = tid & 31;  // K d0, K d1
+            scale = *reinterpret_cast<const float*>(raw + r * kRowB + 256 + 4 * x);
+        }
+        // ---- phase 2: widen ----
+        u4 k_lo, k_hi;
+        {
+            uint32_t h[8];
+            fp8x4_to_h4(kc0[0], h[0], h[1]);
+            fp8x4_to_h4(kc0[1], h[2], h[3]);
+            fp8x4_to_h4(kc1[0], h[4], h[5]);
+            fp8x4_to_h4(kc1[1], h[6], h[7]);
+            k_lo = u4{h[0], h[1], h[2], h[3]};
+            k_hi = u4{h[4], h[5], h[6], h[7]};
+        }
+        {
+            const int pa = t0 + 2 * vp;
+            const bool a_ok = pa >= lo_all && pa <= hi_all, b_ok = pa + 1 >= lo_all && pa + 1 <= hi_all;
+            va[0] = a_ok ? va[0] : 0u, va[1] = a_ok ? va[1] : 0u, da = a_ok ? da : 0.f;
+            vb[0] = b_ok ? vb[0] : 0u, vb[1] = b_ok ? vb[1] : 0u, db = b_ok ? db : 0.f;
+        }
+        float fa[8], fb[8];
+        {
+            float t[4];
+            codes4_to_f32<true>(va[0], t);
+            fa[0] = t[0], fa[1] = t[1], fa[2] = t[2], fa[3] = t[3];
+            codes4_to_f32<true>(va[1], t);
+            fa[4] = t[0], fa[5] = t[1], fa[6] = t[2], fa[7] = t[3];
+            codes4_to_f32<true>(vb[0], t);
+            fb[0] = t[0], fb[1] = t[1], fb[2] = t[2], fb[3] = t[3];
+            codes4_to_f32<true>(vb[1], t);
+            fb[4] = t[0], fb[5] = t[1], fb[6] = t[2], fb[7] = t[3];
+        }
+        // ---- phase 3: writes ----
+        *reinterpret_cast<u4*>(deq + kr * kPfKStride + 32 * kg) = k_lo;
+        *reinterpret_cast<u4*>(deq + kr * kPfKStride + 32 * kg + 16) = k_hi;
+        const int bp = (vp >> 1) & 3, sl = vp >> 3;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int d = 8 * vj + e;
+            // (token 2p, token 2p + 1) of dim d
+            *reinterpret_cast<uint32_t*>(deq + kPfKBytes + d * 64 + 16 * (bp ^ ((d >> 1) & 3)) + 8 * sl + 4 * (vp & 1)) =
+                pack_h2(da * fa[e], db * fb[e]);
+        }
+        if (tid < 64) *reinterpret_cast<float*>(deq + kPfKBytes + kPfVBytes + 4 * tid) = scale;
+    };
+
     auto compute_unit = [&](int deqbuf, int t0, const bool MASKED) {
         const uint8_t* kb = smem + kPfDeqBase + deqbuf * kPfDeqBytes;
         const uint8_t* vb = kb + kPfKBytes;
@@ -386,19 +480,24 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
                 for (int j = 0; j < 8; ++j) o_acc[h][j] *= alpha;
         }
         u4 pb[2];
+        if constexpr (FP8) {  // the value tile already carries its scales
+            pb[0] = u4{pack_h2(p[0], p[1]), pack_h2(p[2], p[3]), pack_h2(p[4], p[5]), pack_h2(p[6], p[7])};
+            pb[1] = pb[0];
+        } else {
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const f4 da = *reinterpret_cast<const f4*>(sc + 64 + 32 * h + 4 * b);
-            const f4 db = *reinterpret_cast<const f4*>(sc + 64 + 32 * h + 16 + 4 * b);
-            float w[8];
+            for (int h = 0; h < 2; ++h) {
+                const f4 da = *reinterpret_cast<const f4*>(sc + 64 + 32 * h + 4 * b);
+                const f4 db = *reinterpret_cast<const f4*>(sc + 64 + 32 * h + 16 + 4 * b);
+                float w[8];
 #pragma unroll
-            for (int t = 0; t < 8; ++t) w[t] = p[t] * (t < 4 ? da[t] : db[t - 4]);
-            if (MASKED) {
-                // select, not multiply: a garbage scale of a row beyond the sequence must not make NaN
+                for (int t = 0; t < 8; ++t) w[t] = p[t] * (t < 4 ? da[t] : db[t - 4]);
+                if (MASKED) {
+                    // select, not multiply: a garbage scale of a row beyond the sequence must not make NaN
 #pragma unroll
-                for (int t = 0; t < 8; ++t) w[t] = p[t] > 0.f ? w[t] : 0.f;
+                    for (int t = 0; t < 8; ++t) w[t] = p[t] > 0.f ? w[t] : 0.f;
+                }
+                pb[h] = u4{pack_h2(w[0], w[1]), pack_h2(w[2], w[3]), pack_h2(w[4], w[5]), pack_h2(w[6], w[7])};
             }
-            pb[h] = u4{pack_h2(w[0], w[1]), pack_h2(w[2], w[3]), pack_h2(w[4], w[5]), pack_h2(w[6], w[7])};
         }
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
@@ -434,7 +533,13 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
 #ifdef W34_TRACE
         if (it >= 8 && it < 16) W34_TP(4 + 5 * (it - 8) + 1);
 #endif
-        if (it + 1 >= 0 && it + 1 < n_units) dequant_unit((it + 1) & 1, (it + 1) & 1);
+        if (it + 1 >= 0 && it + 1 < n_units) {
+            if constexpr (FP8) {
+                dequant_unit_fp8((it + 1) & 1, (it + 1) & 1, (u_first + it + 1) * kUnit);
+            } else {
+                dequant_unit((it + 1) & 1, (it + 1) & 1);
+            }
+        }
 #ifdef W34_TRACE
         if (it >= 8 && it < 16) W34_TP(4 + 5 * (it - 8) + 2);
 #endif
@@ -455,7 +560,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     // ---- epilogue: normalise, transpose through LDS, rotate back, store ----
     l_run = sum_over_rows(l_run);
     float* reg = reinterpret_cast<float*>(smem) + wave * 16 * 260;
-    const float inv = l_run > 0.f ? kLutInvGain / l_run : 0.f;
+    const float inv = l_run > 0.f ? (FP8 ? 1.0f : kLutInvGain) / l_run : 0.f;
 #pragma unroll
     for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -471,9 +576,11 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         const int a = col - t * P.q_group;
         const f4 x = *reinterpret_cast<const f4*>(reg + c * 260 + 4 * lane);
         float o[4] = {x[0], x[1], x[2], x[3]};
-        wht256_wave(o, lane);
+        if (rot_out) {  // values stored rotated: rotate the finished row back
+            wht256_wave(o, lane);
 #pragma unroll
-        for (int k = 0; k < 4; ++k) o[k] = apply_sign(o[k], 4 * lane + k);
+            for (int k = 0; k < 4; ++k) o[k] = apply_sign(o[k], 4 * lane + k);
+        }
         uint2 ob;
         ob.x = (uint32_t)TQ::from_f32(o[0]) | ((uint32_t)TQ::from_f32(o[1]) << 16);
         ob.y = (uint32_t)TQ::from_f32(o[2]) | ((uint32_t)TQ::from_f32(o[3]) << 16);
