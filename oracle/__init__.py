@@ -351,6 +351,32 @@ def apply_attn_output_gate_f16(attn_out, gate, out=None, valid_token_mask=None):
     return out
 
 
+def qsa_sparse_paged_attn_f16(pool, q_bits, sel_phys, sel_log, num_sel, seq_pos, num_q_heads, sm_scale=0.0625,
+                              gate=None, valid_token_mask=None, hadamard64=False):
+    """ops/op_qsa.cu:716-1158,1446-1571: fp16 bits in, fp16 bits out [tokens, q heads, 256]."""
+    q_bits = np.ascontiguousarray(q_bits, dtype=np.uint16)
+    sel_phys = np.ascontiguousarray(sel_phys, dtype=np.int32)
+    sel_log = np.ascontiguousarray(sel_log, dtype=np.int32)
+    num_sel = np.ascontiguousarray(num_sel, dtype=np.int32)
+    seq_pos = np.ascontiguousarray(seq_pos, dtype=np.int32)
+    n_tok, select_k = sel_phys.shape
+    assert sel_log.shape == sel_phys.shape and num_sel.shape == (n_tok,) and seq_pos.shape == (n_tok,)
+    g = None if gate is None else np.ascontiguousarray(gate, dtype=np.uint16)
+    mask = None if valid_token_mask is None else np.ascontiguousarray(valid_token_mask, dtype=np.uint8)
+    out = np.zeros((n_tok, num_q_heads, 256), dtype=np.uint16)
+    fn = lib().tq4o_qsa_sparse_paged_attn_f16
+    fn.restype = C.c_int
+    fn.argtypes = [C.c_void_p] * 9 + [C.c_int, C.c_int, C.c_int, C.c_float, C.c_int]
+    L = pool.layout()
+    rc = fn(C.addressof(L), q_bits.ctypes.data, None if g is None else g.ctypes.data, sel_phys.ctypes.data,
+            sel_log.ctypes.data, num_sel.ctypes.data, seq_pos.ctypes.data,
+            None if mask is None else mask.ctypes.data, out.ctypes.data, n_tok, num_q_heads, select_k,
+            sm_scale, 1 if hadamard64 else 0)
+    if rc:
+        raise RuntimeError("oracle qsa_sparse_paged_attn_f16: rc=%d" % rc)
+    return out
+
+
 def slot_mapping(block_table, ctx_before, n_tokens, block_size):
     """crates/warp34-host/src/model/execution.rs:382-388"""
     pos = np.arange(ctx_before, ctx_before + n_tokens)

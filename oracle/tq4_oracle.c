@@ -843,6 +843,115 @@ void tq4o_fill_kv_rows(uint16_t* dst, size_t rows, int kv_heads, int head_dim, u
     free(perm);
 }
 
+/* ---- QSA sparse paged attention: op_qsa.cu:716-1073 (grouped kernel), :1075-1158 (split merge),
+ * :1161-1445 (generic kernel), hadamard_inline.cuh:11-50 (per-64 output transform) ----
+ * Every query token attends over its own list of selected 4-token groups.  Group j of token t is
+ * rows (phys % gpp) * 4 .. + 3 of physical page phys / gpp with gpp = block_size / 4
+ * (phys = selected_phys_blocks[t * select_k + j]); its keys sit at sequence positions
+ * 4 * selected_logical_blocks[..] + 0..3.  A group with phys < 0 and a key behind token_seq_pos[t]
+ * are skipped.  The normalised sum is rotated back, multiplied by sigmoid(gate) and rounded to
+ * fp16; the hadamard form then transforms every 64-element block of the rounded row.  Masked
+ * tokens and tokens without a visible key give zero rows.  Scores and sums in fp64 (declared
+ * oracle numerics); the per-64 transform in fp32 in the reference's order of additions. */
+static void hadamard64_rows_f16(uint16_t* row, int n) {
+    for (int blk = 0; blk + 64 <= n; blk += 64) {
+        float v[16][4];
+        for (int l = 0; l < 16; ++l) {
+            const float x0 = tq4o_f16_to_f32(row[blk + 4 * l]), x1 = tq4o_f16_to_f32(row[blk + 4 * l + 1]);
+            const float x2 = tq4o_f16_to_f32(row[blk + 4 * l + 2]), x3 = tq4o_f16_to_f32(row[blk + 4 * l + 3]);
+            const float a0 = x0 + x1, a1 = x0 - x1, a2 = x2 + x3, a3 = x2 - x3;
+            v[l][0] = a0 + a2; v[l][1] = a1 + a3; v[l][2] = a0 - a2; v[l][3] = a1 - a3;
+        }
+        for (int h = 1; h < 16; h <<= 1) {
+            float w[16][4];
+            for (int l = 0; l < 16; ++l)
+                for (int k = 0; k < 4; ++k) {
+                    const float o = v[l ^ h][k];
+                    w[l][k] = (l & h) ? (o - v[l][k]) : (v[l][k] + o);
+                }
+            memcpy(v, w, sizeof(v));
+        }
+        for (int l = 0; l < 16; ++l)
+            for (int k = 0; k < 4; ++k) row[blk + 4 * l + k] = tq4o_f32_to_f16(v[l][k] * 0.125f);
+    }
+}
+
+int tq4o_qsa_sparse_paged_attn_f16(const tq4o_layout* L, const uint16_t* q, const uint16_t* gate,
+                                   const int32_t* selected_phys_blocks, const int32_t* selected_logical_blocks,
+                                   const int32_t* num_selected_blocks, const int32_t* token_seq_pos,
+                                   const uint8_t* valid_token_mask, uint16_t* out, int num_tokens,
+                                   int local_q_heads, int select_k_blocks, float sm_scale, int hadamard64) {
+    if (!L || !q || !selected_phys_blocks || !selected_logical_blocks || !num_selected_blocks || !token_seq_pos ||
+        !out || num_tokens < 0 || local_q_heads <= 0 || L->local_kv_heads <= 0 ||
+        local_q_heads % L->local_kv_heads || L->head_dim != 256 || select_k_blocks < 0)
+        return -1;
+    const int hd = 256, g = local_q_heads / L->local_kv_heads, gpp = L->block_size >> 2;
+    if (gpp <= 0 || g > 64) return -1;
+    float* qrows = (float*)malloc((size_t)g * hd * sizeof(float));
+    double* acc = (double*)malloc((size_t)g * hd * sizeof(double));
+    double* sc = (double*)malloc((size_t)(select_k_blocks > 0 ? select_k_blocks : 1) * 4 * g * sizeof(double));
+    const uint8_t** vrows = (const uint8_t**)malloc((size_t)(select_k_blocks > 0 ? select_k_blocks : 1) * 4 * sizeof(void*));
+    float kv[256], res[256];
+    for (int tok = 0; tok < num_tokens; ++tok) {
+        if (valid_token_mask && !valid_token_mask[tok]) {
+            memset(out + (size_t)tok * local_q_heads * hd, 0, (size_t)local_q_heads * hd * 2);
+            continue;
+        }
+        int n_sel = num_selected_blocks[tok];
+        if (n_sel > select_k_blocks) n_sel = select_k_blocks;
+        const int seq_pos = token_seq_pos[tok];
+        for (int h = 0; h < L->local_kv_heads; ++h) {
+            load_q(L, q, TQ4O_DT_F16, tok, local_q_heads, h * g, g, qrows);
+            int n = 0;
+            double m[64];
+            for (int a = 0; a < g; ++a) m[a] = -INFINITY;
+            for (int j = 0; j < n_sel; ++j) {
+                const int32_t phys = selected_phys_blocks[(size_t)tok * select_k_blocks + j];
+                const int32_t lg = selected_logical_blocks[(size_t)tok * select_k_blocks + j];
+                for (int off = 0; off < 4; ++off) {
+                    if (phys < 0 || lg * 4 + off > seq_pos) continue;
+                    const size_t page = (size_t)(phys / gpp), row = (size_t)(phys % gpp) * 4 + off;
+                    read_row(L->k_base + page * L->k_page_stride + (size_t)h * L->k_head_stride + row * L->k_token_stride,
+                             L->k_format, hd, kv);
+                    vrows[n] = L->v_base + page * L->v_page_stride + (size_t)h * L->v_head_stride + row * L->v_token_stride;
+                    for (int a = 0; a < g; ++a) {
+                        double dot = 0.0;
+                        for (int c = 0; c < hd; ++c) dot += (double)qrows[(size_t)a * hd + c] * (double)kv[c];
+                        const double s = dot * (double)sm_scale;
+                        sc[(size_t)n * g + a] = s;
+                        if (s > m[a]) m[a] = s;
+                    }
+                    ++n;
+                }
+            }
+            double l[64];
+            for (int a = 0; a < g; ++a) l[a] = 0.0;
+            for (size_t i = 0; i < (size_t)g * hd; ++i) acc[i] = 0.0;
+            for (int i = 0; i < n; ++i) {
+                read_row(vrows[i], L->v_format, hd, kv);
+                for (int a = 0; a < g; ++a) {
+                    const double p = exp(sc[(size_t)i * g + a] - m[a]);
+                    l[a] += p;
+                    for (int c = 0; c < hd; ++c) acc[(size_t)a * hd + c] += p * (double)kv[c];
+                }
+            }
+            for (int a = 0; a < g; ++a) {
+                const size_t rowi = (size_t)tok * local_q_heads + (size_t)h * g + a;
+                store_out(L, acc + (size_t)a * hd, l[a], res);
+                uint16_t* dst = out + rowi * hd;
+                for (int c = 0; c < hd; ++c) {
+                    double val = (double)res[c];
+                    if (gate) val *= 1.0 / (1.0 + exp(-(double)tq4o_f16_to_f32(gate[rowi * hd + c])));
+                    dst[c] = tq4o_f32_to_f16((float)val);
+                }
+                if (hadamard64) hadamard64_rows_f16(dst, hd);
+            }
+        }
+    }
+    free(qrows); free(acc); free(sc); free(vrows);
+    return 0;
+}
+
 int tq4o_hw_threads(void) {
     long n = sysconf(_SC_NPROCESSORS_ONLN);
     return n > 0 ? (int)n : 1;

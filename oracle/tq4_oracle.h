@@ -40,6 +40,11 @@
  *                     preserved; V bit-identical; cache rows = append of the rotated K.  The
  *                     reference's golden tensors for this operator are not in its tree (LFS
  *                     pointers only), so exact bf16 bits are "parity unpinned"
+ *   tq4o_qsa_sparse   the reference test's known answer (V = 0.25, gate 0 -> 0.125, ple/gpu_tests.rs:677-681);
+ *                     all groups of a sequence selected = dense causal attention of the last token;
+ *                     brute-force fp64 softmax over independently dequantised rows with skipped groups,
+ *                     keys behind the token position and masked tokens; per-64 transform = Sylvester
+ *                     H64 / 8, exact on small integers, an involution
  */
 #ifndef TQ4_ORACLE_H
 #define TQ4_ORACLE_H
@@ -143,6 +148,14 @@ int tq4o_qk_norm_rope_bf16(uint16_t* qkv, uint16_t* q_out, const int32_t* positi
  * g = 0 -> a / 2 exactly, saturation at large |g|. */
 int tq4o_apply_attn_output_gate_f16(const uint16_t* attn_out, const uint16_t* gate, uint16_t* out,
                                     const uint8_t* valid_token_mask, int num_tokens, int total_dim);
+
+/* QSA sparse paged attention over selected 4-token groups (op_qsa.cu:716-1158,1446-1571;
+ * hadamard_inline.cuh:11-50); fp16 query, gate and output bits. */
+int tq4o_qsa_sparse_paged_attn_f16(const tq4o_layout* L, const uint16_t* q, const uint16_t* gate,
+                                   const int32_t* selected_phys_blocks, const int32_t* selected_logical_blocks,
+                                   const int32_t* num_selected_blocks, const int32_t* token_seq_pos,
+                                   const uint8_t* valid_token_mask, uint16_t* out, int num_tokens,
+                                   int local_q_heads, int select_k_blocks, float sm_scale, int hadamard64);
 
 int tq4o_paged_attention(const tq4o_layout* L, const tq4o_batch* B,
                          const uint16_t* q, int q_dtype, float* out, int num_q_heads,

@@ -36,3 +36,22 @@ def make_case(fmt, block_size, seq_lens, q_lens, seed, dtype, kv_heads=2, q_head
     q = oracle.fill_normal(aq[-1] * q_heads * 256, seed + 2, dtype).reshape(aq[-1], q_heads, 256)
     ctx = [s - ql for s, ql in zip(seq_lens, q_lens)]
     return pool, bt, k, v, q, aq, ctx
+
+
+def qsa_groups_of(bt, seq_lens, block_size, select_k):
+    """Every 4-token group of each sequence in logical order, as the selection lists of the QSA
+    sparse attention (ops/op_qsa.cu:812-822): physical group = page * (block_size / 4) + group in
+    page, logical group = position / 4; unused entries are -1."""
+    gpp = block_size // 4
+    n = len(seq_lens)
+    sel_phys = np.full((n, select_k), -1, dtype=np.int32)
+    sel_log = np.zeros((n, select_k), dtype=np.int32)
+    num_sel = np.zeros(n, dtype=np.int32)
+    for r, s in enumerate(seq_lens):
+        groups = (s + 3) // 4
+        assert groups <= select_k
+        lg = np.arange(groups)
+        sel_phys[r, :groups] = np.asarray(bt[r])[lg * 4 // block_size] * gpp + (lg * 4 % block_size) // 4
+        sel_log[r, :groups] = lg
+        num_sel[r] = groups
+    return sel_phys, sel_log, num_sel
