@@ -231,6 +231,31 @@ int warp34_apply_attn_output_gate_f16(const warp34_exec* ex, const void* attn_ou
                                       void* out, const uint8_t* valid_token_mask,
                                       int num_tokens, int total_dim);             /* warp34_cuda.h:297-300 */
 
+/* QSA sparse paged attention: query token t attends over its own list of selected 4-token groups
+ * (replaces ops/op_qsa.cu:716-1158,1446-1571,1711-1751).  Group j of token t is rows
+ * (phys % (block_size / 4)) * 4 .. + 3 of page phys / (block_size / 4), phys =
+ * selected_phys_blocks[t * select_k_blocks + j]; its keys sit at positions
+ * 4 * selected_logical_blocks[..] + 0..3.  Groups with phys < 0, groups at or behind
+ * num_selected_blocks[t] and keys behind token_seq_pos[t] are skipped.  out = fp16(attention *
+ * sigmoid(gate)) (gate may be NULL); the hadamard form then applies H64 / 8 to every 64-element
+ * block of the rounded row (ops/hadamard_inline.cuh:11-50).  Rows of masked tokens and of tokens
+ * without a visible key are written as zeros.  q, gate, out: fp16 [num_tokens, local_q_heads, 256].
+ * Built for rotated TQ4 pages (k/v format TQ4, transform RADEMACHER_WHT256); the reference's other
+ * page formats return hipErrorNotSupported.  Uses ex->scratch for split partials when it is large
+ * enough (num_tokens * local_q_heads * splits * 1040 bytes, splits <= 16). */
+int warp34_qsa_sparse_paged_attn_f16(const warp34_exec* ex, const void* q, const void* gate,
+                                     const warp34_kv_layer_layout* kv_layout,
+                                     const int32_t* selected_phys_blocks,
+                                     const int32_t* selected_logical_blocks,
+                                     const int32_t* num_selected_blocks, const int32_t* token_seq_pos,
+                                     const uint8_t* valid_token_mask, void* out, int num_tokens,
+                                     int local_q_heads, int select_k_blocks, float sm_scale);  /* warp34_cuda.h:851-859 */
+int warp34_qsa_sparse_paged_attn_hadamard_f16(
+    const warp34_exec* ex, const void* q, const void* gate, const warp34_kv_layer_layout* kv_layout,
+    const int32_t* selected_phys_blocks, const int32_t* selected_logical_blocks,
+    const int32_t* num_selected_blocks, const int32_t* token_seq_pos, const uint8_t* valid_token_mask,
+    void* out, int num_tokens, int local_q_heads, int select_k_blocks, float sm_scale);  /* warp34_cuda.h:860-865 */
+
 /* Bytes of scratch the attention entry points can make use of for a batch of this shape
  * (split-K partials).  No counterpart in the reference, whose engine simply guarantees
  * >= 8 MiB (op_paged_attn.cu:1301-1304); provided so a host can size ex->scratch. */

@@ -187,3 +187,25 @@ def assert_close(got_bits, dtype, want_f32, atol=2e-3, rtol=1e-2, what="", scale
         what, float(err.max()), max_rel, worst)
     assert max_rel <= rtol, "%s: max-rel %.3e" % (what, max_rel)
     return float(err.max()) if err.size else 0.0
+
+
+def dev_qsa_sparse(dpool, q_bits, sel_phys, sel_log, num_sel, seq_pos, num_q_heads, sm_scale=0.0625, gate=None,
+                   valid_token_mask=None, hadamard64=False, scratch_bytes=0, sentinel=0x5500, layout=None):
+    """QSA sparse paged attention through the C ABI.  Returns (rc, out_bits uint16 [N, H, 256])."""
+    L = dpool.layout() if layout is None else layout
+    ex, ws = make_exec(scratch_bytes)
+    sel_phys = np.ascontiguousarray(sel_phys, dtype=np.int32)
+    n_tok, select_k = sel_phys.shape
+    d = dict(q=to_dev(q_bits), gate=to_dev(gate), phys=to_dev(sel_phys),
+             log=to_dev(np.ascontiguousarray(sel_log, dtype=np.int32)),
+             num=to_dev(np.ascontiguousarray(num_sel, dtype=np.int32)),
+             pos=to_dev(np.ascontiguousarray(seq_pos, dtype=np.int32)),
+             mask=to_dev(None if valid_token_mask is None else np.ascontiguousarray(valid_token_mask, dtype=np.uint8)))
+    out = torch.full((n_tok, num_q_heads, 256), sentinel, dtype=torch.int16, device=DEV)
+    fn = lib().warp34_qsa_sparse_paged_attn_hadamard_f16 if hadamard64 else lib().warp34_qsa_sparse_paged_attn_f16
+    rc = fn(C.byref(ex), ptr(d["q"]), ptr(d["gate"]), C.byref(L), ptr(d["phys"]), ptr(d["log"]), ptr(d["num"]),
+            ptr(d["pos"]), ptr(d["mask"]), ptr(out), n_tok, num_q_heads, select_k, sm_scale)
+    torch.cuda.synchronize()
+    if ws is not None:
+        assert bool((ws[scratch_bytes:] == 0x5A).all()), "scratch canary overwritten"
+    return rc, out.cpu().numpy().view(np.uint16)

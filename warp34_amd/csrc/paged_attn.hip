@@ -1471,6 +1471,7 @@ __device__ __forceinline__ TileInfo locate_tile(const AttnParams& P, int tile_z,
 
 #include "paged_attn_rows.h"
 #include "paged_prefill_tq4.h"
+#include "qsa_sparse_tq4.h"
 
 namespace w34 {
 
@@ -1847,6 +1848,81 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
     return (int)hipErrorNotSupported;
 }
 
+// QSA sparse paged attention (op_qsa.cu:1446-1571).  Argument checks and error codes follow the
+// reference's launcher; the split count is this kernel's own (enough workgroups to fill the chip,
+// at least one unit per wave and split, scratch permitting).
+static int launch_qsa_sparse(const warp34_exec* ex, const void* q, const void* gate,
+                             const warp34_kv_layer_layout* layout, const int32_t* selected_phys_blocks,
+                             const int32_t* selected_logical_blocks, const int32_t* num_selected_blocks,
+                             const int32_t* token_seq_pos, const uint8_t* valid_token_mask, void* out,
+                             int num_tokens, int local_q_heads, int select_k_blocks, float sm_scale, int had64) {
+    if (!ex || !q || !layout || !selected_phys_blocks || !selected_logical_blocks || !num_selected_blocks ||
+        !token_seq_pos || !out || num_tokens < 0 || local_q_heads <= 0 || layout->local_kv_heads <= 0 ||
+        (local_q_heads % layout->local_kv_heads) != 0 || layout->head_dim != 256 || select_k_blocks < 0) {
+        return (int)hipErrorInvalidValue;
+    }
+    if (num_tokens == 0) return 0;
+    // built for rotated TQ4 pages; the 16-bit and 8-bit page formats of the reference's kernel are
+    // reported as unsupported, never computed some other way
+    if (!is_tq4_wht(layout)) return (int)hipErrorNotSupported;
+    if (!tq4_geometry_ok(layout, q) || (layout->block_size & 3) != 0 || (((uintptr_t)out) & 7u) != 0 ||
+        (gate != nullptr && (((uintptr_t)gate) & 7u) != 0))
+        return (int)hipErrorNotSupported;
+    QsaParams P{};
+    P.L = *layout;
+    P.q = (const uint16_t*)q;
+    P.gate = (const uint16_t*)gate;
+    P.out = (uint16_t*)out;
+    P.sel_phys = selected_phys_blocks;
+    P.sel_log = selected_logical_blocks;
+    P.num_sel = num_selected_blocks;
+    P.seq_pos = token_seq_pos;
+    P.valid_token_mask = valid_token_mask;
+    P.num_tokens = num_tokens;
+    P.num_q_heads = local_q_heads;
+    P.gqa = local_q_heads / layout->local_kv_heads;
+    int q_group = P.gqa;
+    if (q_group > 16) {
+        for (int d = 16; d >= 1; --d)
+            if (P.gqa % d == 0) {
+                q_group = d;
+                break;
+            }
+    }
+    P.q_group = q_group;
+    P.q_subgroups = P.gqa / q_group;
+    P.select_k = select_k_blocks;
+    P.groups_per_page = layout->block_size / 4;
+    P.sm_scale = sm_scale;
+    P.had64 = had64;
+    const int kv_subs = layout->local_kv_heads * P.q_subgroups;
+    const int max_units = (select_k_blocks + 7) / 8;
+    long long want = 256ll / ((long long)num_tokens * kv_subs);
+    if (want > kQsaMaxSplits) want = kQsaMaxSplits;
+    const int by_units = (max_units + kQsaWaves - 1) / kQsaWaves;
+    if (want > by_units) want = by_units;
+    if (want < 1) want = 1;
+    const size_t rows = (size_t)num_tokens * local_q_heads;
+    const size_t need = rows * (size_t)want * (kHeadDim + 4) * sizeof(float);
+    P.n_splits = (want > 1 && ex->scratch_ptr != 0 && ex->scratch_size >= need) ? (int)want : 1;
+    if (P.n_splits > 1) {
+        P.part_acc = reinterpret_cast<float*>((uintptr_t)ex->scratch_ptr);
+        P.part_ml = P.part_acc + rows * P.n_splits * kHeadDim;
+    }
+    hipStream_t stream = (hipStream_t)ex->stream;
+    int rc = ensure_dynamic_lds(qsa_sparse_tq4_kernel, kQsaSmem);
+    if (rc) return rc;
+    hipLaunchKernelGGL(qsa_sparse_tq4_kernel, dim3((unsigned)num_tokens, (unsigned)kv_subs, (unsigned)P.n_splits),
+                       dim3(kQsaWaves * 64), kQsaSmem, stream, P);
+    rc = (int)hipGetLastError();
+    if (rc) return rc;
+    if (P.n_splits > 1) {
+        hipLaunchKernelGGL(qsa_sparse_merge_kernel, dim3((unsigned)rows), dim3(64), 0, stream, P);
+        rc = (int)hipGetLastError();
+    }
+    return rc;
+}
+
 }  // namespace w34
 
 using namespace w34;
@@ -1900,4 +1976,28 @@ extern "C" size_t warp34_paged_attention_scratch_bytes(int total_tokens, int num
                        (size_t)total_tokens * 16;  // + the per-token table
     if (total_tokens >= 2 && bal > bytes) bytes = bal;
     return bytes;
+}
+
+// op_qsa.cu:1711-1730
+extern "C" int warp34_qsa_sparse_paged_attn_f16(const warp34_exec* ex, const void* q, const void* gate,
+                                                const warp34_kv_layer_layout* kv_layout,
+                                                const int32_t* selected_phys_blocks,
+                                                const int32_t* selected_logical_blocks,
+                                                const int32_t* num_selected_blocks, const int32_t* token_seq_pos,
+                                                const uint8_t* valid_token_mask, void* out, int num_tokens,
+                                                int local_q_heads, int select_k_blocks, float sm_scale) {
+    return launch_qsa_sparse(ex, q, gate, kv_layout, selected_phys_blocks, selected_logical_blocks,
+                             num_selected_blocks, token_seq_pos, valid_token_mask, out, num_tokens, local_q_heads,
+                             select_k_blocks, sm_scale, 0);
+}
+
+// op_qsa.cu:1732-1751
+extern "C" int warp34_qsa_sparse_paged_attn_hadamard_f16(
+    const warp34_exec* ex, const void* q, const void* gate, const warp34_kv_layer_layout* kv_layout,
+    const int32_t* selected_phys_blocks, const int32_t* selected_logical_blocks,
+    const int32_t* num_selected_blocks, const int32_t* token_seq_pos, const uint8_t* valid_token_mask, void* out,
+    int num_tokens, int local_q_heads, int select_k_blocks, float sm_scale) {
+    return launch_qsa_sparse(ex, q, gate, kv_layout, selected_phys_blocks, selected_logical_blocks,
+                             num_selected_blocks, token_seq_pos, valid_token_mask, out, num_tokens, local_q_heads,
+                             select_k_blocks, sm_scale, 1);
 }

@@ -119,6 +119,13 @@ SIGNATURES = {
                    C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float]),
     "warp34_apply_attn_output_gate_f16":
         (C.c_int, [_EX, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int]),
+    # QSA sparse paged attention over selected 4-token groups (plain, and with the per-64 output transform)
+    "warp34_qsa_sparse_paged_attn_f16":
+        (C.c_int, [_EX, C.c_void_p, C.c_void_p, _LAY, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                   C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_float]),
+    "warp34_qsa_sparse_paged_attn_hadamard_f16":
+        (C.c_int, [_EX, C.c_void_p, C.c_void_p, _LAY, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                   C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_float]),
     "warp34_cuda_error_string": (C.c_char_p, [C.c_int]),
     "warp34_get_device_count": (C.c_int, [C.POINTER(C.c_int)]),
     "warp34_set_device": (C.c_int, [C.c_int]),
