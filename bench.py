@@ -43,6 +43,11 @@ WORKLOADS = {
     "tq4_norm_rope_append_8192": ("tq4", [8192], 0),
     # consumer side: out = attn_out * sigmoid(gate) over the rows of a 16 384-token prefill step
     "attn_output_gate_16384x4096": ("tq4", [64], 0),
+    # QSA sparse attention: 1, 16 or 256 query tokens, each over its own 513 selected 4-token groups (2 052 keys)
+    # of a 131 072-token sequence
+    "tq4_qsa_sparse_1x513_ctx131072": ("tq4", [131072], 0),
+    "tq4_qsa_sparse_16x513_ctx131072": ("tq4", [131072], 0),
+    "tq4_qsa_sparse_256x513_ctx131072": ("tq4", [131072], 0),
     # 16 sequences of 262 144 tokens that share the pages of a 200 000-token prefix; 4 query tokens each
     "tq4_verify_16x4_ctx262144_shared200k": ("tq4", [262144] * 16, 0),
 }
@@ -313,6 +318,71 @@ def run_gate(args, torch, lib, ffi):
     }))
 
 
+def run_qsa(args, torch, lib, ffi, layers, ctx_len, n_layers, n_tok, select_k=513):
+    """QSA sparse paged attention (gate included): every query token attends over select_k 4-token groups
+    drawn from the sequence's groups (the last group always among them, as the selector keeps the
+    newest keys).  Algorithmic bytes = the selected K and V rows of both kv heads + the gate rows."""
+    dev = "cuda:0"
+    g = torch.Generator(device=dev)
+    g.manual_seed(23)
+    q = torch.randn((n_tok, Q_HEADS, HEAD_DIM), generator=g, device=dev).to(torch.float16)
+    gate = torch.randn((n_tok, Q_HEADS, HEAD_DIM), generator=g, device=dev).to(torch.float16)
+    out = torch.zeros_like(q)
+    n_groups = ctx_len // 4
+    gpp = BLOCK // 4
+    per_layer = []
+    for L in layers:
+        logs = torch.stack([torch.cat([torch.randperm(n_groups - 1, generator=g, device=dev)[:select_k - 1],
+                                       torch.tensor([n_groups - 1], device=dev)]) for _ in range(n_tok)])
+        phys = L.block_tables[0, (logs * 4 // BLOCK)].to(torch.int64) * gpp + (logs * 4 % BLOCK) // 4
+        per_layer.append((phys.to(torch.int32).contiguous(), logs.to(torch.int32).contiguous()))
+    num_sel = torch.full((n_tok,), select_k, dtype=torch.int32, device=dev)
+    seq_pos = torch.full((n_tok,), ctx_len - 1, dtype=torch.int32, device=dev)
+    scratch_bytes = 32 << 20
+    scratch = torch.zeros(scratch_bytes, dtype=torch.uint8, device=dev)
+    ex = ffi.Warp34Exec(torch.cuda.current_stream().cuda_stream, scratch.data_ptr(), scratch_bytes, 0)
+    vp = lambda t: C.c_void_p(t.data_ptr())
+
+    def step(i):
+        L = layers[i % n_layers]
+        phys, logs = per_layer[i % n_layers]
+        rc = lib.warp34_qsa_sparse_paged_attn_f16(C.byref(ex), vp(q), vp(gate), C.byref(L.layout), vp(phys), vp(logs),
+                                                  vp(num_sel), vp(seq_pos), None, vp(out), n_tok, Q_HEADS, select_k,
+                                                  1.0 / 16.0)
+        if rc:
+            raise RuntimeError("warp34_qsa_sparse_paged_attn_f16 rc=%d" % rc)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(args.steps):
+        step(i)
+    e1.record()
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    ms = e0.elapsed_time(e1) / args.steps
+    keys = n_tok * select_k * 4
+    nbytes = keys * KV_HEADS * 2 * ROW_BYTES["tq4"] + n_tok * Q_HEADS * HEAD_DIM * 2
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "QSA sparse paged attention over TQ4 pages: us/layer + achieved HBM GB/s", "value": round(gbs, 1),
+        "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 6),
+        "us_per_layer": round(ms * 1e3, 2), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 MFMA operands (TQ4 codes -> fp16 centroids), f32 accumulate, f16 Q/gate/out", "data": "synthetic",
+        "config": {"workload": args.workload, "query_tokens": n_tok, "selected_groups_per_token": select_k,
+                   "keys_per_token": select_k * 4, "context_tokens": ctx_len, "q_heads": Q_HEADS, "kv_heads": KV_HEADS,
+                   "head_dim": HEAD_DIM, "page_tokens": BLOCK, "kv_format": "tq4+wht256", "kv_pools_cycled": n_layers,
+                   "bytes_per_step": nbytes},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "qsa_sparse_tq4_kernel + qsa_sparse_merge_kernel (whole call)",
+                     "avg_launch_us": round(ms * 1e3, 2)},
+    }))
+
+
 def run_producer(args, torch, lib, ffi, layers, n, n_layers, fmt):
     """QK RMSNorm + RoPE over packed bf16 [n, (16 + 2 * 2) * 256] rows with the K / V rows written
     into TQ4 pages: the fused entry point against the two-call sequence (operator in place, then
@@ -480,6 +550,9 @@ def run_workload(args, torch, lib, ffi, dev):
         return None
     if args.workload.startswith("attn_output_gate"):
         run_gate(args, torch, lib, ffi)
+        return None
+    if "_qsa_sparse_" in args.workload:
+        run_qsa(args, torch, lib, ffi, layers, int(ctx[0]), n_layers, int(args.workload.split("_")[3].split("x")[0]))
         return None
     if "_norm_rope_append_" in args.workload:
         run_producer(args, torch, lib, ffi, layers, int(ctx[0]), n_layers, fmt)

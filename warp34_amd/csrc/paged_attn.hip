@@ -1893,6 +1893,9 @@ static int launch_qsa_sparse(const warp34_exec* ex, const void* q, const void* g
     P.q_subgroups = P.gqa / q_group;
     P.select_k = select_k_blocks;
     P.groups_per_page = layout->block_size / 4;
+    P.gpp_shift = -1;
+    for (int k = 0; k < 30; ++k)
+        if ((1 << k) == P.groups_per_page) P.gpp_shift = k;
     P.sm_scale = sm_scale;
     P.had64 = had64;
     const int kv_subs = layout->local_kv_heads * P.q_subgroups;

@@ -8,7 +8,7 @@
 // lands in LDS in the layout the core expects.  Only the piece addresses change: they are
 // per-lane (group id -> page, row) instead of a wave-uniform run base.
 //
-//   grid  = (query tokens, kv heads x q subgroups, splits), block = 4 waves
+//   grid  = (query tokens, kv heads x q subgroups, splits), block = 8 waves
 //   split = an equal share of the token's units; every split writes an (m, l) record (l = 0
 //           without work), the merge kernel adds them up.  One split finishes in the kernel.
 //   tail  = rotate back, sigmoid gate, fp16 rounding, optional H64 / 8 over every 64-element
@@ -19,7 +19,7 @@
 
 namespace w34 {
 
-constexpr int kQsaWaves = 4;
+constexpr int kQsaWaves = 8;
 constexpr int kQsaLoopBytes = kLutBytes + kQsaWaves * kStageTq4;
 constexpr int kQsaColStride = 260;
 constexpr int kQsaRegion = 16 * kQsaColStride;  // floats per wave
@@ -42,19 +42,23 @@ struct QsaParams {
     float* part_ml;   // [rows][n_splits][4]: m, l, -, -
     int num_tokens, num_q_heads, gqa, q_group, q_subgroups, select_k, n_splits, had64;
     int groups_per_page;
+    int gpp_shift;  // log2(groups_per_page), or -1 when it is not a power of two
     float sm_scale;
 };
 
 // The end of a row: v = element 4 lane + k of the normalised sum in the rotated domain.
+__device__ __forceinline__ uint2 qsa_load_gate(const uint16_t* gate, size_t row, int lane) {
+    return gate != nullptr ? *reinterpret_cast<const uint2*>(gate + row * kHeadDim + 4 * lane) : uint2{0u, 0u};
+}
+// g: the row's gate values (qsa_load_gate, requested by the caller ahead of the sums)
 __device__ __forceinline__ void qsa_finish_row(float (&v)[4], int lane, size_t row, bool rotate,
-                                               const uint16_t* gate, bool had64, uint16_t* out) {
+                                               bool has_gate, uint2 g, bool had64, uint16_t* out) {
     if (rotate) {
         wht256_wave(v, lane);
 #pragma unroll
         for (int k = 0; k < 4; ++k) v[k] = apply_sign(v[k], 4 * lane + k);
     }
-    if (gate != nullptr) {
-        const uint2 g = *reinterpret_cast<const uint2*>(gate + row * kHeadDim + 4 * lane);
+    if (has_gate) {
         const float gv[4] = {F16::to_f32((uint16_t)(g.x & 0xFFFFu)), F16::to_f32((uint16_t)(g.x >> 16)),
                              F16::to_f32((uint16_t)(g.y & 0xFFFFu)), F16::to_f32((uint16_t)(g.y >> 16))};
 #pragma unroll
@@ -106,20 +110,25 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
     const int kv_head = fast_div(kv_sub, P.q_subgroups);
     const int q_head_base = kv_head * P.gqa + (kv_sub - kv_head * P.q_subgroups) * P.q_group;
 
+    W34_TP(0);
     // ---- this token's list ------------------------------------------------------------------------
-    const bool tok_live = P.valid_token_mask == nullptr || P.valid_token_mask[tok] != 0;
-    int n_sel = tok_live ? P.num_sel[tok] : 0;
-    if (n_sel > P.select_k) n_sel = P.select_k;
-    if (n_sel < 0) n_sel = 0;
-    n_sel = __builtin_amdgcn_readfirstlane(n_sel);
-    const int seq_pos = __builtin_amdgcn_readfirstlane(P.seq_pos[tok]);
-    const int n_units = (n_sel + 7) >> 3;
-    const int upc = fast_div(n_units + P.n_splits - 1, P.n_splits);
-    const int cu_first = split * upc;
-    int cu_end = cu_first + upc;
-    if (cu_end > n_units) cu_end = n_units;
+    // The counts and the list entries of this wave's first unit are requested together: the first
+    // unit is guessed from the list's capacity (exact when the list is full, the common case) and
+    // fetched again when the guess is wrong, so the guess changes the latency only.
     const int32_t* tok_phys = P.sel_phys + (size_t)tok * P.select_k;
     const int32_t* tok_log = P.sel_log + (size_t)tok * P.select_k;
+    const int upc_guess = fast_div(((P.select_k + 7) >> 3) + P.n_splits - 1, P.n_splits);
+    const int unit_guess = split * upc_guess + wave;
+    int spec_id = -1, spec_lg = 0;
+    {
+        const int gi = unit_guess * 8 + (lane & 7);
+        if (gi < P.select_k) {
+            spec_id = tok_phys[gi];
+            spec_lg = tok_log[gi];
+        }
+    }
+    int a_live = 1, a_sel = P.num_sel[tok], a_pos = P.seq_pos[tok];  // one vector load each, no scalar-cache trip
+    if (P.valid_token_mask != nullptr) a_live = (int)P.valid_token_mask[tok];
 
     // ---- query rows of this wave's columns (column c = q head q_head_base + c, c < q_group) ----------
     constexpr int kColsPerWave = 16 / kQsaWaves;
@@ -135,12 +144,24 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
     }
     {
         // entry e = (gain * centroid[e & 15], gain * centroid[e >> 4]) as packed fp16, 64 copies
-        const uint32_t v = pack_h2(kLutGain * centroid_of_code(tid & 15), kLutGain * centroid_of_code(tid >> 4));
+        const int e = tid >> 1;
+        const uint32_t v = pack_h2(kLutGain * centroid_of_code(e & 15), kLutGain * centroid_of_code(e >> 4));
         u4 vv = {v, v, v, v};
-        u4* dst = reinterpret_cast<u4*>(smem + tid * 256);
+        u4* dst = reinterpret_cast<u4*>(smem + e * 256 + (tid & 1) * 128);
 #pragma unroll
-        for (int k = 0; k < 16; ++k) dst[k] = vv;
+        for (int k = 0; k < 8; ++k) dst[k] = vv;
     }
+
+    W34_TP(47);
+    int n_sel = __builtin_amdgcn_readfirstlane(a_live) != 0 ? __builtin_amdgcn_readfirstlane(a_sel) : 0;
+    if (n_sel > P.select_k) n_sel = P.select_k;
+    if (n_sel < 0) n_sel = 0;
+    const int seq_pos = __builtin_amdgcn_readfirstlane(a_pos);
+    const int n_units = (n_sel + 7) >> 3;
+    const int upc = fast_div(n_units + P.n_splits - 1, P.n_splits);
+    const int cu_first = split * upc;
+    int cu_end = cu_first + upc;
+    if (cu_end > n_units) cu_end = n_units;
 
     // ---- staging machinery ------------------------------------------------------------------------
     const uint8_t* k_base = reinterpret_cast<const uint8_t*>((uintptr_t)L.k_base) + (size_t)kv_head * L.k_head_stride_bytes;
@@ -165,31 +186,40 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
         id_vec = id;
         pos_vec = id >= 0 ? 4 * lg : 0x3fffffff;
     };
-    auto piece_ptrs = [&](int id, int off16, const uint8_t*& kp, const uint8_t*& vp) {
-        // group id -> (page, row); a skipped group reads group 0 of page 0: any TQ4 bytes
-        // dequantise to finite values, and every key of such a group is masked
+    // Base of a group's four rows in the K and the V slab.  The ids come out of readlane, so this
+    // is scalar arithmetic; a skipped group reads group 0 of page 0: any TQ4 bytes dequantise to
+    // finite values, and every key of such a group is masked.
+    auto group_base = [&](int id, const uint8_t*& kp, const uint8_t*& vp) {
         const int gid = id >= 0 ? id : 0;
-        const int pg = fast_div(gid, P.groups_per_page);
+        // pages of 2^k tokens (the usual case): shift and mask
+        const int pg = P.gpp_shift >= 0 ? gid >> P.gpp_shift : gid / P.groups_per_page;
         const int row = (gid - pg * P.groups_per_page) * 4;
-        kp = k_base + (size_t)pg * L.k_page_stride_bytes + (size_t)row * L.k_token_stride_bytes + 16 * off16;
-        vp = v_base + (size_t)pg * L.v_page_stride_bytes + (size_t)row * L.v_token_stride_bytes + 16 * off16;
+        kp = k_base + (size_t)pg * L.k_page_stride_bytes + (size_t)row * L.k_token_stride_bytes;
+        vp = v_base + (size_t)pg * L.v_page_stride_bytes + (size_t)row * L.v_token_stride_bytes;
     };
     auto issue_loads = [&](int id_vec) {
+        const uint8_t *kt[2], *vt[2];
 #pragma unroll
         for (int hr = 0; hr < 2; ++hr) {  // rows 0-15 / 16-31 of the unit = groups 0-3 / 4-7
-            const uint8_t *ka, *va, *kb, *vb;
-            piece_ptrs(__shfl(id_vec, 4 * hr + pa_g, 64), pa_o, ka, va);
-            piece_ptrs(__shfl(id_vec, 4 * hr + pb_g, 64), pb_o, kb, vb);
+            const uint8_t *kg[4], *vg[4];
+#pragma unroll
+            for (int gi = 0; gi < 4; ++gi) group_base(__builtin_amdgcn_readlane(id_vec, 4 * hr + gi), kg[gi], vg[gi]);
+            // piece lane: group 0 or 1; piece 64 + lane: group 1, 2 or 3
+            const uint8_t* ka = (pa_g == 0 ? kg[0] : kg[1]) + 16 * pa_o;
+            const uint8_t* va = (pa_g == 0 ? vg[0] : vg[1]) + 16 * pa_o;
+            const uint8_t* kb = (pb_g == 1 ? kg[1] : pb_g == 2 ? kg[2] : kg[3]) + 16 * pb_o;
+            const uint8_t* vb = (pb_g == 1 ? vg[1] : pb_g == 2 ? vg[2] : vg[3]) + 16 * pb_o;
             pf[2 * hr] = *(global_cu4*)ka;
             pf[2 * hr + 1] = *(global_cu4*)kb;
             pf[4 + 2 * hr] = *(global_cu4*)va;
             pf[4 + 2 * hr + 1] = *(global_cu4*)vb;
+            kt[hr] = kg[3];
+            vt[hr] = vg[3];
         }
         {
             const int r = (lane >> 2) & 3;  // run: K rows 0-15, K rows 16-31, V rows 0-15, V rows 16-31
-            const uint8_t *kt, *vt;
-            piece_ptrs(__shfl(id_vec, 4 * (r & 1) + 3, 64), pt_o, kt, vt);
-            pf[8] = *(global_cu4*)(r < 2 ? kt : vt);
+            const uint8_t* base = r == 0 ? kt[0] : r == 1 ? kt[1] : r == 2 ? vt[0] : vt[1];
+            pf[8] = *(global_cu4*)(base + 16 * pt_o);
         }
     };
     auto commit_loads = [&]() {
@@ -203,8 +233,18 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
 
     int unit = cu_first + wave;
     int id_vec = -1, pos_vec = 0x3fffffff;
-    if (unit < cu_end) load_groups(unit, id_vec, pos_vec);
+    if (unit < cu_end) {
+        if (unit == unit_guess) {  // wave-uniform
+            const bool in_list = unit * 8 + (lane & 7) < n_sel;
+            id_vec = in_list ? spec_id : -1;
+            pos_vec = id_vec >= 0 ? 4 * spec_lg : 0x3fffffff;
+        } else {
+            load_groups(unit, id_vec, pos_vec);
+        }
+    }
+    W34_TP(41);
     issue_loads(id_vec);  // harmless for a wave without work
+    W34_TP(42);
 
     // ---- rotated, scaled fp16 queries to LDS, then the B operands of the QK MFMAs -----------------
     constexpr int kQStride = 264;
@@ -225,7 +265,9 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
         packed.y = pack_h2(qv[2] * q_scale, qv[3] * q_scale);
         *reinterpret_cast<uint2*>(qlds + col * kQStride + 4 * lane) = packed;
     }
+    W34_TP(44);
     __syncthreads();
+    W34_TP(45);
     h8 bq[9];
     {
         const int kb = 8 * (b & 1) + 4 * (b >> 1);
@@ -246,7 +288,9 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
 #pragma unroll
         for (int m = 0; m < 4; ++m) bq[5 + m] = *reinterpret_cast<const h8*>(qrow + 256 + 16 * (kb + m));
     }
+    W34_TP(46);
     __syncthreads();  // qlds is dead, the staging area may be overwritten; the table is complete
+    W34_TP(2);
 
     const uint32_t lut_lane = (uint32_t)lane << 2;
     const bool col_ok = n < P.q_group;
@@ -403,6 +447,7 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
 
     while (unit < cu_end) {
         commit_loads();
+        W34_TP(4);
         const int cur_pos_vec = pos_vec;
         const int next_unit = unit + kQsaWaves;
         if (next_unit < cu_end) {
@@ -415,10 +460,12 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
         // interior unit: all eight groups present and wholly in front of the token's position
         const bool interior = __ballot(lane < 8 && cur_pos_vec + 3 > seq_pos) == 0ull;
         process_unit(gp0, gp1, !interior);
+        W34_TP(7);
         unit = next_unit;
     }
 
     // ---- merge the waves' states through LDS (layout as in the dense kernel) -------------------------
+    W34_TP(36);
     l_run = sum_over_rows(l_run);
     float* xbuf = reinterpret_cast<float*>(smem);
     float* mlbuf = reinterpret_cast<float*>(smem + (kQsaSmem - kQsaMlBytes));
@@ -426,7 +473,9 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
         mlbuf[(wave * 16 + n) * 2 + 0] = m_run;
         mlbuf[(wave * 16 + n) * 2 + 1] = l_run;
     }
+    W34_TP(49);
     __syncthreads();  // every wave is done with the table and with its staging area
+    W34_TP(50);
     {
         float mt = kNegBig;
 #pragma unroll
@@ -449,7 +498,9 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
             mltot[n * 2 + 1] = lt;
         }
     }
+    W34_TP(51);
     __syncthreads();
+    W34_TP(37);
     const float* mltot = mlbuf + kQsaWaves * 16 * 2;
 
     int merge_slot[4];  // region slot of element 4 lane + k (inverse of tq4_pv_elem)
@@ -470,6 +521,8 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
     }
     for (int col = wave; col < P.q_group; col += kQsaWaves) {
         const size_t row = (size_t)tok * P.num_q_heads + (size_t)(q_head_base + col);
+        uint2 g = {0u, 0u};
+        if (P.n_splits == 1) g = qsa_load_gate(P.gate, row, lane);
         float v[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int w = 0; w < kQsaWaves; ++w) {
@@ -491,9 +544,10 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
             const float inv = kLutInvGain / l_col;
 #pragma unroll
             for (int k = 0; k < 4; ++k) v[k] *= inv;
-            qsa_finish_row(v, lane, row, true, P.gate, P.had64 != 0, P.out);
+            qsa_finish_row(v, lane, row, true, P.gate != nullptr, g, P.had64 != 0, P.out);
         }
     }
+    W34_TP(40);
 }
 
 // One wave per (token, q head) row: lane s holds the record of split s (n_splits <= 16).
@@ -504,6 +558,7 @@ __global__ __launch_bounds__(64) void qsa_sparse_merge_kernel(const QsaParams P)
     const float* acc = P.part_acc + row * P.n_splits * kHeadDim;
     f4 rec = {kNegBig, 0.f, 0.f, 0.f};
     if (lane < P.n_splits) rec = *reinterpret_cast<const f4*>(ml + 4 * lane);
+    const uint2 g = qsa_load_gate(P.gate, row, lane);
     f4 a[kQsaMaxSplits];
 #pragma unroll
     for (int s = 0; s < kQsaMaxSplits; ++s) {
@@ -535,7 +590,7 @@ __global__ __launch_bounds__(64) void qsa_sparse_merge_kernel(const QsaParams P)
     const float inv = kLutInvGain / l_tot;
 #pragma unroll
     for (int k = 0; k < 4; ++k) v[k] *= inv;
-    qsa_finish_row(v, lane, row, true, P.gate, P.had64 != 0, P.out);
+    qsa_finish_row(v, lane, row, true, P.gate != nullptr, g, P.had64 != 0, P.out);
 }
 
 }  // namespace w34
