@@ -120,3 +120,70 @@ def test_decode_step_replays_with_growing_sequences():
         hb = oracle.HostBatch(np.arange(R + 1), [c + 1 for c in cur], bt, context_lens_before=cur)
         ref = oracle.paged_attention(host, hb, q_in.cpu().numpy().view(np.uint16), DT_BF16, q_heads, n_threads=4)
         G.assert_close(got, DT_BF16, ref, what="replay %d vs oracle" % t)
+
+
+def test_qsa_sparse_attention_replays_with_new_selections():
+    """The QSA sparse attention inside a captured graph: the selection lists, counts and positions
+    change on the device between replays; every replay equals the eager call bit for bit."""
+    import torch
+
+    import gpu_harness as G
+    from cases import qsa_groups_of
+    from oracle import DT_F16
+    from warp34_amd import ffi
+
+    lib = G.lib()
+    seq, heads, n_tok, select_k = 900, 16, 3, 40
+    pool, bt, k, v, _, _, _ = make_case(FMT_TQ4, 64, [seq], [1], 701, DT_F16)
+    dpool = G.DevPool(pool)
+    dpool.upload()
+    L = dpool.layout()
+    all_phys, all_log, _ = qsa_groups_of(bt, [seq], 64, select_k=(seq + 3) // 4)
+    n_groups = (seq + 3) // 4
+    q = G.to_dev(oracle.fill_normal(n_tok * heads * 256, 702, DT_F16).reshape(n_tok, heads, 256))
+    gate = G.to_dev(oracle.fill_normal(n_tok * heads * 256, 703, DT_F16).reshape(n_tok, heads, 256))
+    phys = torch.zeros((n_tok, select_k), dtype=torch.int32, device=G.DEV)
+    logs = torch.zeros_like(phys)
+    num = torch.zeros(n_tok, dtype=torch.int32, device=G.DEV)
+    pos = torch.zeros(n_tok, dtype=torch.int32, device=G.DEV)
+    out = torch.zeros((n_tok, heads, 256), dtype=torch.int16, device=G.DEV)
+    scratch = torch.zeros(16 << 20, dtype=torch.uint8, device=G.DEV)
+
+    def call():
+        ex = ffi.Warp34Exec(torch.cuda.current_stream().cuda_stream, scratch.data_ptr(), scratch.numel(), 0)
+        rc = lib.warp34_qsa_sparse_paged_attn_f16(C.byref(ex), G.ptr(q), G.ptr(gate), C.byref(L), G.ptr(phys), G.ptr(logs),
+                                                  G.ptr(num), G.ptr(pos), None, G.ptr(out), n_tok, heads, select_k, 0.0625)
+        assert rc == 0
+
+    def set_state(t):
+        rng = np.random.default_rng(100 + t)
+        pick = np.stack([rng.permutation(n_groups)[:select_k] for _ in range(n_tok)])
+        phys.copy_(G.to_dev(all_phys[0, pick].astype(np.int32)))
+        logs.copy_(G.to_dev(all_log[0, pick].astype(np.int32)))
+        num.copy_(G.to_dev(np.array([select_k, select_k - 7 * t, 1 + t], dtype=np.int32)))
+        pos.copy_(G.to_dev(np.array([seq - 1, seq - 1 - 50 * t, seq - 1], dtype=np.int32)))
+        return pick
+
+    set_state(0)
+    call()  # eager warm-up: configures the kernel's dynamic LDS once
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        call()
+    for t in range(4):
+        set_state(t)
+        out.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        got = out.cpu().numpy().view(np.uint16).copy()
+        out.zero_()
+        call()
+        torch.cuda.synchronize()
+        want = out.cpu().numpy().view(np.uint16)
+        assert got.tobytes() == want.tobytes(), "replay %d differs from the eager call" % t
+        ref = oracle.qsa_sparse_paged_attn_f16(pool, q.cpu().numpy().view(np.uint16), phys.cpu().numpy(),
+                                               logs.cpu().numpy(), num.cpu().numpy(), pos.cpu().numpy(), heads,
+                                               gate=gate.cpu().numpy().view(np.uint16))
+        vmax = np.abs(oracle.bits_to_f32(v, DT_F16)).max(axis=0)
+        scale = np.broadcast_to(np.maximum(1.0, np.repeat(vmax, heads // 2, axis=0))[None], (n_tok, heads, 256))
+        G.assert_close(got, DT_F16, oracle.f16_bits_to_f32(ref), what="replay %d vs oracle" % t, scale=scale)
