@@ -953,6 +953,14 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         }
     };
     for (int j = 0; unit < cu_end; ++j) {
+        // the two waves of a SIMD take turns at the higher issue priority, unit by unit
+        if constexpr (kWaves == 8) {
+            if ((j + (wave >> 2)) & 1) {
+                __builtin_amdgcn_s_setprio(1);
+            } else {
+                __builtin_amdgcn_s_setprio(0);
+            }
+        }
         commit_loads();
 #ifdef W34_TRACE
         if (trace_it < 8) W34_TP(4 + 4 * trace_it);
@@ -967,6 +975,7 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
 #endif
         unit = next_unit;
     }
+    __builtin_amdgcn_s_setprio(0);
     W34_TP(36);
 
     // ---- combine the per-lane partial sums of l over the four k-block lanes of a column ------
