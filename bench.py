@@ -48,6 +48,7 @@ WORKLOADS = {
     "tq4_qsa_sparse_1x513_ctx131072": ("tq4", [131072], 0),
     "tq4_qsa_sparse_16x513_ctx131072": ("tq4", [131072], 0),
     "tq4_qsa_sparse_256x513_ctx131072": ("tq4", [131072], 0),
+    "fp8_qsa_sparse_16x513_ctx131072": ("fp8", [131072], 0),
     # 16 sequences of 262 144 tokens that share the pages of a 200 000-token prefix; 4 query tokens each
     "tq4_verify_16x4_ctx262144_shared200k": ("tq4", [262144] * 16, 0),
 }
@@ -318,7 +319,7 @@ def run_gate(args, torch, lib, ffi):
     }))
 
 
-def run_qsa(args, torch, lib, ffi, layers, ctx_len, n_layers, n_tok, select_k=513):
+def run_qsa(args, torch, lib, ffi, layers, ctx_len, n_layers, n_tok, fmt, select_k=513):
     """QSA sparse paged attention (gate included): every query token attends over select_k 4-token groups
     drawn from the sequence's groups (the last group always among them, as the selector keeps the
     newest keys).  Algorithmic bytes = the selected K and V rows of both kv heads + the gate rows."""
@@ -365,20 +366,23 @@ def run_qsa(args, torch, lib, ffi, layers, ctx_len, n_layers, n_tok, select_k=51
     assert torch.isfinite(out.float()).all()
     ms = e0.elapsed_time(e1) / args.steps
     keys = n_tok * select_k * 4
-    nbytes = keys * KV_HEADS * 2 * ROW_BYTES["tq4"] + n_tok * Q_HEADS * HEAD_DIM * 2
+    nbytes = keys * KV_HEADS * 2 * ROW_BYTES[fmt] + n_tok * Q_HEADS * HEAD_DIM * 2
     gbs = nbytes / (ms * 1e-3) / 1e9
     print(json.dumps({
-        "metric": "QSA sparse paged attention over TQ4 pages: us/layer + achieved HBM GB/s", "value": round(gbs, 1),
+        "metric": "QSA sparse paged attention over %s pages: us/layer + achieved HBM GB/s" % fmt.upper(), "value": round(gbs, 1),
         "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 6),
         "us_per_layer": round(ms * 1e3, 2), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16 MFMA operands (TQ4 codes -> fp16 centroids), f32 accumulate, f16 Q/gate/out", "data": "synthetic",
+        "dtype": "f16 MFMA operands (%s), f32 accumulate, f16 Q/gate/out" %
+                 ("TQ4 codes -> fp16 centroids" if fmt == "tq4" else "E4M3 codes widened, fp32 block scales"),
+        "data": "synthetic",
         "config": {"workload": args.workload, "query_tokens": n_tok, "selected_groups_per_token": select_k,
                    "keys_per_token": select_k * 4, "context_tokens": ctx_len, "q_heads": Q_HEADS, "kv_heads": KV_HEADS,
-                   "head_dim": HEAD_DIM, "page_tokens": BLOCK, "kv_format": "tq4+wht256", "kv_pools_cycled": n_layers,
-                   "bytes_per_step": nbytes},
+                   "head_dim": HEAD_DIM, "page_tokens": BLOCK, "kv_format": "tq4+wht256" if fmt == "tq4" else fmt,
+                   "kv_pools_cycled": n_layers, "bytes_per_step": nbytes},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "qsa_sparse_tq4_kernel + qsa_sparse_merge_kernel (whole call)",
+                     "kernel": ("qsa_sparse_tq4_kernel" if fmt == "tq4" else "qsa_sparse_rows_kernel") +
+                               " + qsa_sparse_merge_kernel (whole call)",
                      "avg_launch_us": round(ms * 1e3, 2)},
     }))
 
@@ -552,7 +556,7 @@ def run_workload(args, torch, lib, ffi, dev):
         run_gate(args, torch, lib, ffi)
         return None
     if "_qsa_sparse_" in args.workload:
-        run_qsa(args, torch, lib, ffi, layers, int(ctx[0]), n_layers, int(args.workload.split("_")[3].split("x")[0]))
+        run_qsa(args, torch, lib, ffi, layers, int(ctx[0]), n_layers, int(args.workload.split("_")[3].split("x")[0]), fmt)
         return None
     if "_norm_rope_append_" in args.workload:
         run_producer(args, torch, lib, ffi, layers, int(ctx[0]), n_layers, fmt)

@@ -240,8 +240,8 @@ int warp34_apply_attn_output_gate_f16(const warp34_exec* ex, const void* attn_ou
  * sigmoid(gate)) (gate may be NULL); the hadamard form then applies H64 / 8 to every 64-element
  * block of the rounded row (ops/hadamard_inline.cuh:11-50).  Rows of masked tokens and of tokens
  * without a visible key are written as zeros.  q, gate, out: fp16 [num_tokens, local_q_heads, 256].
- * Built for rotated TQ4 pages (k/v format TQ4, transform RADEMACHER_WHT256); the reference's other
- * page formats return hipErrorNotSupported.  Uses ex->scratch for split partials when it is large
+ * Page formats: rotated TQ4, FP16, FP8-E4M3 and Q8_0 (8-bit rows plain or rotated), K and V alike;
+ * other layouts return hipErrorNotSupported.  Uses ex->scratch for split partials when it is large
  * enough (num_tokens * local_q_heads * splits * 1040 bytes, splits <= 16). */
 int warp34_qsa_sparse_paged_attn_f16(const warp34_exec* ex, const void* q, const void* gate,
                                      const warp34_kv_layer_layout* kv_layout,

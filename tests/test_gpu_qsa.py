@@ -1,5 +1,5 @@
-"""GPU parity of the QSA sparse paged attention over TQ4 pages against the oracle, through the C
-ABI (warp34_qsa_sparse_paged_attn_f16 / _hadamard_f16; ops/op_qsa.cu:716-1158,1446-1571).
+"""GPU parity of the QSA sparse paged attention (TQ4, FP16, FP8-E4M3 and Q8_0 pages) against the oracle,
+through the C ABI (warp34_qsa_sparse_paged_attn_f16 / _hadamard_f16; ops/op_qsa.cu:716-1158,1446-1571).
 
 Tolerance: max-abs 2e-3 (relative to the magnitude of the values being averaged) + max-rel 1e-2
 against the oracle's fp16 output, as for the dense attention; the hadamard form is compared on the
@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 
 import oracle
-from oracle import DT_F16, FMT_FP16, FMT_TQ4, XF_IDENTITY, XF_WHT256
+from oracle import DT_F16, FMT_BF16, FMT_FP16, FMT_FP8, FMT_Q8_0, FMT_TQ4, XF_IDENTITY, XF_WHT256
 from cases import make_case, qsa_groups_of
 
 pytestmark = pytest.mark.gpu
@@ -117,6 +117,56 @@ def test_skipped_groups_short_lists_masked_tokens_and_empty_rows():
         assert np.all(got[3] == 0) and np.all(got[4] == 0) and np.all(got[5] == 0)
 
 
+ROW_FORMS = [(FMT_FP16, XF_IDENTITY), (FMT_FP8, XF_IDENTITY), (FMT_FP8, XF_WHT256), (FMT_Q8_0, XF_IDENTITY),
+             (FMT_Q8_0, XF_WHT256)]
+
+
+@pytest.mark.parametrize("fmt,xf", ROW_FORMS)
+def test_row_format_pages(fmt, xf):
+    """The FP16 / FP8 / Q8_0 branches of the operator: selected groups on permuted pages with a
+    partial tail group, skipped groups, a short list, a masked token, an empty row; gate; with and
+    without split partials; the hadamard form."""
+    rng = np.random.default_rng(fmt * 7 + xf)
+    for block_size, seq, select_k, heads, kvh in ((16, 50, 5, 2, 1), (64, 1111, 70, 16, 2)):
+        pool, bt, k, v, _, _, _ = make_case(fmt, block_size, [seq], [1], 681, DT_F16, kv_heads=kvh, xf=xf)
+        n_tok = 5
+        q = oracle.fill_normal(n_tok * heads * 256, 682, DT_F16).reshape(n_tok, heads, 256)
+        gate = oracle.fill_normal(n_tok * heads * 256, 683, DT_F16).reshape(n_tok, heads, 256)
+        sel_phys, sel_log, num_sel = _selection(bt, seq, block_size, n_tok, select_k, rng)
+        seq_pos = np.array([seq - 1, seq - 2, seq - 1, 2, seq - 1], dtype=np.int32)
+        sel_phys[0, 1] = -1
+        num_sel[2] = max(1, select_k // 3)
+        sel_log[3, :] = 9
+        mask = np.array([1, 1, 1, 1, 0], dtype=np.uint8)
+        for scratch in (0, SCRATCH):
+            got, _ = _check(pool, v, q, sel_phys, sel_log, num_sel, seq_pos, heads, gate=gate, mask=mask,
+                            scratch=scratch, what="fmt %d xf %d bs %d" % (fmt, xf, block_size))
+            assert np.all(got[3] == 0) and np.all(got[4] == 0)
+        _check(pool, v, q, sel_phys, sel_log, num_sel, seq_pos, heads, gate=gate, mask=mask, had=True,
+               what="hadamard form, fmt %d xf %d" % (fmt, xf))
+
+
+@pytest.mark.parametrize("fmt,xf", [(FMT_FP8, XF_IDENTITY), (FMT_FP16, XF_IDENTITY)])
+def test_row_format_513_groups_and_unwritten_rows(fmt, xf):
+    """513 groups of a 6 002-token sequence (split partials over 16 splits); the rows behind the
+    sequence end hold 0xFF bytes (NaN codes and scales) and must not leak through the partial
+    tail group."""
+    rng = np.random.default_rng(29)
+    seq = 6002
+    pool, bt, k, v, _, _, _ = make_case(fmt, 16, [seq], [1], 691, DT_F16, kv_heads=1)
+    kk = pool.k.reshape(-1, pool.kv_heads, pool.block_size, pool.tok)
+    vv = pool.v.reshape(-1, pool.kv_heads, pool.block_size, pool.tok)
+    last = bt[0, (seq - 1) // 16]
+    kk[last, :, seq % 16:, :] = 0xFF
+    vv[last, :, seq % 16:, :] = 0xFF
+    heads, n_tok = 6, 2
+    q = oracle.fill_normal(n_tok * heads * 256, 692, DT_F16).reshape(n_tok, heads, 256)
+    sel_phys, sel_log, num_sel = _selection(bt, seq, 16, n_tok, 513, rng)
+    seq_pos = np.full(n_tok, seq - 1, dtype=np.int32)
+    _check(pool, v, q, sel_phys, sel_log, num_sel, seq_pos, heads, what="513 groups, fmt %d" % fmt)
+    _check(pool, v, q, sel_phys, sel_log, num_sel, seq_pos, heads, scratch=0, what="513 groups single pass, fmt %d" % fmt)
+
+
 def test_all_groups_selected_matches_dense_decode_kernel():
     import gpu_harness as G
 
@@ -192,8 +242,8 @@ def test_argument_checks_and_unsupported_formats():
     # q heads not a multiple of kv heads -> invalid value (1), as the reference's launcher
     rc, _ = G.dev_qsa_sparse(dpool, np.zeros((1, 3, 256), dtype=np.uint16), one, one, [1], [3], 3)
     assert rc == 1
-    # 16-bit pages: declared unsupported (801), never computed some other way
-    p16 = oracle.HostPool(2, 2, 256, 16, FMT_FP16, XF_IDENTITY)
+    # BF16 pages (not a format of this operator): declared unsupported (801), never computed some other way
+    p16 = oracle.HostPool(2, 2, 256, 16, FMT_BF16, XF_IDENTITY)
     rc, _ = G.dev_qsa_sparse(G.DevPool(p16), q, one, one, [1], [3], 8)
     assert rc == 801
     # no tokens: success, nothing written

@@ -1481,6 +1481,7 @@ __device__ __forceinline__ TileInfo locate_tile(const AttnParams& P, int tile_z,
 #include "paged_attn_rows.h"
 #include "paged_prefill_tq4.h"
 #include "qsa_sparse_tq4.h"
+#include "qsa_sparse_rows.h"
 
 namespace w34 {
 
@@ -1871,12 +1872,26 @@ static int launch_qsa_sparse(const warp34_exec* ex, const void* q, const void* g
         return (int)hipErrorInvalidValue;
     }
     if (num_tokens == 0) return 0;
-    // built for rotated TQ4 pages; the 16-bit and 8-bit page formats of the reference's kernel are
-    // reported as unsupported, never computed some other way
-    if (!is_tq4_wht(layout)) return (int)hipErrorNotSupported;
-    if (!tq4_geometry_ok(layout, q) || (layout->block_size & 3) != 0 || (((uintptr_t)out) & 7u) != 0 ||
-        (gate != nullptr && (((uintptr_t)gate) & 7u) != 0))
+    // page formats: rotated TQ4, FP16, FP8-E4M3 and Q8_0 (plain or rotated); anything else
+    // (mixed K / V formats, BF16 pages) is reported as unsupported, never computed some other way
+    constexpr int kFormTq4 = 1000;  // not a WARP34_KV_FORMAT_* value (FP16 is 0)
+    int form = -1;  // kFormTq4, else the row format
+    if (is_tq4_wht(layout)) {
+        if (!tq4_geometry_ok(layout, q) || (((uintptr_t)out) & 7u) != 0) return (int)hipErrorNotSupported;
+        form = kFormTq4;
+    } else if (is_kv16(layout, WARP34_KV_FORMAT_FP16)) {
+        if (!kv16_geometry_ok(layout, q, out)) return (int)hipErrorNotSupported;
+        form = WARP34_KV_FORMAT_FP16;
+    } else if (is_kv8(layout, WARP34_KV_FORMAT_FP8_E4M3)) {
+        if (!kv8_geometry_ok(layout, q, out, 264)) return (int)hipErrorNotSupported;
+        form = WARP34_KV_FORMAT_FP8_E4M3;
+    } else if (is_kv8(layout, WARP34_KV_FORMAT_Q8_0)) {
+        if (!kv8_geometry_ok(layout, q, out, 272)) return (int)hipErrorNotSupported;
+        form = WARP34_KV_FORMAT_Q8_0;
+    } else {
         return (int)hipErrorNotSupported;
+    }
+    if (gate != nullptr && (((uintptr_t)gate) & 7u) != 0) return (int)hipErrorNotSupported;
     QsaParams P{};
     P.L = *layout;
     P.q = (const uint16_t*)q;
@@ -1907,8 +1922,12 @@ static int launch_qsa_sparse(const warp34_exec* ex, const void* q, const void* g
         if ((1 << k) == P.groups_per_page) P.gpp_shift = k;
     P.sm_scale = sm_scale;
     P.had64 = had64;
+    P.out_scale = form == kFormTq4 ? kLutInvGain : 1.0f;
+    P.rot_q = layout->k_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 ? 1 : 0;
+    P.rot_out = layout->v_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 ? 1 : 0;
     const int kv_subs = layout->local_kv_heads * P.q_subgroups;
-    const int max_units = (select_k_blocks + 7) / 8;
+    // work items of a token: 32-key units (TQ4) or 16-key halves (row formats), one per wave and turn
+    const int max_units = form == kFormTq4 ? (select_k_blocks + 7) / 8 : (select_k_blocks + 3) / 4;
     long long want = 256ll / ((long long)num_tokens * kv_subs);
     if (want > kQsaMaxSplits) want = kQsaMaxSplits;
     const int by_units = (max_units + kQsaWaves - 1) / kQsaWaves;
@@ -1922,11 +1941,27 @@ static int launch_qsa_sparse(const warp34_exec* ex, const void* q, const void* g
         P.part_ml = P.part_acc + rows * P.n_splits * kHeadDim;
     }
     hipStream_t stream = (hipStream_t)ex->stream;
-    int rc = ensure_dynamic_lds(qsa_sparse_tq4_kernel, kQsaSmem);
-    if (rc) return rc;
-    hipLaunchKernelGGL(qsa_sparse_tq4_kernel, dim3((unsigned)num_tokens, (unsigned)kv_subs, (unsigned)P.n_splits),
-                       dim3(kQsaWaves * 64), kQsaSmem, stream, P);
-    rc = (int)hipGetLastError();
+    const dim3 grid((unsigned)num_tokens, (unsigned)kv_subs, (unsigned)P.n_splits);
+    int rc;
+    auto launch_rows_form = [&](auto kernel) {
+        const int smem = kv16_smem_bytes(1);
+        int r = ensure_dynamic_lds(kernel, smem);
+        if (r) return r;
+        hipLaunchKernelGGL(kernel, grid, dim3(kKv16Waves * 64), smem, stream, P);
+        return (int)hipGetLastError();
+    };
+    if (form == kFormTq4) {
+        rc = ensure_dynamic_lds(qsa_sparse_tq4_kernel, kQsaSmem);
+        if (rc) return rc;
+        hipLaunchKernelGGL(qsa_sparse_tq4_kernel, grid, dim3(kQsaWaves * 64), kQsaSmem, stream, P);
+        rc = (int)hipGetLastError();
+    } else if (form == WARP34_KV_FORMAT_FP16) {
+        rc = launch_rows_form(qsa_sparse_rows_kernel<WARP34_KV_FORMAT_FP16>);
+    } else if (form == WARP34_KV_FORMAT_FP8_E4M3) {
+        rc = launch_rows_form(qsa_sparse_rows_kernel<WARP34_KV_FORMAT_FP8_E4M3>);
+    } else {
+        rc = launch_rows_form(qsa_sparse_rows_kernel<WARP34_KV_FORMAT_Q8_0>);
+    }
     if (rc) return rc;
     if (P.n_splits > 1) {
         hipLaunchKernelGGL(qsa_sparse_merge_kernel, dim3((unsigned)rows), dim3(64), 0, stream, P);

@@ -44,6 +44,9 @@ struct QsaParams {
     int groups_per_page;
     int gpp_shift;  // log2(groups_per_page), or -1 when it is not a power of two
     float sm_scale;
+    float out_scale;  // factor of the un-normalised sums (the table gain of the TQ4 form, else 1)
+    int rot_q;        // row-format form: K rows are stored rotated, rotate the query rows
+    int rot_out;      // V rows are stored rotated: rotate the finished row back
 };
 
 // The end of a row: v = element 4 lane + k of the normalised sum in the rotated domain.
@@ -587,10 +590,10 @@ __global__ __launch_bounds__(64) void qsa_sparse_merge_kernel(const QsaParams P)
         *reinterpret_cast<uint2*>(P.out + row * kHeadDim + 4 * lane) = uint2{0u, 0u};
         return;
     }
-    const float inv = kLutInvGain / l_tot;
+    const float inv = P.out_scale / l_tot;
 #pragma unroll
     for (int k = 0; k < 4; ++k) v[k] *= inv;
-    qsa_finish_row(v, lane, row, true, P.gate != nullptr, g, P.had64 != 0, P.out);
+    qsa_finish_row(v, lane, row, P.rot_out != 0, P.gate != nullptr, g, P.had64 != 0, P.out);
 }
 
 }  // namespace w34
