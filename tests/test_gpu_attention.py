@@ -362,6 +362,31 @@ def test_prefill_tile_kernel_fp8_pages(xf, dtype):
         _prefill_case(dtype, 64, [700], [333], 333, fmt=FMT_FP8, xf=xf, mask_mode=1, window=64, force=1)
 
 
+@pytest.mark.parametrize("dtype", [DT_BF16, DT_F16])
+def test_prefill_tile_kernel_16bit_pages(dtype):
+    """The tile kernel over FP16 / BF16 pages (rows copied as stored, MFMAs in the storage type; BF16
+    probabilities split into two bf16 operands), through the automatic dispatch: causal chunks on a
+    prefix, a sliding window, and 0xFF-filled rows behind the sequence ends."""
+    import gpu_harness as G
+
+    fmt = FMT_BF16 if dtype == DT_BF16 else FMT_FP16
+    _prefill_case(dtype, 64, [1500, 900], [1100, 650], 351, fmt=fmt)
+    _prefill_case(dtype, 16, [1301, 77], [1301, 40], 352, fmt=fmt, mask_mode=0, window=200)
+    seq_lens, q_lens = [1500, 901], [1100, 650]
+    pool, bt, k, v, q, aq, ctx = make_case(fmt, 64, seq_lens, q_lens, 353, dtype, q_heads=16)
+    hb = oracle.HostBatch(aq, seq_lens, bt, context_lens_before=ctx)
+    want = oracle.paged_attention(pool, hb, q, dtype, 16, n_threads=8)
+    kk = pool.k.reshape(-1, pool.kv_heads, pool.block_size, pool.tok)
+    vv = pool.v.reshape(-1, pool.kv_heads, pool.block_size, pool.tok)
+    for r, s_ in enumerate(seq_lens):
+        last = bt[r, (s_ - 1) // 64]
+        kk[last, :, s_ % 64:, :] = 0xFF
+        vv[last, :, s_ % 64:, :] = 0xFF
+    rc, got, _ = G.dev_attention(_dev_pool(pool), hb, q, dtype, 16, scratch_bytes=SCRATCH)
+    assert rc == 0
+    G.assert_close(got, dtype, want, what="poisoned tail, 16-bit tile kernel", scale=G.channel_scale(v, dtype, hb, 16))
+
+
 def test_prefill_tile_kernel_fp8_unwritten_rows_do_not_leak():
     """Rows beyond the sequence hold 0xFF bytes (NaN codes, NaN scales) in the last page of each
     request: the tile kernel must keep them out of the P V product."""

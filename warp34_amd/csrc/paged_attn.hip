@@ -1839,6 +1839,12 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
     // point, BF16 pages with the bf16 one, as in the reference)
     if (is_kv16(layout, TQ::kStorageFormat)) {
         if (!kv16_geometry_ok(layout, q, out)) return (int)hipErrorNotSupported;
+        // many query rows per request: the tile kernel (rows copied as stored).  The test selector
+        // keeps its meaning of "one pass of the row kernel" for these pages.
+        const bool many_rows = batch->max_q_len >= 32 &&
+                               (long long)batch->total_tokens * num_q_heads >= 128ll * kPfRows;
+        if (!force_single && many_rows && prefill_tq4_applicable(layout, batch, num_q_heads))
+            return launch_prefill_tq4<TQ, TQ::kStorageFormat>(ex, layout, batch, q, out, num_q_heads);
         return launch_rows<TQ, TQ::kStorageFormat>(ex, layout, batch, q, out, num_q_heads, force_single);
     }
     // 8-bit pages (the tail layers of the default TQ4 policy, cache.rs:87-109)

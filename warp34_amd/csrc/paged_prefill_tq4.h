@@ -1,8 +1,10 @@
-// Chunked-prefill attention over TQ4 or FP8-E4M3 pages for gfx950: many query rows per workgroup,
+// Chunked-prefill attention over TQ4, FP8-E4M3, FP16 or BF16 pages for gfx950: many query rows per workgroup,
 // every K/V unit dequantised ONCE per workgroup and shared by all waves through LDS.  (FP8 rows
 // have the same shape as TQ4 rows -- two scale blocks of 128 elements -- so only the loader and
 // the dequantiser differ: codes are widened with v_cvt_scalef32_pk_f16_fp8 instead of the table,
-// there is no table in LDS and, for un-rotated layers, no rotation.)
+// there is no table in LDS and, for un-rotated layers, no rotation.  16-bit rows are copied into
+// the same two tiles as stored and multiplied in their own type; BF16 probabilities are split
+// into a high and a low bf16 part.)
 // Replaces paged_attention_prefill_mma_f16_kernel + launch_prefill
 // (op_paged_attn.cu:594-1128,1220-1259).  Included by paged_attn.hip.
 //
@@ -34,10 +36,11 @@ constexpr int kPfDeqBytes = kPfKBytes + kPfVBytes + kPfScaleBytes;
 template <int KVF>
 struct PfLds {
     static constexpr bool kFp8 = KVF == WARP34_KV_FORMAT_FP8_E4M3;
-    static constexpr int kRowBytes = kFp8 ? 264 : kTq4RowBytes;
-    static constexpr int kRun = 16 * kRowBytes;                // 16 rows: 2112 B / 4224 B
+    static constexpr bool k16 = KVF == WARP34_KV_FORMAT_FP16 || KVF == WARP34_KV_FORMAT_BF16;
+    static constexpr int kRowBytes = k16 ? 512 : kFp8 ? 264 : kTq4RowBytes;
+    static constexpr int kRun = 16 * kRowBytes;                // 16 rows: 2112 B / 4224 B / 8192 B
     static constexpr int kRaw = 4 * kRun;                      // K rows 0-31, V rows 0-31
-    static constexpr int kDeqBase = kFp8 ? 0 : kLutBytes;
+    static constexpr int kDeqBase = (kFp8 || k16) ? 0 : kLutBytes;
     static constexpr int kRawBase = kDeqBase + 2 * kPfDeqBytes;
     static constexpr int kLoop = kRawBase + 2 * kRaw + 256;
     static constexpr int kEpilogue = kPfWaves * 16 * 260 * 4;  // the output transpose regions
@@ -49,10 +52,23 @@ static_assert(kPfWaves * 16 * 264 * 2 <= 2 * kPfDeqBytes, "query staging must fi
 
 typedef __attribute__((address_space(3))) uint32_t lds_u32;
 
+// 16x16x32 MFMA on fp16 or bf16 operands given as raw bits
+template <bool IS_BF16>
+__device__ __forceinline__ f4 pf_mfma32(h8 a, h8 b, f4 c) {
+    if constexpr (IS_BF16) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8, a), __builtin_bit_cast(bf8, b), c, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+}
+
 template <typename TQ, int KVF>
 __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(const AttnParams P) {
     using M = PfLds<KVF>;
     constexpr bool FP8 = M::kFp8;
+    constexpr bool K16 = M::k16;  // 16-bit rows, read as stored: the MFMAs run in the storage type
+    constexpr bool IS_BF16 = KVF == WARP34_KV_FORMAT_BF16;
+    static_assert(!K16 || KVF == TQ::kStorageFormat, "16-bit pages are read in the query type");
     constexpr int kPfDeqBase = M::kDeqBase, kPfRawBase = M::kRawBase, kPfRawBytes = M::kRaw;
     constexpr int kRowB = M::kRowBytes, kRunB = M::kRun;
     extern __shared__ __align__(16) uint8_t smem[];
@@ -86,7 +102,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     if (tile_tokens > B.total_tokens - tok0) tile_tokens = B.total_tokens - tok0;
 
     // ---- the pair table (64 lane replicas, as in the decode kernel) ----
-    if constexpr (!FP8) {
+    if constexpr (!FP8 && !K16) {
         const int e = tid >> 1;
         const uint32_t v = pack_h2(kLutGain * centroid_of_code(e & 15), kLutGain * centroid_of_code(e >> 4));
         u4 vv = {v, v, v, v};
@@ -129,9 +145,9 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     // ---- rotated, scaled queries of this wave's 16 columns -> LDS -> MFMA B operands ----
     constexpr int kQStride = 264;
     _Float16* qbuf = reinterpret_cast<_Float16*>(smem + kPfDeqBase) + wave * 16 * kQStride;
-    const float q_scale = B.sm_scale * kLog2e * (FP8 ? 1.0f : kLutInvGain);
-    const bool rot_q = !FP8 || P.rot_q != 0;
-    const bool rot_out = !FP8 || P.rot_out != 0;
+    const float q_scale = B.sm_scale * kLog2e * ((FP8 || K16) ? 1.0f : kLutInvGain);
+    const bool rot_q = !K16 && (!FP8 || P.rot_q != 0);
+    const bool rot_out = !K16 && (!FP8 || P.rot_out != 0);
     {
         uint2 q_raw[16];
 #pragma unroll
@@ -157,8 +173,12 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             }
             uint2 packed = {0u, 0u};  // dead columns: zero query
             if ((ok_mask >> c) & 1u) {
-                packed.x = pack_h2(v[0] * q_scale, v[1] * q_scale);
-                packed.y = pack_h2(v[2] * q_scale, v[3] * q_scale);
+                if constexpr (K16) {
+                    packed = q_raw[c];  // as given: the scores are scaled after the MFMAs
+                } else {
+                    packed.x = pack_h2(v[0] * q_scale, v[1] * q_scale);
+                    packed.y = pack_h2(v[2] * q_scale, v[3] * q_scale);
+                }
             }
             *reinterpret_cast<uint2*>(qbuf + c * kQStride + 4 * lane) = packed;
         }
@@ -186,15 +206,16 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     const int32_t* req_blocks = B.block_tables + (size_t)req * B.max_blocks_per_req;
     const int ld_run = wave >> 1;
     const bool ld_is_v = ld_run >= 2;
-    const bool ld_tail = FP8 || (wave & 1) == 0;  // wave-uniform
+    const bool ld_tail = !K16 && (FP8 || (wave & 1) == 0);  // wave-uniform
     const uint8_t* ld_base = ld_is_v ? v_base : k_base;
     const uint64_t ld_page_stride = ld_is_v ? L.v_page_stride_bytes : L.k_page_stride_bytes;
     const uint64_t ld_tok_stride = ld_is_v ? L.v_token_stride_bytes : L.k_token_stride_bytes;
-    const uint32_t ld_lane_off = (uint32_t)((wave & 1) * (FP8 ? 2112 : 1024) + 16 * lane);
+    // 16-bit rows: a run is 8192 B = 512 pieces; each wave of the pair loads 256 (four per lane), no tail
+    const uint32_t ld_lane_off = (uint32_t)((wave & 1) * (K16 ? 4096 : FP8 ? 2112 : 1024) + 16 * lane);
     const uint32_t ld_tail_off = (uint32_t)((FP8 ? (wave & 1) * 2112 : 0) + 2048 + 16 * (lane & 3));
     const uint32_t ld_commit0 = (uint32_t)(ld_run * kRunB) + ld_lane_off;
     const uint32_t ld_commit1 = (uint32_t)(ld_run * kRunB) + ld_tail_off;
-    u4 pf[FP8 ? 3 : 2];
+    u4 pf[K16 ? 4 : FP8 ? 3 : 2];
     // page id of unit k (relative to u_first) for this wave's run; -1 = nothing to fetch.
     // Only groups that overlap the visible key range are fetched: block-table entries beyond
     // the request's pages are unspecified.
@@ -214,14 +235,24 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         if (pg >= 0) off = (size_t)pg * ld_page_stride + (size_t)in_page * ld_tok_stride;
         const uint8_t* src = ld_base + off;
         pf[0] = *(global_cu4*)(src + ld_lane_off);
-        if (ld_tail) pf[1] = *(global_cu4*)(src + ld_tail_off);
-        if constexpr (FP8) pf[2] = *(global_cu4*)(src + ld_lane_off + 1024);
+        if constexpr (K16) {
+#pragma unroll
+            for (int i = 1; i < 4; ++i) pf[i] = *(global_cu4*)(src + ld_lane_off + 1024 * i);
+        } else {
+            if (ld_tail) pf[1] = *(global_cu4*)(src + ld_tail_off);
+            if constexpr (FP8) pf[2] = *(global_cu4*)(src + ld_lane_off + 1024);
+        }
     };
     auto commit_loads = [&](int buf) {
         uint8_t* raw = smem + kPfRawBase + buf * kPfRawBytes;
         *reinterpret_cast<u4*>(raw + ld_commit0) = pf[0];
-        if (ld_tail && lane < 4) *reinterpret_cast<u4*>(raw + ld_commit1) = pf[1];
-        if constexpr (FP8) *reinterpret_cast<u4*>(raw + ld_commit0 + 1024) = pf[2];
+        if constexpr (K16) {
+#pragma unroll
+            for (int i = 1; i < 4; ++i) *reinterpret_cast<u4*>(raw + ld_commit0 + 1024 * i) = pf[i];
+        } else {
+            if (ld_tail && lane < 4) *reinterpret_cast<u4*>(raw + ld_commit1) = pf[1];
+            if constexpr (FP8) *reinterpret_cast<u4*>(raw + ld_commit0 + 1024) = pf[2];
+        }
     };
 
     // ---- dequantiser ----
@@ -423,6 +454,38 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         if (tid < 64) *reinterpret_cast<float*>(deq + kPfKBytes + kPfVBytes + 4 * tid) = scale;
     };
 
+    // 16-bit rows: nothing to dequantise.  K: thread (row r = tid / 16, segment g = tid % 16)
+    // copies elements 16 g .. 16 g + 15 into the padded row-major tile.  V: thread (token pair
+    // p = tid % 16, group j = tid / 16) stores dims 8 j .. 8 j + 7 of tokens 2p, 2p + 1 as (token 2p,
+    // token 2p + 1) pairs into the transposed tile.  Value rows outside the visible key range
+    // become zeros (unwritten pool memory may hold NaN patterns).
+    auto dequant_unit_16 = [&](int rawbuf, int deqbuf, int t0) {
+        const uint8_t* raw = smem + kPfRawBase + rawbuf * kPfRawBytes;
+        uint8_t* deq = smem + kPfDeqBase + deqbuf * kPfDeqBytes;
+        const int kr = tid >> 4, kg = tid & 15;
+        const int vp = tid & 15, vj = tid >> 4;
+        const u4 k_lo = *reinterpret_cast<const u4*>(raw + kr * kRowB + 32 * kg);
+        const u4 k_hi = *reinterpret_cast<const u4*>(raw + kr * kRowB + 32 * kg + 16);
+        u4 ha = *reinterpret_cast<const u4*>(raw + kPfRawBytes / 2 + (2 * vp) * kRowB + 16 * vj);
+        u4 hb = *reinterpret_cast<const u4*>(raw + kPfRawBytes / 2 + (2 * vp + 1) * kRowB + 16 * vj);
+        {
+            const int pa = t0 + 2 * vp;
+            const bool a_ok = pa >= lo_all && pa <= hi_all, b_ok = pa + 1 >= lo_all && pa + 1 <= hi_all;
+            if (!a_ok) ha = u4{0u, 0u, 0u, 0u};
+            if (!b_ok) hb = u4{0u, 0u, 0u, 0u};
+        }
+        *reinterpret_cast<u4*>(deq + kr * kPfKStride + 32 * kg) = k_lo;
+        *reinterpret_cast<u4*>(deq + kr * kPfKStride + 32 * kg + 16) = k_hi;
+        const int bp = (vp >> 1) & 3, sl = vp >> 3;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int d = 8 * vj + e;
+            const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
+            const uint32_t pair = __builtin_amdgcn_perm(hb[e >> 1], ha[e >> 1], sel);
+            *reinterpret_cast<uint32_t*>(deq + kPfKBytes + d * 64 + 16 * (bp ^ ((d >> 1) & 3)) + 8 * sl + 4 * (vp & 1)) = pair;
+        }
+    };
+
     auto compute_unit = [&](int deqbuf, int t0, const bool MASKED) {
         const uint8_t* kb = smem + kPfDeqBase + deqbuf * kPfDeqBytes;
         const uint8_t* vb = kb + kPfKBytes;
@@ -436,16 +499,20 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
 #pragma unroll
                 for (int m = 0; m < 4; ++m)
                     a[h][m] = *reinterpret_cast<const h8*>(kb + (16 * s + n) * kPfKStride + 2 * (128 * h + 32 * m + 8 * b));
-            const f4 kd0 = *reinterpret_cast<const f4*>(sc + 16 * s + 4 * b);
-            const f4 kd1 = *reinterpret_cast<const f4*>(sc + 32 + 16 * s + 4 * b);
             f4 s_acc[2] = {f4{0.f, 0.f, 0.f, 0.f}, f4{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
             for (int m = 0; m < 4; ++m)
 #pragma unroll
-                for (int h = 0; h < 2; ++h)
-                    s_acc[h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[h][m], bq[h][m], s_acc[h], 0, 0, 0);
+                for (int h = 0; h < 2; ++h) s_acc[h] = pf_mfma32<IS_BF16>(a[h][m], bq[h][m], s_acc[h]);
+            if constexpr (K16) {  // rows as stored: no scales, the softmax factor comes in here
 #pragma unroll
-            for (int i = 0; i < 4; ++i) score[4 * s + i] = kd0[i] * s_acc[0][i] + kd1[i] * s_acc[1][i];
+                for (int i = 0; i < 4; ++i) score[4 * s + i] = (s_acc[0][i] + s_acc[1][i]) * q_scale;
+            } else {
+                const f4 kd0 = *reinterpret_cast<const f4*>(sc + 16 * s + 4 * b);
+                const f4 kd1 = *reinterpret_cast<const f4*>(sc + 32 + 16 * s + 4 * b);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) score[4 * s + i] = kd0[i] * s_acc[0][i] + kd1[i] * s_acc[1][i];
+            }
         }
         // (the MASKED tests sit outside the unrolled loops: one wave-uniform branch per block)
         if (MASKED) {
@@ -480,7 +547,19 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
                 for (int j = 0; j < 8; ++j) o_acc[h][j] *= alpha;
         }
         u4 pb[2];
-        if constexpr (FP8) {  // the value tile already carries its scales
+        u4 pb_lo = {0u, 0u, 0u, 0u};
+        if constexpr (IS_BF16) {
+            // bf16 keeps 8 bits of a probability: the rest goes into a second operand (two MFMAs)
+            uint32_t hi[8], lo[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                hi[t] = BF16::from_f32(p[t]);
+                lo[t] = BF16::from_f32(p[t] - BF16::to_f32((uint16_t)hi[t]));
+            }
+            pb[0] = u4{hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16), hi[4] | (hi[5] << 16), hi[6] | (hi[7] << 16)};
+            pb[1] = pb[0];
+            pb_lo = u4{lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16), lo[4] | (lo[5] << 16), lo[6] | (lo[7] << 16)};
+        } else if constexpr (FP8 || K16) {  // the value tile already carries its scales
             pb[0] = u4{pack_h2(p[0], p[1]), pack_h2(p[2], p[3]), pack_h2(p[4], p[5]), pack_h2(p[6], p[7])};
             pb[1] = pb[0];
         } else {
@@ -508,8 +587,10 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
                 a[j] = *reinterpret_cast<const h8*>(vb + d * 64 + 16 * (b ^ ((d >> 1) & 3)));
             }
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
-                o_acc[h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j], __builtin_bit_cast(h8, pb[h]), o_acc[h][j], 0, 0, 0);
+            for (int j = 0; j < 8; ++j) {
+                o_acc[h][j] = pf_mfma32<IS_BF16>(a[j], __builtin_bit_cast(h8, pb[h]), o_acc[h][j]);
+                if constexpr (IS_BF16) o_acc[h][j] = pf_mfma32<true>(a[j], __builtin_bit_cast(h8, pb_lo), o_acc[h][j]);
+            }
         }
     };
 
@@ -534,7 +615,9 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         if (it >= 8 && it < 16) W34_TP(4 + 5 * (it - 8) + 1);
 #endif
         if (it + 1 >= 0 && it + 1 < n_units) {
-            if constexpr (FP8) {
+            if constexpr (K16) {
+                dequant_unit_16((it + 1) & 1, (it + 1) & 1, (u_first + it + 1) * kUnit);
+            } else if constexpr (FP8) {
                 dequant_unit_fp8((it + 1) & 1, (it + 1) & 1, (u_first + it + 1) * kUnit);
             } else {
                 dequant_unit((it + 1) & 1, (it + 1) & 1);
@@ -560,7 +643,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     // ---- epilogue: normalise, transpose through LDS, rotate back, store ----
     l_run = sum_over_rows(l_run);
     float* reg = reinterpret_cast<float*>(smem) + wave * 16 * 260;
-    const float inv = l_run > 0.f ? (FP8 ? 1.0f : kLutInvGain) / l_run : 0.f;
+    const float inv = l_run > 0.f ? ((FP8 || K16) ? 1.0f : kLutInvGain) / l_run : 0.f;
 #pragma unroll
     for (int h = 0; h < 2; ++h)
 #pragma unroll
