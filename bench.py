@@ -40,6 +40,7 @@ WORKLOADS = {
     "tq4_prefill_8x2048_ctx16384": ("tq4", [18432] * 8, 0),
     "fp8_prefill_8x2048_ctx16384": ("fp8", [18432] * 8, 0),
     "bf16_prefill_8x2048_ctx16384": ("bf16", [18432] * 8, 0),
+    "q8_0_prefill_8x2048_ctx16384": ("q8_0", [18432] * 8, 0),
     # producer side: QK RMSNorm + RoPE fused with the TQ4 append of an 8 192-token chunk
     "tq4_norm_rope_append_8192": ("tq4", [8192], 0),
     # consumer side: out = attn_out * sigmoid(gate) over the rows of a 16 384-token prefill step
@@ -262,7 +263,8 @@ def run_prefill(args, torch, lib, ffi, layers, ctx, n_layers, pool_pages, fmt):
         "ms_per_step": round(ms_step, 4), "ms_attention_only": round(ms_attn, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 MFMA operands (%s), f32 accumulate, bf16 Q/out"
-                 % {"tq4": "TQ4 codes -> fp16 centroids", "fp8": "E4M3 codes widened"}.get(fmt, "rows as stored"),
+                 % {"tq4": "TQ4 codes -> fp16 centroids", "fp8": "E4M3 codes widened",
+                    "q8_0": "fp16(d * int8 code)"}.get(fmt, "rows as stored"),
         "data": "synthetic",
         "config": {"workload": args.workload, "requests": R, "chunk_tokens": n, "prefix_tokens": int(ctx[0]) - n,
                    "q_heads": Q_HEADS, "kv_heads": KV_HEADS, "head_dim": HEAD_DIM, "page_tokens": BLOCK,

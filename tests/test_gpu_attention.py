@@ -351,15 +351,17 @@ def test_prefill_tile_kernel_windows(mask_mode, window):
     _prefill_case(DT_F16, 16, [400, 130], [90, 130], 221, force=0, mask_mode=mask_mode, window=window)
 
 
+@pytest.mark.parametrize("fmt", [FMT_FP8, FMT_Q8_0])
 @pytest.mark.parametrize("xf", [XF_IDENTITY, XF_WHT256])
 @pytest.mark.parametrize("dtype", [DT_BF16, DT_F16])
-def test_prefill_tile_kernel_fp8_pages(xf, dtype):
-    """The tile kernel over FP8-E4M3 pages (same row shape as TQ4: two scale blocks of 128), plain
-    and rotated, through the automatic dispatch and the test selector."""
-    _prefill_case(dtype, 64, [1500, 900], [1100, 650], 331, fmt=FMT_FP8, xf=xf)
+def test_prefill_tile_kernel_8bit_pages(xf, dtype, fmt):
+    """The tile kernel over FP8-E4M3 pages (same row shape as TQ4: two scale blocks of 128) and
+    Q8_0 pages (four blocks of 64, dequantised into both tiles), plain and rotated, through the
+    automatic dispatch and the test selector."""
+    _prefill_case(dtype, 64, [1500, 900], [1100, 650], 331, fmt=fmt, xf=xf)
     if dtype == DT_F16:  # the test selector is an f16 entry point
-        _prefill_case(dtype, 16, [300, 77], [130, 40], 332, fmt=FMT_FP8, xf=xf, force=1)
-        _prefill_case(dtype, 64, [700], [333], 333, fmt=FMT_FP8, xf=xf, mask_mode=1, window=64, force=1)
+        _prefill_case(dtype, 16, [300, 77], [130, 40], 332, fmt=fmt, xf=xf, force=1)
+        _prefill_case(dtype, 64, [700], [333], 333, fmt=fmt, xf=xf, mask_mode=1, window=64, force=1)
 
 
 @pytest.mark.parametrize("dtype", [DT_BF16, DT_F16])
@@ -387,13 +389,14 @@ def test_prefill_tile_kernel_16bit_pages(dtype):
     G.assert_close(got, dtype, want, what="poisoned tail, 16-bit tile kernel", scale=G.channel_scale(v, dtype, hb, 16))
 
 
-def test_prefill_tile_kernel_fp8_unwritten_rows_do_not_leak():
+@pytest.mark.parametrize("fmt", [FMT_FP8, FMT_Q8_0])
+def test_prefill_tile_kernel_8bit_unwritten_rows_do_not_leak(fmt):
     """Rows beyond the sequence hold 0xFF bytes (NaN codes, NaN scales) in the last page of each
     request: the tile kernel must keep them out of the P V product."""
     import gpu_harness as G
 
     seq_lens, q_lens = [1500, 901], [1100, 650]
-    pool, bt, k, v, q, aq, ctx = make_case(FMT_FP8, 64, seq_lens, q_lens, 341, DT_F16, q_heads=16)
+    pool, bt, k, v, q, aq, ctx = make_case(fmt, 64, seq_lens, q_lens, 341, DT_F16, q_heads=16)
     hb = oracle.HostBatch(aq, seq_lens, bt, context_lens_before=ctx)
     want = oracle.paged_attention(pool, hb, q, DT_F16, 16, n_threads=8)
     kk = pool.k.reshape(-1, pool.kv_heads, pool.block_size, pool.tok)

@@ -1859,6 +1859,10 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
     }
     if (is_kv8(layout, WARP34_KV_FORMAT_Q8_0)) {
         if (!kv8_geometry_ok(layout, q, out, 272)) return (int)hipErrorNotSupported;
+        const bool many_rows = batch->max_q_len >= 32 &&
+                               (long long)batch->total_tokens * num_q_heads >= 128ll * kPfRows;
+        if ((force_single || many_rows) && prefill_tq4_applicable(layout, batch, num_q_heads))
+            return launch_prefill_tq4<TQ, WARP34_KV_FORMAT_Q8_0>(ex, layout, batch, q, out, num_q_heads);
         return launch_rows<TQ, WARP34_KV_FORMAT_Q8_0>(ex, layout, batch, q, out, num_q_heads, force_single);
     }
     return (int)hipErrorNotSupported;

@@ -1,4 +1,4 @@
-// Chunked-prefill attention over TQ4, FP8-E4M3, FP16 or BF16 pages for gfx950: many query rows per workgroup,
+// Chunked-prefill attention over TQ4, FP8-E4M3, Q8_0, FP16 or BF16 pages for gfx950: many query rows per workgroup,
 // every K/V unit dequantised ONCE per workgroup and shared by all waves through LDS.  (FP8 rows
 // have the same shape as TQ4 rows -- two scale blocks of 128 elements -- so only the loader and
 // the dequantiser differ: codes are widened with v_cvt_scalef32_pk_f16_fp8 instead of the table,
@@ -37,10 +37,11 @@ template <int KVF>
 struct PfLds {
     static constexpr bool kFp8 = KVF == WARP34_KV_FORMAT_FP8_E4M3;
     static constexpr bool k16 = KVF == WARP34_KV_FORMAT_FP16 || KVF == WARP34_KV_FORMAT_BF16;
-    static constexpr int kRowBytes = k16 ? 512 : kFp8 ? 264 : kTq4RowBytes;
-    static constexpr int kRun = 16 * kRowBytes;                // 16 rows: 2112 B / 4224 B / 8192 B
+    static constexpr bool kQ8 = KVF == WARP34_KV_FORMAT_Q8_0;
+    static constexpr int kRowBytes = k16 ? 512 : kFp8 ? 264 : kQ8 ? 272 : kTq4RowBytes;
+    static constexpr int kRun = 16 * kRowBytes;                // 16 rows: 2112 B / 4224 B / 4352 B / 8192 B
     static constexpr int kRaw = 4 * kRun;                      // K rows 0-31, V rows 0-31
-    static constexpr int kDeqBase = (kFp8 || k16) ? 0 : kLutBytes;
+    static constexpr int kDeqBase = (kFp8 || k16 || kQ8) ? 0 : kLutBytes;
     static constexpr int kRawBase = kDeqBase + 2 * kPfDeqBytes;
     static constexpr int kLoop = kRawBase + 2 * kRaw + 256;
     static constexpr int kEpilogue = kPfWaves * 16 * 260 * 4;  // the output transpose regions
@@ -67,6 +68,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     using M = PfLds<KVF>;
     constexpr bool FP8 = M::kFp8;
     constexpr bool K16 = M::k16;  // 16-bit rows, read as stored: the MFMAs run in the storage type
+    constexpr bool Q8 = M::kQ8;   // Q8_0 rows: both tiles hold fp16(d * code), no scales afterwards
+    constexpr bool TQ4F = !FP8 && !K16 && !Q8;
     constexpr bool IS_BF16 = KVF == WARP34_KV_FORMAT_BF16;
     static_assert(!K16 || KVF == TQ::kStorageFormat, "16-bit pages are read in the query type");
     constexpr int kPfDeqBase = M::kDeqBase, kPfRawBase = M::kRawBase, kPfRawBytes = M::kRaw;
@@ -102,7 +105,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     if (tile_tokens > B.total_tokens - tok0) tile_tokens = B.total_tokens - tok0;
 
     // ---- the pair table (64 lane replicas, as in the decode kernel) ----
-    if constexpr (!FP8 && !K16) {
+    if constexpr (TQ4F) {
         const int e = tid >> 1;
         const uint32_t v = pack_h2(kLutGain * centroid_of_code(e & 15), kLutGain * centroid_of_code(e >> 4));
         u4 vv = {v, v, v, v};
@@ -145,9 +148,9 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     // ---- rotated, scaled queries of this wave's 16 columns -> LDS -> MFMA B operands ----
     constexpr int kQStride = 264;
     _Float16* qbuf = reinterpret_cast<_Float16*>(smem + kPfDeqBase) + wave * 16 * kQStride;
-    const float q_scale = B.sm_scale * kLog2e * ((FP8 || K16) ? 1.0f : kLutInvGain);
-    const bool rot_q = !K16 && (!FP8 || P.rot_q != 0);
-    const bool rot_out = !K16 && (!FP8 || P.rot_out != 0);
+    const float q_scale = B.sm_scale * kLog2e * (TQ4F ? kLutInvGain : 1.0f);
+    const bool rot_q = !K16 && (TQ4F || P.rot_q != 0);
+    const bool rot_out = !K16 && (TQ4F || P.rot_out != 0);
     {
         uint2 q_raw[16];
 #pragma unroll
@@ -206,16 +209,19 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     const int32_t* req_blocks = B.block_tables + (size_t)req * B.max_blocks_per_req;
     const int ld_run = wave >> 1;
     const bool ld_is_v = ld_run >= 2;
-    const bool ld_tail = !K16 && (FP8 || (wave & 1) == 0);  // wave-uniform
+    // Q8_0: a run is 4352 B = 272 pieces; each wave of the pair loads 136 (two per lane and an eight-lane tail)
+    const bool ld_tail = !K16 && (FP8 || Q8 || (wave & 1) == 0);  // wave-uniform
+    constexpr int kTailLanes = Q8 ? 8 : 4;
     const uint8_t* ld_base = ld_is_v ? v_base : k_base;
     const uint64_t ld_page_stride = ld_is_v ? L.v_page_stride_bytes : L.k_page_stride_bytes;
     const uint64_t ld_tok_stride = ld_is_v ? L.v_token_stride_bytes : L.k_token_stride_bytes;
     // 16-bit rows: a run is 8192 B = 512 pieces; each wave of the pair loads 256 (four per lane), no tail
-    const uint32_t ld_lane_off = (uint32_t)((wave & 1) * (K16 ? 4096 : FP8 ? 2112 : 1024) + 16 * lane);
-    const uint32_t ld_tail_off = (uint32_t)((FP8 ? (wave & 1) * 2112 : 0) + 2048 + 16 * (lane & 3));
+    const uint32_t ld_lane_off = (uint32_t)((wave & 1) * (K16 ? 4096 : FP8 ? 2112 : Q8 ? 2176 : 1024) + 16 * lane);
+    const uint32_t ld_tail_off = (uint32_t)((FP8 ? (wave & 1) * 2112 : Q8 ? (wave & 1) * 2176 : 0) + 2048 +
+                                            16 * (lane & (kTailLanes - 1)));
     const uint32_t ld_commit0 = (uint32_t)(ld_run * kRunB) + ld_lane_off;
     const uint32_t ld_commit1 = (uint32_t)(ld_run * kRunB) + ld_tail_off;
-    u4 pf[K16 ? 4 : FP8 ? 3 : 2];
+    u4 pf[K16 ? 4 : (FP8 || Q8) ? 3 : 2];
     // page id of unit k (relative to u_first) for this wave's run; -1 = nothing to fetch.
     // Only groups that overlap the visible key range are fetched: block-table entries beyond
     // the request's pages are unspecified.
@@ -240,7 +246,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             for (int i = 1; i < 4; ++i) pf[i] = *(global_cu4*)(src + ld_lane_off + 1024 * i);
         } else {
             if (ld_tail) pf[1] = *(global_cu4*)(src + ld_tail_off);
-            if constexpr (FP8) pf[2] = *(global_cu4*)(src + ld_lane_off + 1024);
+            if constexpr (FP8 || Q8) pf[2] = *(global_cu4*)(src + ld_lane_off + 1024);
         }
     };
     auto commit_loads = [&](int buf) {
@@ -250,8 +256,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
 #pragma unroll
             for (int i = 1; i < 4; ++i) *reinterpret_cast<u4*>(raw + ld_commit0 + 1024 * i) = pf[i];
         } else {
-            if (ld_tail && lane < 4) *reinterpret_cast<u4*>(raw + ld_commit1) = pf[1];
-            if constexpr (FP8) *reinterpret_cast<u4*>(raw + ld_commit0 + 1024) = pf[2];
+            if (ld_tail && lane < kTailLanes) *reinterpret_cast<u4*>(raw + ld_commit1) = pf[1];
+            if constexpr (FP8 || Q8) *reinterpret_cast<u4*>(raw + ld_commit0 + 1024) = pf[2];
         }
     };
 
@@ -454,6 +460,69 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         if (tid < 64) *reinterpret_cast<float*>(deq + kPfKBytes + kPfVBytes + 4 * tid) = scale;
     };
 
+    // Q8_0 rows: four blocks of {fp32 d, 64 int8}.  Both tiles receive fp16(d * code), every element
+    // rounded on its own from fp32 (what the reference's MMA kernels stage, op_paged_attn.cu:59-71);
+    // thread roles as for FP8 rows.
+    auto dequant_unit_q8 = [&](int rawbuf, int deqbuf, int t0) {
+        const uint8_t* raw = smem + kPfRawBase + rawbuf * kPfRawBytes;
+        uint8_t* deq = smem + kPfDeqBase + deqbuf * kPfDeqBytes;
+        const int kr = tid >> 4, kg = tid & 15;
+        const int vp = tid & 15, vj = tid >> 4;
+        // ---- phase 1: raw codes and scales ----
+        const uint8_t* krow = raw + kr * kRowB + 68 * (kg >> 2);
+        const float kd = *reinterpret_cast<const float*>(krow);
+        uint32_t kc[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) kc[i] = *reinterpret_cast<const uint32_t*>(krow + 4 + 16 * (kg & 3) + 4 * i);
+        const uint8_t* va_row = raw + kPfRawBytes / 2 + (2 * vp) * kRowB + 68 * (vj >> 3);
+        const uint8_t* vb_row = va_row + kRowB;
+        float da = *reinterpret_cast<const float*>(va_row);
+        float db = *reinterpret_cast<const float*>(vb_row);
+        uint32_t va[2], vb[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            va[i] = *reinterpret_cast<const uint32_t*>(va_row + 4 + 8 * (vj & 7) + 4 * i);
+            vb[i] = *reinterpret_cast<const uint32_t*>(vb_row + 4 + 8 * (vj & 7) + 4 * i);
+        }
+        // ---- phase 2: dequantise ----
+        uint32_t kh[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float f[4];
+            codes4_to_f32<false>(kc[i], f);
+            kh[2 * i] = pack_h2(kd * f[0], kd * f[1]);
+            kh[2 * i + 1] = pack_h2(kd * f[2], kd * f[3]);
+        }
+        {
+            const int pa = t0 + 2 * vp;
+            const bool a_ok = pa >= lo_all && pa <= hi_all, b_ok = pa + 1 >= lo_all && pa + 1 <= hi_all;
+            va[0] = a_ok ? va[0] : 0u, va[1] = a_ok ? va[1] : 0u, da = a_ok ? da : 0.f;
+            vb[0] = b_ok ? vb[0] : 0u, vb[1] = b_ok ? vb[1] : 0u, db = b_ok ? db : 0.f;
+        }
+        float fa[8], fb[8];
+        {
+            float t[4];
+            codes4_to_f32<false>(va[0], t);
+            fa[0] = t[0], fa[1] = t[1], fa[2] = t[2], fa[3] = t[3];
+            codes4_to_f32<false>(va[1], t);
+            fa[4] = t[0], fa[5] = t[1], fa[6] = t[2], fa[7] = t[3];
+            codes4_to_f32<false>(vb[0], t);
+            fb[0] = t[0], fb[1] = t[1], fb[2] = t[2], fb[3] = t[3];
+            codes4_to_f32<false>(vb[1], t);
+            fb[4] = t[0], fb[5] = t[1], fb[6] = t[2], fb[7] = t[3];
+        }
+        // ---- phase 3: writes ----
+        *reinterpret_cast<u4*>(deq + kr * kPfKStride + 32 * kg) = u4{kh[0], kh[1], kh[2], kh[3]};
+        *reinterpret_cast<u4*>(deq + kr * kPfKStride + 32 * kg + 16) = u4{kh[4], kh[5], kh[6], kh[7]};
+        const int bp = (vp >> 1) & 3, sl = vp >> 3;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int d = 8 * vj + e;
+            *reinterpret_cast<uint32_t*>(deq + kPfKBytes + d * 64 + 16 * (bp ^ ((d >> 1) & 3)) + 8 * sl + 4 * (vp & 1)) =
+                pack_h2(da * fa[e], db * fb[e]);
+        }
+    };
+
     // 16-bit rows: nothing to dequantise.  K: thread (row r = tid / 16, segment g = tid % 16)
     // copies elements 16 g .. 16 g + 15 into the padded row-major tile.  V: thread (token pair
     // p = tid % 16, group j = tid / 16) stores dims 8 j .. 8 j + 7 of tokens 2p, 2p + 1 as (token 2p,
@@ -507,6 +576,9 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             if constexpr (K16) {  // rows as stored: no scales, the softmax factor comes in here
 #pragma unroll
                 for (int i = 0; i < 4; ++i) score[4 * s + i] = (s_acc[0][i] + s_acc[1][i]) * q_scale;
+            } else if constexpr (Q8) {  // the key tile already carries its scales
+#pragma unroll
+                for (int i = 0; i < 4; ++i) score[4 * s + i] = s_acc[0][i] + s_acc[1][i];
             } else {
                 const f4 kd0 = *reinterpret_cast<const f4*>(sc + 16 * s + 4 * b);
                 const f4 kd1 = *reinterpret_cast<const f4*>(sc + 32 + 16 * s + 4 * b);
@@ -559,7 +631,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             pb[0] = u4{hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16), hi[4] | (hi[5] << 16), hi[6] | (hi[7] << 16)};
             pb[1] = pb[0];
             pb_lo = u4{lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16), lo[4] | (lo[5] << 16), lo[6] | (lo[7] << 16)};
-        } else if constexpr (FP8 || K16) {  // the value tile already carries its scales
+        } else if constexpr (FP8 || K16 || Q8) {  // the value tile already carries its scales
             pb[0] = u4{pack_h2(p[0], p[1]), pack_h2(p[2], p[3]), pack_h2(p[4], p[5]), pack_h2(p[6], p[7])};
             pb[1] = pb[0];
         } else {
@@ -617,6 +689,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         if (it + 1 >= 0 && it + 1 < n_units) {
             if constexpr (K16) {
                 dequant_unit_16((it + 1) & 1, (it + 1) & 1, (u_first + it + 1) * kUnit);
+            } else if constexpr (Q8) {
+                dequant_unit_q8((it + 1) & 1, (it + 1) & 1, (u_first + it + 1) * kUnit);
             } else if constexpr (FP8) {
                 dequant_unit_fp8((it + 1) & 1, (it + 1) & 1, (u_first + it + 1) * kUnit);
             } else {
@@ -643,7 +717,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     // ---- epilogue: normalise, transpose through LDS, rotate back, store ----
     l_run = sum_over_rows(l_run);
     float* reg = reinterpret_cast<float*>(smem) + wave * 16 * 260;
-    const float inv = l_run > 0.f ? ((FP8 || K16) ? 1.0f : kLutInvGain) / l_run : 0.f;
+    const float inv = l_run > 0.f ? (TQ4F ? kLutInvGain : 1.0f) / l_run : 0.f;
 #pragma unroll
     for (int h = 0; h < 2; ++h)
 #pragma unroll
