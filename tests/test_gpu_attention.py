@@ -351,6 +351,40 @@ def test_prefill_tile_kernel_windows(mask_mode, window):
     _prefill_case(DT_F16, 16, [400, 130], [90, 130], 221, force=0, mask_mode=mask_mode, window=window)
 
 
+@pytest.mark.parametrize("dtype", [DT_BF16, DT_F16])
+def test_prefill_tile_kernel_long_chunks(dtype):
+    """The TQ4 tile kernel on chunks of a thousand tokens and more, through the automatic dispatch:
+    causal chunks on a prefix with ragged last tiles, 4, 8 and 16 q heads per kv head, 16- and
+    64-token pages, a sliding window, the non-causal window mode, a token mask, and
+    page-permutation invariance."""
+    import gpu_harness as G
+
+    _prefill_case(dtype, 64, [1500, 900], [1100, 650], 361)                       # gqa 8: 16-token tiles, ragged tails
+    _prefill_case(dtype, 16, [2100, 131], [2100, 90], 362, q_heads=8)             # gqa 4: 32-token tiles, no prefix
+    _prefill_case(dtype, 64, [700, 1300], [700, 530], 363, q_heads=32)            # gqa 16: 8-token tiles
+    _prefill_case(dtype, 16, [1301, 77], [1301, 40], 364, mask_mode=0, window=200)
+    _prefill_case(dtype, 64, [1100], [1100], 365, mask_mode=1, window=96)
+    # token mask + two page permutations of the same data
+    seq_lens, q_lens = [1400, 300], [1200, 300]
+    outs = []
+    for perm_seed in (1, 2):
+        pool, bt, k, v, q, aq, ctx = make_case(FMT_TQ4, 16, seq_lens, q_lens, 366, dtype, q_heads=16, perm_seed=perm_seed)
+        tmask = np.ones(sum(q_lens), dtype=np.uint8)
+        tmask[5:40] = 0
+        tmask[1199] = 0
+        hb = oracle.HostBatch(aq, seq_lens, bt, context_lens_before=ctx, valid_token_mask=tmask)
+        rc, got, _ = G.dev_attention(_dev_pool(pool), hb, q, dtype, 16, scratch_bytes=SCRATCH, sentinel=0x5500)
+        assert rc == 0
+        outs.append(got)
+        if perm_seed == 1:
+            want = oracle.paged_attention(pool, hb, q, dtype, 16, n_threads=8)
+            live = tmask.astype(bool)
+            G.assert_close(got[live], dtype, want[live], what="long chunks, token mask",
+                           scale=G.channel_scale(v, dtype, hb, 16)[live])
+            assert np.all(got[~live] == 0x5500), "masked rows must stay untouched"
+    assert outs[0].tobytes() == outs[1].tobytes(), "result depends on the physical page numbering"
+
+
 @pytest.mark.parametrize("fmt", [FMT_FP8, FMT_Q8_0])
 @pytest.mark.parametrize("xf", [XF_IDENTITY, XF_WHT256])
 @pytest.mark.parametrize("dtype", [DT_BF16, DT_F16])
