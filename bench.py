@@ -619,7 +619,8 @@ def run_workload(args, torch, lib, ffi, dev):
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": {"tq4": "f16 MFMA operands (TQ4 codes -> fp16 centroids), f32 accumulate, bf16 Q/out",
+        "dtype": "bf16" if fmt == "bf16" else "f16",  # type of the MFMA operands; sums and softmax in f32
+        "dtype_detail": {"tq4": "f16 MFMA operands (TQ4 codes -> fp16 centroids), f32 accumulate, bf16 Q/out",
                   "bf16": "bf16 MFMA operands, f32 accumulate, bf16 Q/out",
                   "fp8": "f16 MFMA operands (E4M3 codes widened, fp32 block scales), f32 accumulate, bf16 Q/out",
                   "q8_0": "f16 MFMA operands (int8 codes widened, fp32 block scales), f32 accumulate, bf16 Q/out"}[fmt],
