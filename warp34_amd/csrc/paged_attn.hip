@@ -1489,7 +1489,7 @@ namespace w34 {
 constexpr int kMaxChunksCap = 256;
 // 256 tokens, one unit per wave: 7 to 12 % faster than 16 at 16K-32K keys, same as 4
 constexpr int kMinUnitsPerChunk = 8;
-constexpr int kTargetWorkgroupsPerHead = 128;
+constexpr int kTargetWorkgroups = 256;  // one workgroup per compute unit
 constexpr int kBalWorkgroups = 256;  // balanced decode: one workgroup per compute unit
 
 static size_t partial_bytes(long long rows, int max_chunks) {
@@ -1497,10 +1497,13 @@ static size_t partial_bytes(long long rows, int max_chunks) {
 }
 
 // Cap on chunks per tile: a function of total_tokens (tiles) and the scratch size only.
-static int choose_max_chunks(const warp34_exec* ex, int total_tokens, int num_q_heads, int tok_tile) {
+static int choose_max_chunks(const warp34_exec* ex, int total_tokens, int num_q_heads, int tok_tile, int kv_subs) {
     if (ex->scratch_ptr == 0 || (ex->scratch_ptr & 15u) != 0u) return 1;
     const int tiles = (total_tokens + tok_tile - 1) / tok_tile;
-    int want = kTargetWorkgroupsPerHead / (tiles > 0 ? tiles : 1);
+    // chunks x (kv heads x q subgroups) x tiles workgroups fill the chip once: a rank that holds
+    // one kv head of a sharded model cuts its tiles into twice as many chunks as one that holds two
+    const long long per_chunk = (long long)(tiles > 0 ? tiles : 1) * (kv_subs > 0 ? kv_subs : 1);
+    int want = (int)(kTargetWorkgroups / per_chunk);
     if (want > kMaxChunksCap) want = kMaxChunksCap;
     if (want < 2) return 1;
     const long long rows = (long long)total_tokens * num_q_heads;
@@ -1571,21 +1574,26 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     P.tok_tile = (16 * nt) / q_group;
     if (P.tok_tile < 1) P.tok_tile = 1;
     P.min_upc = kMinUnitsPerChunk;
-    P.max_chunks = force_single ? 1 : choose_max_chunks(ex, batch->total_tokens, num_q_heads, P.tok_tile);
+    P.max_chunks = force_single ? 1 : choose_max_chunks(ex, batch->total_tokens, num_q_heads, P.tok_tile,
+                                                        layout->local_kv_heads * P.q_subgroups);
     P.part_acc = nullptr;
     P.part_ml = nullptr;
     const long long rows = (long long)batch->total_tokens * num_q_heads;
-    if (P.max_chunks > 1) {
-        uint8_t* ws = reinterpret_cast<uint8_t*>((uintptr_t)ex->scratch_ptr);
-        P.part_acc = reinterpret_cast<float*>(ws);
-        P.part_ml = P.part_acc + (size_t)rows * P.max_chunks * kHeadDim;
-    }
     // grid.x: chunks that can exist given the host's upper bound on the sequence length
     int grid_x = P.max_chunks;
     if (batch->max_seq_len > 0) {
         const int units = (batch->max_seq_len + kUnit - 1) / kUnit + 1;
         const int bound = (units + P.min_upc - 1) / P.min_upc;
         if (bound < grid_x) grid_x = bound < 1 ? 1 : bound;
+    }
+    // No tile has more chunks than that: the cap is lowered to it, which changes no chunk (a
+    // tile's count is limited by its own units first) and keeps the partial records, and what
+    // the merge kernel loads ahead of knowing the count, as small as the bound allows.
+    P.max_chunks = grid_x;
+    if (P.max_chunks > 1) {
+        uint8_t* ws = reinterpret_cast<uint8_t*>((uintptr_t)ex->scratch_ptr);
+        P.part_acc = reinterpret_cast<float*>(ws);
+        P.part_ml = P.part_acc + (size_t)rows * P.max_chunks * kHeadDim;
     }
     // grid.z: tiles.  One per request when no request can have two; otherwise the upper bound
     // sum_r ceil(q_r / tok_tile) <= total_tokens / tok_tile + num_reqs
@@ -1655,20 +1663,25 @@ static int launch_rows(const warp34_exec* ex, const warp34_kv_layer_layout* layo
     P.tok_tile = 16 / q_group;  // one N tile
     if (P.tok_tile < 1) P.tok_tile = 1;
     P.min_upc = kMinUnitsPerChunk;
-    P.max_chunks = force_single ? 1 : choose_max_chunks(ex, batch->total_tokens, num_q_heads, P.tok_tile);
+    P.max_chunks = force_single ? 1 : choose_max_chunks(ex, batch->total_tokens, num_q_heads, P.tok_tile,
+                                                        layout->local_kv_heads * P.q_subgroups);
     P.part_acc = nullptr;
     P.part_ml = nullptr;
     const long long rows = (long long)batch->total_tokens * num_q_heads;
-    if (P.max_chunks > 1) {
-        uint8_t* ws = reinterpret_cast<uint8_t*>((uintptr_t)ex->scratch_ptr);
-        P.part_acc = reinterpret_cast<float*>(ws);
-        P.part_ml = P.part_acc + (size_t)rows * P.max_chunks * kHeadDim;
-    }
     int grid_x = P.max_chunks;
     if (batch->max_seq_len > 0) {
         const int units = (batch->max_seq_len + kUnit - 1) / kUnit + 1;
         const int bound = (units + P.min_upc - 1) / P.min_upc;
         if (bound < grid_x) grid_x = bound < 1 ? 1 : bound;
+    }
+    // No tile has more chunks than that: the cap is lowered to it, which changes no chunk (a
+    // tile's count is limited by its own units first) and keeps the partial records, and what
+    // the merge kernel loads ahead of knowing the count, as small as the bound allows.
+    P.max_chunks = grid_x;
+    if (P.max_chunks > 1) {
+        uint8_t* ws = reinterpret_cast<uint8_t*>((uintptr_t)ex->scratch_ptr);
+        P.part_acc = reinterpret_cast<float*>(ws);
+        P.part_ml = P.part_acc + (size_t)rows * P.max_chunks * kHeadDim;
     }
     P.tiles_by_request = (batch->max_q_len > 0 && batch->max_q_len <= P.tok_tile) ? 1 : 0;
     P.rot_q = layout->k_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 ? 1 : 0;
@@ -2024,7 +2037,7 @@ extern "C" int warp34_paged_attention_f16_force_kernel_for_test(
 extern "C" size_t warp34_paged_attention_scratch_bytes(int total_tokens, int num_q_heads, int max_seq_len) {
     (void)max_seq_len;
     if (total_tokens <= 0 || num_q_heads <= 0) return 0;
-    int want = kTargetWorkgroupsPerHead / total_tokens;
+    int want = kTargetWorkgroups / total_tokens;  // the layout is not known here: one kv head, one q subgroup
     if (want > kMaxChunksCap) want = kMaxChunksCap;
     if (want < 2) want = 2;
     size_t bytes = partial_bytes((long long)total_tokens * num_q_heads, want);
