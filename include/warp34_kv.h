@@ -260,6 +260,11 @@ int warp34_qsa_sparse_paged_attn_hadamard_f16(
  * (split-K partials).  No counterpart in the reference, whose engine simply guarantees
  * >= 8 MiB (op_paged_attn.cu:1301-1304); provided so a host can size ex->scratch. */
 size_t warp34_paged_attention_scratch_bytes(int total_tokens, int num_q_heads, int max_seq_len);
+/* The same for a known layout and request count: the exact figure the launchers use (the form
+ * above does not know local_kv_heads and returns the largest need over all layouts).
+ * num_reqs < 0: unknown, total_tokens is assumed.  No counterpart in the reference. */
+size_t warp34_paged_attention_scratch_bytes_for_layout(const warp34_kv_layer_layout* layout, int total_tokens,
+                                                       int num_reqs, int num_q_heads, int max_seq_len);
 
 /* ------------------------------------------------------------------------------------
  * Runtime shims a standalone harness needs (replace op_init.cu; warp34_cuda.h:135,142-164).

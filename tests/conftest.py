@@ -27,3 +27,15 @@ def pytest_collection_modifyitems(config, items):
                     have_gpu = False
             if not have_gpu:
                 item.add_marker(pytest.mark.skip(reason="no GPU visible"))
+
+
+def pytest_terminal_summary(terminalreporter):
+    """Parity figures of the GPU tests: one line per comparison against the oracle."""
+    try:
+        import gpu_harness
+    except Exception:
+        return
+    if gpu_harness.PARITY_LOG:
+        terminalreporter.section("attention parity against the oracle (unscaled contract figures)")
+        for line in gpu_harness.PARITY_LOG:
+            terminalreporter.write_line(line)

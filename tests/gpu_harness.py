@@ -1,6 +1,7 @@
 """Device-side harness for the GPU parity tests: torch supplies device memory and the
 stream, every compute call goes through the C ABI of libwarp34_kernels.so."""
 import ctypes as C
+import os
 
 import numpy as np
 import torch
@@ -160,33 +161,63 @@ def channel_scale(v_bits, dtype, hbatch, num_q_heads):
     return out
 
 
-def assert_close(got_bits, dtype, want_f32, atol=2e-3, rtol=1e-2, what="", scale=None):
-    """Target tolerance (max-abs 2e-3, max-rel 1e-2 against the fp32-dequant / fp64-accumulate
-    oracle), with the absolute part relative to the magnitude of the data being averaged:
+# one line per assert_close call, printed in pytest's terminal summary (tests/conftest.py)
+PARITY_LOG = []
+OUTLIER_FROM = 8.0  # a channel whose values reach this magnitude is one of the x20 outlier channels
 
-        |got - want| <= atol * scale + rtol * |want|
 
-    An attention output is a probability-weighted mean of V rows, so an error eps in the
-    probabilities moves channel c by up to eps * max_t |V[t, c]|; `scale` is that magnitude
-    (channel_scale()), or, when not given, max(1, max|want_row|).  It differs from 1 only for
-    the x20 outlier channels of the benchmark inputs, where a single fp16 / bf16 output ulp
-    already exceeds 2e-3.  On unit-scale data this is exactly 2e-3 + 1e-2 |want|.
-    The max-rel figure max|err| / max|want| must also stay below rtol.
+def assert_close(got_bits, dtype, want_f32, atol=2e-3, rtol=1e-2, what="", scale=None, plain_excess=0.0):
+    """The contract: max-abs 2e-3, max-rel 1e-2 against the fp32-dequant / fp64-accumulate oracle,
+    read per element as  |got - want| <= atol + rtol * |want|.
+
+    That bound is asserted as it stands on every channel of unit-scale data.  `scale`
+    (channel_scale(): max |V[t, c]| over the keys being averaged, at least 1) names the x20
+    outlier channels of the benchmark inputs, those with scale >= OUTLIER_FROM; on them the
+    absolute part is taken relative to the data,  atol * scale + rtol * |want|:  the kernels
+    multiply fp16 operands as the reference's MMA kernels do (op_paged_attn.cu:33-58 rounds
+    d * centroid to fp16, :450-560 the probabilities), one operand rounding is 2^-11 relative, and
+    an output of such a channel is a sum of products p * V with |V| up to `scale`, so an error of
+    2^-11 * scale ~ 5e-4 * scale is inherent to that arithmetic whatever |want| cancels to.
+    Without `scale` every channel is held to the plain bound.
+
+    `plain_excess` (default 0) is an absolute allowance on top of the plain bound for the few
+    cases that sit on the floor of fp16 operand arithmetic with x20 outlier inputs; a test that
+    passes one says which mechanism it is for.  Two exist.  (1) The dequantisation table holds
+    fp16 centroids (relative error up to 9.4e-5, the same for every element with the same code);
+    a rotated row with outlier channels has elements of magnitude ~|V_c| / 16 everywhere, and
+    the inverse rotation turns that code-wise error into single plain channels (c1 ^ c2 ^ c3 of
+    the outlier channels): a few 1e-4 in rows that one key dominates.  (2) fp16 probability and
+    value operands, as in the reference's MMA kernels: up to 2 * 2^-11 * sum_t p_t |V[t, c]|,
+    which passes 2e-3 when large values of opposite sign cancel in `want`.
+
+    Every call is logged with the unscaled figures: max-abs error, max-rel (max|err| / max|want|)
+    and the worst excess over atol + rtol * |want| on all channels (<= 0 means the plain contract
+    holds everywhere, outlier channels included).
     """
     got = oracle.bits_to_f32(got_bits, dtype).astype(np.float64)
     want = np.asarray(want_f32, dtype=np.float64)
     assert got.shape == want.shape
     assert np.isfinite(got).all(), "non-finite output " + what
     err = np.abs(got - want)
+    plain_bound = atol + rtol * np.abs(want)
     if scale is None:
-        scale = np.maximum(1.0, np.abs(want).max(axis=-1, keepdims=True))
-    bound = atol * scale + rtol * np.abs(want)
+        bound = plain_bound + plain_excess
+        n_outlier = 0
+    else:
+        scale = np.broadcast_to(np.asarray(scale, dtype=np.float64), want.shape)
+        outlier = scale >= OUTLIER_FROM
+        bound = np.where(outlier, atol * scale, atol + plain_excess) + rtol * np.abs(want)
+        n_outlier = int(outlier.sum())
     worst = float((err - bound).max()) if err.size else 0.0
+    worst_plain = float((err - plain_bound).max()) if err.size else 0.0
+    max_abs = float(err.max()) if err.size else 0.0
     max_rel = float(err.max() / max(np.abs(want).max(), 1e-30)) if err.size else 0.0
-    assert worst <= 0.0, "%s: max-abs err %.3e, max-rel %.3e (bound exceeded by %.3e)" % (
-        what, float(err.max()), max_rel, worst)
+    PARITY_LOG.append("%s | %s: max-abs %.3e max-rel %.3e excess over 2e-3+1e-2|want| %+.3e (%d of %d elements on outlier channels)"
+                      % (os.environ.get("PYTEST_CURRENT_TEST", "-").split(" ")[0], what, max_abs, max_rel, worst_plain,
+                         n_outlier, err.size))
+    assert worst <= 0.0, "%s: max-abs err %.3e, max-rel %.3e (bound exceeded by %.3e)" % (what, max_abs, max_rel, worst)
     assert max_rel <= rtol, "%s: max-rel %.3e" % (what, max_rel)
-    return float(err.max()) if err.size else 0.0
+    return max_abs
 
 
 def dev_qsa_sparse(dpool, q_bits, sel_phys, sel_log, num_sel, seq_pos, num_q_heads, sm_scale=0.0625, gate=None,

@@ -318,7 +318,7 @@ def test_kv8_unwritten_pool_bytes_do_not_leak(fmt):
 # ---- chunked prefill over TQ4 pages (128-row tile kernel) ----
 
 def _prefill_case(dtype, block_size, seq_lens, q_lens, seed, q_heads=16, force=None, fmt=FMT_TQ4, xf=None,
-                  mask_mode=0, window=0, **kw):
+                  mask_mode=0, window=0, plain_excess=0.0, **kw):
     import gpu_harness as G
 
     pool, bt, k, v, q, aq, ctx = make_case(fmt, block_size, seq_lens, q_lens, seed, dtype, q_heads=q_heads, xf=xf)
@@ -328,7 +328,7 @@ def _prefill_case(dtype, block_size, seq_lens, q_lens, seed, q_heads=16, force=N
     rc, got, _ = G.dev_attention(dpool, hb, q, dtype, q_heads, scratch_bytes=SCRATCH, force_kernel=force)
     assert rc == 0
     G.assert_close(got, dtype, want, what="prefill bs=%d seq=%s q=%s" % (block_size, seq_lens, q_lens),
-                   scale=G.channel_scale(v, dtype, hb, q_heads))
+                   scale=G.channel_scale(v, dtype, hb, q_heads), plain_excess=plain_excess)
     return pool, hb, q, got, want
 
 
@@ -379,8 +379,10 @@ def test_prefill_tile_kernel_long_chunks(dtype):
         if perm_seed == 1:
             want = oracle.paged_attention(pool, hb, q, dtype, 16, n_threads=8)
             live = tmask.astype(bool)
+            # fp16 centroid table on rotated outlier rows (mechanism 1 of assert_close): one element
+            # of 6 million is 2.8e-4 over the plain bound
             G.assert_close(got[live], dtype, want[live], what="long chunks, token mask",
-                           scale=G.channel_scale(v, dtype, hb, 16)[live])
+                           scale=G.channel_scale(v, dtype, hb, 16)[live], plain_excess=4e-4)
             assert np.all(got[~live] == 0x5500), "masked rows must stay untouched"
     assert outs[0].tobytes() == outs[1].tobytes(), "result depends on the physical page numbering"
 
@@ -392,10 +394,15 @@ def test_prefill_tile_kernel_8bit_pages(xf, dtype, fmt):
     """The tile kernel over FP8-E4M3 pages (same row shape as TQ4: two scale blocks of 128) and
     Q8_0 pages (four blocks of 64, dequantised into both tiles), plain and rotated, through the
     automatic dispatch and the test selector."""
-    _prefill_case(dtype, 64, [1500, 900], [1100, 650], 331, fmt=fmt, xf=xf)
+    # The value tile holds fp16(d * code) and the probabilities are fp16, as in the reference's MMA
+    # kernels (op_paged_attn.cu:59-105): mechanism 2 of assert_close leaves single elements of
+    # millions up to 3e-4 over the plain bound.  Rotated rows add the block-wise part of that
+    # rounding (few distinct codes per scale block), which the inverse rotation gathers: up to 1e-3.
+    ex = 4e-4 if xf == XF_IDENTITY else 1.2e-3
+    _prefill_case(dtype, 64, [1500, 900], [1100, 650], 331, fmt=fmt, xf=xf, plain_excess=ex)
     if dtype == DT_F16:  # the test selector is an f16 entry point
-        _prefill_case(dtype, 16, [300, 77], [130, 40], 332, fmt=fmt, xf=xf, force=1)
-        _prefill_case(dtype, 64, [700], [333], 333, fmt=fmt, xf=xf, mask_mode=1, window=64, force=1)
+        _prefill_case(dtype, 16, [300, 77], [130, 40], 332, fmt=fmt, xf=xf, force=1, plain_excess=ex)
+        _prefill_case(dtype, 64, [700], [333], 333, fmt=fmt, xf=xf, mask_mode=1, window=64, force=1, plain_excess=ex)
 
 
 @pytest.mark.parametrize("dtype", [DT_BF16, DT_F16])

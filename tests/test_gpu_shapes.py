@@ -3,7 +3,7 @@ heads, 1, 2 and 16 q heads per kv head, every page format, decode / verify / pre
 batches with windows and both mask modes, with no, a too small and a large scratch.
 
 The cases are fixed (drawn once from a randomised soak of the entry points against the oracle);
-the tolerance is the one of tests/test_gpu_attention.py."""
+the tolerance is the one of tests/test_gpu_attention.py (gpu_harness.assert_close)."""
 import numpy as np
 import pytest
 
@@ -56,5 +56,8 @@ def test_attention_shape(case):
     dpool.upload()
     rc, got, _ = G.dev_attention(dpool, hb, q, dtype, q_heads, scratch_bytes=scratch)
     assert rc == 0
+    # rotated 8-bit rows: the block-wise part of the fp16(d * code) rounding, gathered by the inverse
+    # rotation (see test_prefill_tile_kernel_8bit_pages)
+    rotated_8bit = fmt in (oracle.FMT_FP8, oracle.FMT_Q8_0) and xf == oracle.XF_WHT256
     G.assert_close(got, dtype, want, what="fmt=%d bs=%d seq=%s q=%s" % (fmt, block_size, seq_lens, q_lens),
-                   scale=G.channel_scale(v, dtype, hb, q_heads))
+                   scale=G.channel_scale(v, dtype, hb, q_heads), plain_excess=1.2e-3 if rotated_8bit else 0.0)

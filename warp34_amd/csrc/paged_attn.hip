@@ -38,6 +38,7 @@
 //
 // MFMA use: v_mfma_f32_16x16x32_f16.  A = K rows (QK) or V^T (PV) so that every lane owns one
 // query column: softmax state and the O rescale are per-lane scalars.
+#include <atomic>
 #include <type_traits>
 
 #include "kv_common.h"
@@ -206,6 +207,17 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
     f2 f = {a, b};
     h2 h = __builtin_convertvector(f, h2);
     return __builtin_bit_cast(uint32_t, h);
+}
+// Two fp16 operands for one fp32 weight pair: hi = fp16(w), lo = fp16(w - hi).  A value scale
+// that is folded into the probabilities (w = p * d) reaches every element of a 128-wide scale
+// block through ONE number; rounded to fp16 once, its error is the same for the whole block,
+// and the inverse rotation gathers such a block-wide error into a single output channel
+// (channel c ^ 128 of a channel c with large values).  With the low-order operand the weight
+// carries 22 bits and that error disappears; the price is a second MFMA per value tile.
+__device__ __forceinline__ void split_h2(float a, float b, uint32_t& hi, uint32_t& lo) {
+    const h2 h = __builtin_convertvector(f2{a, b}, h2);
+    hi = __builtin_bit_cast(uint32_t, h);
+    lo = pack_h2(a - (float)h[0], b - (float)h[1]);
 }
 __device__ __forceinline__ float half_lo_to_f32(uint32_t w) {
     return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xFFFFu));
@@ -837,7 +849,7 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         }
 
         // ---- online softmax (log2 domain), per lane = per query column --------------------
-        uint32_t pb[NT][2][4];
+        float p[NT][8];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             float mx = fmaxf(fmaxf(fmaxf(sc[nt][0], sc[nt][1]), fmaxf(sc[nt][2], sc[nt][3])),
@@ -846,44 +858,23 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
             const float m_new = fmaxf(m_run[nt], mx);
             const float alpha = __builtin_amdgcn_exp2f(m_run[nt] - m_new);
             m_run[nt] = m_new;
-            float p[8];
             float psum = 0.f;
             // (the MASKED tests sit outside the unrolled loops: one wave-uniform branch per block
             // instead of one per element, and the eight exponentials can overlap)
 #pragma unroll
-            for (int t = 0; t < 8; ++t) p[t] = __builtin_amdgcn_exp2f(sc[nt][t] - m_new);
+            for (int t = 0; t < 8; ++t) p[nt][t] = __builtin_amdgcn_exp2f(sc[nt][t] - m_new);
             if (MASKED) {
 #pragma unroll
-                for (int t = 0; t < 8; ++t) p[t] = sc[nt][t] > 0.5f * kNegBig ? p[t] : 0.f;
+                for (int t = 0; t < 8; ++t) p[nt][t] = sc[nt][t] > 0.5f * kNegBig ? p[nt][t] : 0.f;
             }
 #pragma unroll
-            for (int t = 0; t < 8; ++t) psum += p[t];
+            for (int t = 0; t < 8; ++t) psum += p[nt][t];
             l_run[nt] = l_run[nt] * alpha + psum;
             if (__ballot(alpha != 1.0f) != 0ull) {
 #pragma unroll
                 for (int h = 0; h < 2; ++h)
 #pragma unroll
                     for (int j = 0; j < 8; ++j) o_acc[nt][h][j] *= alpha;
-            }
-            float w0[8], w1[8];
-#pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                w0[t] = p[t] * half_lo_to_f32(vd0[t]);
-                w1[t] = p[t] * half_hi_to_f32(vd16[t]);
-            }
-            if (MASKED) {
-                // masked tokens have p == 0; select instead of multiply so that a garbage scale
-                // (rows beyond the sequence end) cannot inject NaN
-#pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    w0[t] = p[t] > 0.f ? w0[t] : 0.f;
-                    w1[t] = p[t] > 0.f ? w1[t] : 0.f;
-                }
-            }
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                pb[nt][0][k] = pack_h2(w0[2 * k], w0[2 * k + 1]);
-                pb[nt][1][k] = pack_h2(w1[2 * k], w1[2 * k + 1]);
             }
         }
 
@@ -893,6 +884,24 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         // ---- O^T += V^T P^T ------------------------------------------------------------------
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
+            // weights of this half: probability times the half-row scale of the value row, as a
+            // high and a low fp16 operand (split_h2)
+            uint32_t pb_hi[NT][4], pb_lo[NT][4];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                float w[8];
+#pragma unroll
+                for (int t = 0; t < 8; ++t)
+                    w[t] = p[nt][t] * (h == 0 ? half_lo_to_f32(vd0[t]) : half_hi_to_f32(vd16[t]));
+                if (MASKED) {
+                    // masked tokens have p == 0; select instead of multiply so that a garbage scale
+                    // (rows beyond the sequence end) cannot inject NaN
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) w[t] = p[nt][t] > 0.f ? w[t] : 0.f;
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) split_h2(w[2 * k], w[2 * k + 1], pb_hi[nt][k], pb_lo[nt][k]);
+            }
             uint32_t lo[4], hi[4];
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
@@ -926,9 +935,12 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
                 const h8 av = __builtin_bit_cast(h8, a[j]);
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
-                    u4 pbv = {pb[nt][h][0], pb[nt][h][1], pb[nt][h][2], pb[nt][h][3]};
+                    const u4 ph = {pb_hi[nt][0], pb_hi[nt][1], pb_hi[nt][2], pb_hi[nt][3]};
+                    const u4 pl = {pb_lo[nt][0], pb_lo[nt][1], pb_lo[nt][2], pb_lo[nt][3]};
                     o_acc[nt][h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                        av, __builtin_bit_cast(h8, pbv), o_acc[nt][h][j], 0, 0, 0);
+                        av, __builtin_bit_cast(h8, ph), o_acc[nt][h][j], 0, 0, 0);
+                    o_acc[nt][h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                        av, __builtin_bit_cast(h8, pl), o_acc[nt][h][j], 0, 0, 0);
                 }
             }
         }
@@ -1104,8 +1116,8 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
 template <typename TQ, int NT>
 __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(const AttnParams P) {
     extern __shared__ __align__(16) uint8_t smem[];
-    // lut_read() addresses the table absolutely
-    if ((uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem != 0u) __builtin_trap();
+    // lut_read() addresses the table absolutely: the dynamic block starts at LDS address 0 because
+    // the kernel has no static LDS (checked on the host before the first launch)
     tq4_tile<TQ, NT, false>(P, smem, BalItem{});
 }
 
@@ -1209,7 +1221,6 @@ __device__ __forceinline__ void bal_for_each_piece(const AttnParams& P, TileFn&&
 template <typename TQ>
 __global__ __launch_bounds__(waves_for(1) * 64, 1) void paged_attn_tq4_balanced_kernel(const AttnParams P) {
     extern __shared__ __align__(16) uint8_t smem[];
-    if ((uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem != 0u) __builtin_trap();
     bal_for_each_piece(P, [&](const BalItem& it) { tq4_tile<TQ, 1, true>(P, smem, it); });
 }
 
@@ -1489,21 +1500,26 @@ namespace w34 {
 constexpr int kMaxChunksCap = 256;
 // 256 tokens, one unit per wave: 7 to 12 % faster than 16 at 16K-32K keys, same as 4
 constexpr int kMinUnitsPerChunk = 8;
-constexpr int kTargetWorkgroups = 256;  // one workgroup per compute unit
-constexpr int kBalWorkgroups = 256;  // balanced decode: one workgroup per compute unit
+// Split geometry is sized for the layout the path is built for, two kv heads per device: 128
+// chunks (or shares) per kv head.  The counts below depend on the batch and on gqa only, never
+// on local_kv_heads: a rank that holds one kv head of a sharded model computes every row with
+// the same chunks, in the same order, as a rank that holds all of them (bit-identical outputs
+// under head sharding, op_paged_attn.cu:1301-1304), at the price of half-filled compute units
+// on such a rank.
+constexpr int kTargetWorkgroupsPerHead = 128;
 
 static size_t partial_bytes(long long rows, int max_chunks) {
     return (size_t)rows * (size_t)max_chunks * (kHeadDim + 4) * sizeof(float);
 }
 
-// Cap on chunks per tile: a function of total_tokens (tiles) and the scratch size only.
-static int choose_max_chunks(const warp34_exec* ex, int total_tokens, int num_q_heads, int tok_tile, int kv_subs) {
+// Cap on chunks per tile: a function of total_tokens (tiles), gqa (q subgroups per kv head) and
+// the scratch size only.
+static int choose_max_chunks(const warp34_exec* ex, int total_tokens, int num_q_heads, int tok_tile,
+                             int q_subgroups) {
     if (ex->scratch_ptr == 0 || (ex->scratch_ptr & 15u) != 0u) return 1;
     const int tiles = (total_tokens + tok_tile - 1) / tok_tile;
-    // chunks x (kv heads x q subgroups) x tiles workgroups fill the chip once: a rank that holds
-    // one kv head of a sharded model cuts its tiles into twice as many chunks as one that holds two
-    const long long per_chunk = (long long)(tiles > 0 ? tiles : 1) * (kv_subs > 0 ? kv_subs : 1);
-    int want = (int)(kTargetWorkgroups / per_chunk);
+    const long long per_chunk = (long long)(tiles > 0 ? tiles : 1) * (q_subgroups > 0 ? q_subgroups : 1);
+    int want = (int)(kTargetWorkgroupsPerHead / per_chunk);
     if (want > kMaxChunksCap) want = kMaxChunksCap;
     if (want < 2) return 1;
     const long long rows = (long long)total_tokens * num_q_heads;
@@ -1511,24 +1527,45 @@ static int choose_max_chunks(const warp34_exec* ex, int total_tokens, int num_q_
     return want < 2 ? 1 : want;
 }
 
+// One attribute call per kernel instantiation and device.  The record is process-wide and
+// lock-free: slot i belongs to the first kernel that claims it, bit d of its mask says that
+// device d is configured.  Kernels that address their dequantisation table absolutely
+// (lds_base_zero) also have their static LDS size checked here: it must be zero, so that the
+// dynamic block starts at LDS address 0.
+constexpr int kLdsRecordSlots = 96;
+static std::atomic<const void*> g_lds_fn[kLdsRecordSlots];
+static std::atomic<unsigned long long> g_lds_devs[kLdsRecordSlots];
+
 template <typename KernelT>
-static int ensure_dynamic_lds(KernelT kernel, int bytes) {
-    // one attribute call per kernel instantiation and device
-    static thread_local const void* done_fn[16];
-    static thread_local int done_dev[16];
-    static thread_local int n_done = 0;
+static int ensure_dynamic_lds(KernelT kernel, int bytes, bool lds_base_zero = false) {
     int dev = 0;
     hipError_t rc = hipGetDevice(&dev);
     if (rc != hipSuccess) return (int)rc;
-    for (int i = 0; i < n_done; ++i)
-        if (done_fn[i] == (const void*)kernel && done_dev[i] == dev) return 0;
-    rc = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    if (rc != hipSuccess) return (int)rc;
-    if (n_done < 16) {
-        done_fn[n_done] = (const void*)kernel;
-        done_dev[n_done] = dev;
-        ++n_done;
+    const void* fn = (const void*)kernel;
+    int slot = -1;
+    for (int i = 0; i < kLdsRecordSlots; ++i) {
+        const void* cur = g_lds_fn[i].load(std::memory_order_acquire);
+        if (cur == nullptr) {
+            const void* expect = nullptr;
+            if (g_lds_fn[i].compare_exchange_strong(expect, fn, std::memory_order_acq_rel)) cur = fn;
+            else cur = expect;
+        }
+        if (cur == fn) {
+            slot = i;
+            break;
+        }
     }
+    const bool tracked = slot >= 0 && dev >= 0 && dev < 64;
+    if (tracked && ((g_lds_devs[slot].load(std::memory_order_acquire) >> dev) & 1ull)) return 0;
+    if (lds_base_zero) {
+        hipFuncAttributes attr;
+        rc = hipFuncGetAttributes(&attr, fn);
+        if (rc != hipSuccess) return (int)rc;
+        if (attr.sharedSizeBytes != 0) return (int)hipErrorInvalidConfiguration;
+    }
+    rc = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (rc != hipSuccess) return (int)rc;
+    if (tracked) g_lds_devs[slot].fetch_or(1ull << dev, std::memory_order_release);
     return 0;
 }
 
@@ -1539,8 +1576,9 @@ static bool balanced_decode_applicable(const warp34_exec* ex, const warp34_atten
     return tiles_by_request && batch->num_reqs >= 2 && !force_single && batch->sliding_window <= 0 &&
            batch->valid_token_mask == nullptr && ex->scratch_ptr != 0 && (ex->scratch_ptr & 15u) == 0u;
 }
-static int balanced_groups(int kv_subs) {
-    int groups = kBalWorkgroups / kv_subs;
+// shares of a balanced decode batch per (kv head, q subgroup): a function of gqa only
+static int balanced_groups(int q_subgroups) {
+    int groups = kTargetWorkgroupsPerHead / (q_subgroups > 0 ? q_subgroups : 1);
     if (groups > kMergeGroups * kMergeMaxPerGroup - 1) groups = kMergeGroups * kMergeMaxPerGroup - 1;
     return groups < 1 ? 1 : groups;
 }
@@ -1575,7 +1613,7 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     if (P.tok_tile < 1) P.tok_tile = 1;
     P.min_upc = kMinUnitsPerChunk;
     P.max_chunks = force_single ? 1 : choose_max_chunks(ex, batch->total_tokens, num_q_heads, P.tok_tile,
-                                                        layout->local_kv_heads * P.q_subgroups);
+                                                        P.q_subgroups);
     P.part_acc = nullptr;
     P.part_ml = nullptr;
     const long long rows = (long long)batch->total_tokens * num_q_heads;
@@ -1606,14 +1644,14 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     // Decode batches of several requests: equal shares of the batch's units per workgroup
     // instead of per-request chunks (the requests' lengths are unknown to the host and differ).
     if (balanced_decode_applicable(ex, batch, P.tiles_by_request, force_single)) {
-        const int groups = balanced_groups(kv_subs);
+        const int groups = balanced_groups(P.q_subgroups);
         const size_t prows = bal_partial_row(groups + batch->num_reqs, kv_subs, 0, 0);
         if (partial_bytes((long long)prows, 1) + (size_t)batch->total_tokens * 16 <= ex->scratch_size) {
             P.part_acc = reinterpret_cast<float*>((uintptr_t)ex->scratch_ptr);
             P.part_ml = P.part_acc + prows * kHeadDim;
             P.bal_table = reinterpret_cast<int32_t*>(P.part_ml + prows * 4);
             P.max_chunks = groups + 1;
-            rc = ensure_dynamic_lds(paged_attn_tq4_balanced_kernel<TQ>, smem_bytes_for(1));
+            rc = ensure_dynamic_lds(paged_attn_tq4_balanced_kernel<TQ>, smem_bytes_for(1), true);
             if (rc) return rc;
             hipLaunchKernelGGL((paged_attn_tq4_balanced_kernel<TQ>), dim3((unsigned)groups, (unsigned)kv_subs),
                                dim3(waves_for(1) * 64), smem_bytes_for(1), stream, P);
@@ -1625,7 +1663,7 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
             return (int)hipGetLastError();
         }
     }
-    rc = ensure_dynamic_lds(paged_attn_tq4_kernel<TQ, 1>, smem_bytes_for(1));
+    rc = ensure_dynamic_lds(paged_attn_tq4_kernel<TQ, 1>, smem_bytes_for(1), true);
     if (rc) return rc;
     hipLaunchKernelGGL((paged_attn_tq4_kernel<TQ, 1>), grid, dim3(waves_for(1) * 64), smem_bytes_for(1), stream, P);
     rc = (int)hipGetLastError();
@@ -1664,7 +1702,7 @@ static int launch_rows(const warp34_exec* ex, const warp34_kv_layer_layout* layo
     if (P.tok_tile < 1) P.tok_tile = 1;
     P.min_upc = kMinUnitsPerChunk;
     P.max_chunks = force_single ? 1 : choose_max_chunks(ex, batch->total_tokens, num_q_heads, P.tok_tile,
-                                                        layout->local_kv_heads * P.q_subgroups);
+                                                        P.q_subgroups);
     P.part_acc = nullptr;
     P.part_ml = nullptr;
     const long long rows = (long long)batch->total_tokens * num_q_heads;
@@ -1692,7 +1730,7 @@ static int launch_rows(const warp34_exec* ex, const warp34_kv_layer_layout* layo
     hipStream_t stream = (hipStream_t)ex->stream;
     int rc;
     if (balanced_decode_applicable(ex, batch, P.tiles_by_request, force_single)) {
-        const int groups = balanced_groups(kv_subs);
+        const int groups = balanced_groups(P.q_subgroups);
         const size_t prows = bal_partial_row(groups + batch->num_reqs, kv_subs, 0, 0);
         if (partial_bytes((long long)prows, 1) + (size_t)batch->total_tokens * 16 <= ex->scratch_size) {
             P.part_acc = reinterpret_cast<float*>((uintptr_t)ex->scratch_ptr);
@@ -1770,7 +1808,7 @@ static int launch_prefill_tq4(const warp34_exec* ex, const warp34_kv_layer_layou
     const dim3 grid((unsigned)tiles, (unsigned)(layout->local_kv_heads * P.q_subgroups), (unsigned)batch->num_reqs);
     P.rot_q = layout->k_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 ? 1 : 0;
     P.rot_out = layout->v_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 ? 1 : 0;
-    int rc = ensure_dynamic_lds(paged_prefill_tq4_kernel<TQ, KVF>, PfLds<KVF>::kSmem);
+    int rc = ensure_dynamic_lds(paged_prefill_tq4_kernel<TQ, KVF>, PfLds<KVF>::kSmem, true);
     if (rc) return rc;
     hipLaunchKernelGGL((paged_prefill_tq4_kernel<TQ, KVF>), grid, dim3(kPfWaves * 64), PfLds<KVF>::kSmem,
                        (hipStream_t)ex->stream, P);
@@ -1959,7 +1997,9 @@ static int launch_qsa_sparse(const warp34_exec* ex, const void* q, const void* g
     if (want < 1) want = 1;
     const size_t rows = (size_t)num_tokens * local_q_heads;
     const size_t need = rows * (size_t)want * (kHeadDim + 4) * sizeof(float);
-    P.n_splits = (want > 1 && ex->scratch_ptr != 0 && ex->scratch_size >= need) ? (int)want : 1;
+    P.n_splits = (want > 1 && ex->scratch_ptr != 0 && (ex->scratch_ptr & 15u) == 0u && ex->scratch_size >= need)
+                     ? (int)want
+                     : 1;
     if (P.n_splits > 1) {
         P.part_acc = reinterpret_cast<float*>((uintptr_t)ex->scratch_ptr);
         P.part_ml = P.part_acc + rows * P.n_splits * kHeadDim;
@@ -1975,7 +2015,7 @@ static int launch_qsa_sparse(const warp34_exec* ex, const void* q, const void* g
         return (int)hipGetLastError();
     };
     if (form == kFormTq4) {
-        rc = ensure_dynamic_lds(qsa_sparse_tq4_kernel, kQsaSmem);
+        rc = ensure_dynamic_lds(qsa_sparse_tq4_kernel, kQsaSmem, true);
         if (rc) return rc;
         hipLaunchKernelGGL(qsa_sparse_tq4_kernel, grid, dim3(kQsaWaves * 64), kQsaSmem, stream, P);
         rc = (int)hipGetLastError();
@@ -2034,19 +2074,58 @@ extern "C" int warp34_paged_attention_f16_force_kernel_for_test(
     return attention_entry<F16>(ex, layout, batch, q_in, attn_out, num_q_heads, 1);
 }
 
-extern "C" size_t warp34_paged_attention_scratch_bytes(int total_tokens, int num_q_heads, int max_seq_len) {
-    (void)max_seq_len;
+// Scratch that lets a batch split fully, computed the way the launchers compute it.
+// q_group / q_subgroups as in launch_tq4 / launch_rows; local_kv_heads <= 0: not known, take the
+// largest need over all layouts with this many q heads.
+static size_t scratch_bytes_for(int local_kv_heads, int total_tokens, int num_reqs, int num_q_heads,
+                                int max_seq_len, int max_q_len = 0) {
     if (total_tokens <= 0 || num_q_heads <= 0) return 0;
-    int want = kTargetWorkgroups / total_tokens;  // the layout is not known here: one kv head, one q subgroup
+    int q_group = 1, q_subgroups = 1, kv_subs = num_q_heads;  // the bound when the layout is unknown
+    int tok_tile = 16;
+    if (local_kv_heads > 0 && num_q_heads % local_kv_heads == 0) {
+        const int gqa = num_q_heads / local_kv_heads;
+        q_group = gqa;
+        if (q_group > 16) {
+            for (int d = 16; d >= 1; --d)
+                if (gqa % d == 0) {
+                    q_group = d;
+                    break;
+                }
+        }
+        q_subgroups = gqa / q_group;
+        kv_subs = local_kv_heads * q_subgroups;
+        tok_tile = 16 / q_group < 1 ? 1 : 16 / q_group;
+    }
+    const int tiles = (total_tokens + tok_tile - 1) / tok_tile;
+    long long want = kTargetWorkgroupsPerHead / ((long long)tiles * q_subgroups);
     if (want > kMaxChunksCap) want = kMaxChunksCap;
-    if (want < 2) want = 2;
-    size_t bytes = partial_bytes((long long)total_tokens * num_q_heads, want);
-    // balanced decode: (workgroups + requests) partial slots of 16 columns per (kv head, q subgroup);
-    // requests <= total_tokens and subgroups <= num_q_heads bound it without the layout
-    const size_t bal = partial_bytes(((long long)kBalWorkgroups + (long long)total_tokens * num_q_heads) * 16, 1) +
-                       (size_t)total_tokens * 16;  // + the per-token table
-    if (total_tokens >= 2 && bal > bytes) bytes = bal;
+    if (max_seq_len > 0) {
+        const int units = (max_seq_len + kUnit - 1) / kUnit + 1;
+        const int bound = (units + kMinUnitsPerChunk - 1) / kMinUnitsPerChunk;
+        if (bound < want) want = bound;
+    }
+    size_t bytes = want >= 2 ? partial_bytes((long long)total_tokens * num_q_heads, (int)want) : 0;
+    // balanced decode: (shares + requests) partial slots of 16 columns per (kv head, q subgroup)
+    // and the per-token table
+    // (only batches in which no request has more than one tile take it; max_q_len <= 0: not known)
+    if (num_reqs < 0 || num_reqs > total_tokens) num_reqs = total_tokens;
+    if (num_reqs >= 2 && max_q_len <= tok_tile) {
+        const size_t prows = bal_partial_row(balanced_groups(q_subgroups) + num_reqs, kv_subs, 0, 0);
+        const size_t bal = partial_bytes((long long)prows, 1) + (size_t)total_tokens * 16;
+        if (bal > bytes) bytes = bal;
+    }
     return bytes;
+}
+
+extern "C" size_t warp34_paged_attention_scratch_bytes(int total_tokens, int num_q_heads, int max_seq_len) {
+    return scratch_bytes_for(0, total_tokens, -1, num_q_heads, max_seq_len);
+}
+
+extern "C" size_t warp34_paged_attention_scratch_bytes_for_layout(const warp34_kv_layer_layout* layout,
+                                                                  int total_tokens, int num_reqs, int num_q_heads,
+                                                                  int max_seq_len) {
+    if (!layout) return 0;
+    return scratch_bytes_for(layout->local_kv_heads, total_tokens, num_reqs, num_q_heads, max_seq_len);
 }
 
 // op_qsa.cu:1711-1730

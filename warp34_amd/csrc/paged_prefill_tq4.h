@@ -75,7 +75,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     constexpr int kPfDeqBase = M::kDeqBase, kPfRawBase = M::kRawBase, kPfRawBytes = M::kRaw;
     constexpr int kRowB = M::kRowBytes, kRunB = M::kRun;
     extern __shared__ __align__(16) uint8_t smem[];
-    if ((uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem != 0u) __builtin_trap();
+    // (the pair table is addressed absolutely: the dynamic block starts at LDS address 0 because the
+    // kernel has no static LDS, which the host checks before the first launch)
 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
@@ -636,6 +637,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         }
         u4 pb[2];
         u4 pb_lo = {0u, 0u, 0u, 0u};
+        u4 pb_l2[2] = {u4{0u, 0u, 0u, 0u}, u4{0u, 0u, 0u, 0u}};  // TQ4: low-order operands per half
         if constexpr (IS_BF16) {
             // bf16 keeps 8 bits of a probability: the rest goes into a second operand (two MFMAs)
             uint32_t hi[8], lo[8];
@@ -663,7 +665,15 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
 #pragma unroll
                     for (int t = 0; t < 8; ++t) w[t] = p[t] > 0.f ? w[t] : 0.f;
                 }
-                pb[h] = u4{pack_h2(w[0], w[1]), pack_h2(w[2], w[3]), pack_h2(w[4], w[5]), pack_h2(w[6], w[7])};
+                // high and low fp16 operand (split_h2): one rounding of p * d would be shared by the
+                // whole 128-element scale block
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    uint32_t whi, wlo;
+                    split_h2(w[2 * k], w[2 * k + 1], whi, wlo);
+                    pb[h][k] = whi;
+                    pb_l2[h][k] = wlo;
+                }
             }
         }
 #pragma unroll
@@ -678,6 +688,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             for (int j = 0; j < 8; ++j) {
                 o_acc[h][j] = pf_mfma32<IS_BF16>(a[j], __builtin_bit_cast(h8, pb[h]), o_acc[h][j]);
                 if constexpr (IS_BF16) o_acc[h][j] = pf_mfma32<true>(a[j], __builtin_bit_cast(h8, pb_lo), o_acc[h][j]);
+                if constexpr (TQ4F) o_acc[h][j] = pf_mfma32<false>(a[j], __builtin_bit_cast(h8, pb_l2[h]), o_acc[h][j]);
             }
         }
     };

@@ -96,8 +96,8 @@ __device__ __forceinline__ void qsa_finish_row(float (&v)[4], int lane, size_t r
 
 __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const QsaParams P) {
     extern __shared__ __align__(16) uint8_t smem[];
-    // lut_read() addresses the table absolutely
-    if ((uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem != 0u) __builtin_trap();
+    // lut_read() addresses the table absolutely: the dynamic block starts at LDS address 0 because
+    // the kernel has no static LDS (checked on the host before the first launch)
     uint8_t* stage_all = smem + kLutBytes;
 
     const int tid = (int)threadIdx.x;
@@ -368,14 +368,13 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
             vwr[t] = row32[n];
             vw1[t] = row32[17 + n];
         }
-        uint32_t pb[2][4];
+        float p[8];
         {
             float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
             mx = max_over_rows(mx);
             const float m_new = fmaxf(m_run, mx);
             const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
             m_run = m_new;
-            float p[8];
             float psum = 0.f;
 #pragma unroll
             for (int t = 0; t < 8; ++t) p[t] = __builtin_amdgcn_exp2f(sc[t] - m_new);
@@ -392,27 +391,23 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
 #pragma unroll
                     for (int j = 0; j < 8; ++j) o_acc[h][j] *= alpha;
             }
-            float w0[8], w1[8];
-#pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                w0[t] = p[t] * half_lo_to_f32(vd0[t]);
-                w1[t] = p[t] * half_hi_to_f32(vd16[t]);
-            }
-            if (MASKED) {
-#pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    w0[t] = p[t] > 0.f ? w0[t] : 0.f;
-                    w1[t] = p[t] > 0.f ? w1[t] : 0.f;
-                }
-            }
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                pb[0][k] = pack_h2(w0[2 * k], w0[2 * k + 1]);
-                pb[1][k] = pack_h2(w1[2 * k], w1[2 * k + 1]);
-            }
         }
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
+            // probability times the half-row scale of the value row, as a high and a low fp16
+            // operand (split_h2): one rounding would be shared by the whole scale block
+            uint32_t pb_hi[4], pb_lo[4];
+            {
+                float w[8];
+#pragma unroll
+                for (int t = 0; t < 8; ++t) w[t] = p[t] * (h == 0 ? half_lo_to_f32(vd0[t]) : half_hi_to_f32(vd16[t]));
+                if (MASKED) {
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) w[t] = p[t] > 0.f ? w[t] : 0.f;
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) split_h2(w[2 * k], w[2 * k + 1], pb_hi[k], pb_lo[k]);
+            }
             uint32_t lo[4], hi[4];
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
@@ -440,11 +435,15 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
-            const u4 pbv = {pb[h][0], pb[h][1], pb[h][2], pb[h][3]};
+            const u4 ph = {pb_hi[0], pb_hi[1], pb_hi[2], pb_hi[3]};
+            const u4 pl = {pb_lo[0], pb_lo[1], pb_lo[2], pb_lo[3]};
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
+            for (int j = 0; j < 8; ++j) {
                 o_acc[h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a[j]),
-                                                                    __builtin_bit_cast(h8, pbv), o_acc[h][j], 0, 0, 0);
+                                                                    __builtin_bit_cast(h8, ph), o_acc[h][j], 0, 0, 0);
+                o_acc[h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a[j]),
+                                                                    __builtin_bit_cast(h8, pl), o_acc[h][j], 0, 0, 0);
+            }
         }
     };
 
