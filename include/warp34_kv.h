@@ -266,6 +266,21 @@ size_t warp34_paged_attention_scratch_bytes(int total_tokens, int num_q_heads, i
 size_t warp34_paged_attention_scratch_bytes_for_layout(const warp34_kv_layer_layout* layout, int total_tokens,
                                                        int num_reqs, int num_q_heads, int max_seq_len);
 
+/* warp34_paged_attention_bf16 for callers that cannot allocate or provide a workspace (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  The split-K partials go to a WARP34_STATIC_SCRATCH_BYTES array inside the library,
+ * one copy per device, held until the process ends; ex->scratch_ptr / scratch_size are ignored and
+ * nothing is allocated or freed.  A batch that would want more scratch than that
+ * (warp34_paged_attention_scratch_bytes_for_layout) is refused with hipErrorOutOfMemory (2) and
+ * nothing is launched.  Results equal warp34_paged_attention_bf16 with an 8 MiB scratch bit for
+ * bit.  All calls on one device share the array: calls that overlap in time on one device (two
+ * streams) race on it and must be ordered by the caller.  The first call on a device looks up the
+ * array's address; make it outside stream capture. */
+#define WARP34_STATIC_SCRATCH_BYTES (8u << 20)
+int warp34_paged_attention_bf16_static_scratch(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
+                                               const warp34_attention_batch* batch, const void* q_in,
+                                               void* attn_out, int num_q_heads);
+
 /* ------------------------------------------------------------------------------------
  * Runtime shims a standalone harness needs (replace op_init.cu; warp34_cuda.h:135,142-164).
  * ------------------------------------------------------------------------------------ */

@@ -2151,3 +2151,54 @@ extern "C" int warp34_qsa_sparse_paged_attn_hadamard_f16(
                              num_selected_blocks, token_seq_pos, valid_token_mask, out, num_tokens, local_q_heads,
                              select_k_blocks, sm_scale, 1);
 }
+
+// ---- an entry point that allocates nothing -----------------------------------------------------
+// warp34_paged_attention_bf16 with the split-K scratch in a file-scope device array instead of
+// ex->scratch_ptr, for callers that cannot provide (or allocate) a workspace.  Every device the
+// library runs on holds its own copy of the array at its own address; the address is looked up
+// once per device, with that device current, and kept.  The array's NAME is a host-side stand-in
+// and is never passed to a kernel or a runtime call: only the looked-up address is.
+namespace w34 {
+constexpr size_t kStaticScratchBytes = WARP34_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBytes];
+constexpr int kStaticScratchDevices = 64;
+static std::atomic<uintptr_t> g_static_scratch_addr[kStaticScratchDevices];
+
+static int static_scratch_address(uintptr_t* out) {
+    int dev = 0;
+    hipError_t rc = hipGetDevice(&dev);
+    if (rc != hipSuccess) return (int)rc;
+    if (dev < 0 || dev >= kStaticScratchDevices) return (int)hipErrorInvalidDevice;
+    uintptr_t addr = g_static_scratch_addr[dev].load(std::memory_order_acquire);
+    if (addr == 0) {
+        void* sym = nullptr;
+        rc = hipGetSymbolAddress(&sym, HIP_SYMBOL(g_static_scratch));
+        if (rc != hipSuccess) return (int)rc;
+        if (sym == nullptr || ((uintptr_t)sym & 15u) != 0u) return (int)hipErrorInvalidSymbol;
+        addr = (uintptr_t)sym;
+        g_static_scratch_addr[dev].store(addr, std::memory_order_release);
+    }
+    *out = addr;
+    return 0;
+}
+}  // namespace w34
+
+extern "C" int warp34_paged_attention_bf16_static_scratch(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
+                                                          const warp34_attention_batch* batch, const void* q_in,
+                                                          void* attn_out, int num_q_heads) {
+    const int rc = common_checks(ex, layout, batch, q_in, attn_out, num_q_heads);
+    if (rc) return rc;
+    if (num_q_heads <= 0 || batch->total_tokens < 0) return (int)hipErrorInvalidValue;
+    if (!batch->total_tokens) return 0;
+    // a batch that would want more scratch than the array holds is refused, not run with fewer chunks
+    const size_t need = scratch_bytes_for(layout->local_kv_heads, batch->total_tokens, batch->num_reqs, num_q_heads,
+                                          batch->max_seq_len, batch->max_q_len);
+    if (need > kStaticScratchBytes) return (int)hipErrorOutOfMemory;
+    uintptr_t addr = 0;
+    const int arc = static_scratch_address(&addr);
+    if (arc) return arc;
+    warp34_exec own = *ex;
+    own.scratch_ptr = addr;
+    own.scratch_size = kStaticScratchBytes;
+    return attention_entry<BF16>(&own, layout, batch, q_in, attn_out, num_q_heads, 0);
+}
