@@ -52,21 +52,27 @@ typedef float f2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u2v __attribute__((ext_vector_type(2)));
 
-// waves per workgroup: 8 for one N tile (<= 256 VGPRs each), 4 for two N tiles (the second
-// tile's accumulators and operands need the full 512-register budget)
-__host__ __device__ constexpr int waves_for(int nt) { return nt == 1 ? 8 : 4; }
+// waves per workgroup of the TQ4 decode kernel: ten (SIMDs 0 and 1 run three, SIMDs 2 and 3 two),
+// which caps a wave at 168 registers and is what the LDS holds: table + 10 staging areas + the
+// query operand table = 159 232 of 163 840 bytes
+constexpr int kTq4Waves = 8;
+__host__ __device__ constexpr int waves_for(int nt) { return nt == 1 ? kTq4Waves : 4; }
 constexpr int kUnit = 32;             // tokens per wave iteration
 constexpr int kLutBytes = 256 * 256;  // 256 entries x 64 lane replicas x 4 B
 constexpr int kRunBytes = 16 * kTq4RowBytes;  // 16 rows = 2112 B = 132 16-byte pieces
 constexpr int kStageTq4 = 4 * kRunBytes;      // K rows 0-31 then V rows 0-31: 8448 B
-__host__ __device__ constexpr int merge_floats_for(int nt) {
-    return waves_for(nt) * (nt * 16 * 260) + (waves_for(nt) + 1) * nt * 16 * 2;
+__host__ __device__ constexpr int merge_floats_for(int nt) {  // one region of 8 columns per wave
+    return waves_for(nt) * (nt * 8 * 260);
+}
+constexpr int kQopBytes = 16 * 4 * 9 * 16;  // query operand table: 16 columns x 4 k-blocks x 9 operands
+__host__ __device__ constexpr int ml_offset_for(int nt) {  // (m, l) tables of the merge: behind everything the loop uses
+    return kLutBytes + waves_for(nt) * kStageTq4 + kQopBytes;
 }
 __host__ __device__ constexpr int smem_bytes_for(int nt) {
-    const int loop_bytes = kLutBytes + waves_for(nt) * kStageTq4;
-    const int merge_bytes = merge_floats_for(nt) * 4;
-    return (loop_bytes > merge_bytes ? loop_bytes : merge_bytes) + 256;
+    return ml_offset_for(nt) + (waves_for(nt) + 1) * nt * 16 * 2 * 4;
 }
+static_assert(merge_floats_for(1) * 4 <= kLutBytes + waves_for(1) * kStageTq4, "merge regions alias the table and the staging areas only");
+static_assert(smem_bytes_for(1) <= 160 * 1024, "decode LDS budget");
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kNegBig = -1.0e30f;  // "minus infinity" that stays finite under subtraction
 // The table holds fp16(kLutGain * centroid); the gain is divided out of the query (K side)
@@ -75,23 +81,6 @@ constexpr float kNegBig = -1.0e30f;  // "minus infinity" that stays finite under
 // the accuracy of the scores.
 constexpr float kLutGain = 1.908032f;
 constexpr float kLutInvGain = 1.0f / kLutGain;
-
-#ifdef W34_TRACE
-#ifndef W34_TRACE_Z
-#define W34_TRACE_Z 0
-#endif
-__device__ unsigned long long g_trace[64 * 64];
-#define W34_TP(slot)                                                                   \
-    do {                                                                               \
-        if (lane == 0 && (blockIdx.x == 0 || blockIdx.x == 77) && blockIdx.y == 0 && blockIdx.z == W34_TRACE_Z) {  \
-            g_trace[((blockIdx.x ? 8 : 0) + wave) * 64 + (slot)] = __builtin_readcyclecounter(); \
-            if ((slot) == 0) g_trace[((blockIdx.x ? 8 : 0) + wave) * 64 + 63] = wall_clock64(); \
-            if ((slot) == 40) g_trace[((blockIdx.x ? 8 : 0) + wave) * 64 + 62] = wall_clock64(); \
-        }                                                                              \
-    } while (0)
-#else
-#define W34_TP(slot) do {} while (0)
-#endif
 
 struct AttnParams {
     warp34_kv_layer_layout L;
@@ -335,13 +324,102 @@ struct BalItem {
     int u_begin, u_end, n_chunks, slot;
 };
 
+// Tile lookup shared by the kernels that do not split it around other work (see the TQ4
+// decode kernel for the scheme): blockIdx.z counts tiles; request z when no request can have
+// two tiles, a prefix sum over the requests' tile counts otherwise.
+struct TileInfo {
+    bool hit;
+    int req, rq_start, rq_end, seq_after, ctx_before, tile_in_req;
+};
+__device__ __forceinline__ TileInfo locate_tile(const AttnParams& P, int tile_z, int lane) {
+    const warp34_attention_batch& B = P.B;
+    TileInfo t{false, -1, 0, 0, 0, 0, 0};
+    if (P.tiles_by_request) {
+        t.req = tile_z;
+        const int lo = B.query_start_loc[tile_z];
+        const int hi = B.query_start_loc[tile_z + 1];
+        const int sa = B.seq_lens_after[tile_z];
+        const int cb = B.context_lens_before != nullptr ? B.context_lens_before[tile_z] : 0;
+        const int rm = B.valid_req_mask != nullptr ? (int)B.valid_req_mask[tile_z] : 1;
+        t.rq_start = __builtin_amdgcn_readfirstlane(lo);
+        t.rq_end = __builtin_amdgcn_readfirstlane(hi);
+        t.seq_after = __builtin_amdgcn_readfirstlane(sa);
+        t.ctx_before = B.context_lens_before != nullptr ? __builtin_amdgcn_readfirstlane(cb)
+                                                        : t.seq_after - (t.rq_end - t.rq_start);
+        t.hit = __builtin_amdgcn_readfirstlane(rm) != 0 && t.rq_end > t.rq_start;
+        return t;
+    }
+    int tiles_before = 0;
+    for (int base = 0; base < B.num_reqs; base += 64) {
+        const int r = base + lane;
+        const bool inb = r < B.num_reqs;
+        const int lo = inb ? B.query_start_loc[r] : 0;
+        const int hi = inb ? B.query_start_loc[r + 1] : 0;
+        const int sa = inb ? B.seq_lens_after[r] : 0;
+        const int cb = (inb && B.context_lens_before != nullptr) ? B.context_lens_before[r] : 0;
+        const int rm = (inb && B.valid_req_mask != nullptr) ? (int)B.valid_req_mask[r] : 1;
+        const int cnt = hi > lo ? fast_div(hi - lo + P.tok_tile - 1, P.tok_tile) : 0;
+        int incl = cnt;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int up = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += up;
+        }
+        const int first = tiles_before + incl - cnt;
+        const unsigned long long hits = __ballot(cnt > 0 && tile_z >= first && tile_z < first + cnt);
+        if (hits != 0ull) {
+            const int src = __builtin_ctzll(hits);
+            t.req = base + src;
+            t.rq_start = __builtin_amdgcn_readlane(lo, src);
+            t.rq_end = __builtin_amdgcn_readlane(hi, src);
+            t.seq_after = __builtin_amdgcn_readlane(sa, src);
+            t.ctx_before = B.context_lens_before != nullptr ? __builtin_amdgcn_readlane(cb, src)
+                                                            : t.seq_after - (t.rq_end - t.rq_start);
+            t.tile_in_req = tile_z - __builtin_amdgcn_readlane(first, src);
+            t.hit = __builtin_amdgcn_readlane(rm, src) != 0;
+            return t;
+        }
+        tiles_before += __builtin_amdgcn_readlane(incl, 63);
+    }
+    return t;
+}
+
+// LDS-direct loads (gfx950): each active lane's 16 bytes go from global memory straight to LDS at
+// m0 + OFFSET + lane * 16, without passing through registers; the immediate OFFSET is added to
+// the global address as well.  Written as assembly so that
+// the compiler does not know the instruction writes LDS: it would otherwise make every later
+// table read (absolute addresses it cannot tell apart from the staging area) wait for the load
+// unit.  The waits are placed by hand (wait_vm): loads return in order, so "all but the N most
+// recent" is a safe condition whatever other loads the compiler has in flight.
+template <int OFFSET>
+__device__ __forceinline__ void lds_load16(uint32_t voffset, const uint8_t* sbase, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3"
+                 :
+                 : "v"(voffset), "s"(sbase), "s"(lds_addr), "n"(OFFSET)
+                 : "memory");
+}
+// lane L of every row of 16 lanes, in all lanes of that row (one VALU move)
+template <int L>
+__device__ __forceinline__ uint32_t row_bcast(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x150 + L, 0xF, 0xF, true);  // row_newbcast:L
+}
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+__device__ __forceinline__ void wait_lds_reads() { asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory"); }
+
 // The work of one workgroup on one tile.  BAL = false: the tile and the chunk come from
 // blockIdx (grid = chunks x (kv head, q subgroup) x tiles).  BAL = true: they come from `item`
 // (balanced decode: every workgroup owns an equal share of the batch's units).
-template <typename TQ, int NT, bool BAL>
+//
+// LDS: [pair table 64 KB][kTq4Waves staging areas of 8448 B][query operand table 9216 B][(m, l) tables].
+// A staging area holds one 32-token unit as it lies in the pages, written by LDS-direct loads:
+// K rows 0-31, then V rows 0-31, 132 bytes each (four runs of 16 rows = 2112 bytes).
+template <typename TQ, bool BAL>
 __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, const BalItem& item) {
-    constexpr int kWaves = waves_for(NT);
-    uint8_t* stage_all = smem + kLutBytes;  // kWaves * kStageTq4 bytes, reused by prologue/epilogue
+    constexpr int kWaves = kTq4Waves;
+    uint8_t* stage_all = smem + kLutBytes;
 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
@@ -362,15 +440,13 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
     const int q_head_base = kv_head * P.gqa + (kv_sub - kv_head * P.q_subgroups) * P.q_group;
     const int chunk = BAL ? 0 : (int)blockIdx.x;
 
-    W34_TP(0);
-
     // Work that depends on nothing goes first so that it overlaps the request lookup below:
     // the raw query rows of this wave's columns and the table.  The first token of the tile is
     // guessed (exact when every request has a whole number of tiles); a wrong guess is
     // corrected after the lookup.
     const int tok_guess = BAL ? item.rq_start
                               : min(P.tiles_by_request ? tile_z : tile_z * P.tok_tile, B.total_tokens - 1);
-    constexpr int kColsPerWave = (16 * NT + kWaves - 1) / kWaves;
+    constexpr int kColsPerWave = (16 + kWaves - 1) / kWaves;
     uint2 q_raw[kColsPerWave];
     auto load_q = [&](int tokbase) {
 #pragma unroll
@@ -379,7 +455,7 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
             const int t = fast_div(col, P.q_group);
             const int a = col - t * P.q_group;
             q_raw[c] = uint2{0u, 0u};
-            if (col < 16 * NT && tokbase + t < B.total_tokens) {
+            if (col < 16 && tokbase + t < B.total_tokens) {
                 const uint16_t* qrow =
                     P.q + ((size_t)(tokbase + t) * P.num_q_heads + (size_t)(q_head_base + a)) * kHeadDim;
                 q_raw[c] = *reinterpret_cast<const uint2*>(qrow + 4 * lane);
@@ -387,15 +463,12 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         }
     };
     load_q(tok_guess);
-    // per-token validity of this lane's columns
-    bool tok_ok[NT];
+    // validity of the token of this lane's column
+    bool tok_ok;
     auto load_tok_ok = [&](int tokbase) {
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            const int tok = tokbase + fast_div(nt * 16 + n, P.q_group);
-            tok_ok[nt] = tok < B.total_tokens &&
-                         (B.valid_token_mask == nullptr || B.valid_token_mask[min(tok, B.total_tokens - 1)] != 0);
-        }
+        const int tok = tokbase + fast_div(n, P.q_group);
+        tok_ok = tok < B.total_tokens &&
+                 (B.valid_token_mask == nullptr || B.valid_token_mask[min(tok, B.total_tokens - 1)] != 0);
     };
     load_tok_ok(tok_guess);
 
@@ -436,52 +509,26 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         a_cb = B.context_lens_before != nullptr ? B.context_lens_before[req] : 0;
         a_rm = B.valid_req_mask != nullptr ? (int)B.valid_req_mask[req] : 1;
     } else {
-        // lane l examines request base + l; an inclusive prefix sum of the tile counts over the
-        // lanes locates the request that owns tile z (requests are disjoint, ascending ranges
-        // of tokens: op_kv_cache.cu:385-398)
-        int tiles_before = 0;
-        for (int base = 0; base < B.num_reqs; base += 64) {
-            const int r = base + lane;
-            const bool inb = r < B.num_reqs;
-            const int lo = inb ? B.query_start_loc[r] : 0;
-            const int hi = inb ? B.query_start_loc[r + 1] : 0;
-            const int sa = inb ? B.seq_lens_after[r] : 0;
-            const int cb = (inb && B.context_lens_before != nullptr) ? B.context_lens_before[r] : 0;
-            const int rm = (inb && B.valid_req_mask != nullptr) ? (int)B.valid_req_mask[r] : 1;
-            const int cnt = hi > lo ? fast_div(hi - lo + P.tok_tile - 1, P.tok_tile) : 0;
-            int incl = cnt;
-#pragma unroll
-            for (int off = 1; off < 64; off <<= 1) {
-                const int up = __shfl_up(incl, off, 64);
-                if (lane >= off) incl += up;
-            }
-            const int first = tiles_before + incl - cnt;
-            const unsigned long long hits = __ballot(cnt > 0 && tile_z >= first && tile_z < first + cnt);
-            if (hits != 0ull) {
-                const int src = __builtin_ctzll(hits);
-                req = base + src;
-                rq_start = __builtin_amdgcn_readlane(lo, src);
-                rq_end = __builtin_amdgcn_readlane(hi, src);
-                seq_after = __builtin_amdgcn_readlane(sa, src);
-                ctx_before = B.context_lens_before != nullptr ? __builtin_amdgcn_readlane(cb, src)
-                                                              : seq_after - (rq_end - rq_start);
-                tile_in_req = tile_z - __builtin_amdgcn_readlane(first, src);
-                req_hit = __builtin_amdgcn_readlane(rm, src) != 0;
-                break;
-            }
-            tiles_before += __builtin_amdgcn_readlane(incl, 63);
-        }
+        const TileInfo ti = locate_tile(P, tile_z, lane);
+        req = ti.req;
+        rq_start = ti.rq_start;
+        rq_end = ti.rq_end;
+        seq_after = ti.seq_after;
+        ctx_before = ti.ctx_before;
+        tile_in_req = ti.tile_in_req;
+        req_hit = ti.hit;
     }
     {
-        // entry e = (gain*centroid[e & 15], gain*centroid[e >> 4]) as packed fp16, 64 copies
-        constexpr int kThreadsPerEntry = kWaves * 64 / 256;      // 2 or 1
-        constexpr int kBytesPerThread = 256 / kThreadsPerEntry;  // 128 or 256
-        const int e = tid / kThreadsPerEntry;
-        const uint32_t v = pack_h2(kLutGain * centroid_of_code(e & 15), kLutGain * centroid_of_code(e >> 4));
-        u4 vv = {v, v, v, v};
-        u4* dst = reinterpret_cast<u4*>(smem + e * 256 + (tid % kThreadsPerEntry) * kBytesPerThread);
-#pragma unroll
-        for (int k = 0; k < kBytesPerThread / 16; ++k) dst[k] = vv;
+        // entry e = (gain*centroid[e & 15], gain*centroid[e >> 4]) as packed fp16, 64 copies:
+        // 16 KB per pass of 1024 "slots" of 16 bytes each
+        constexpr int kThreads = kWaves * 64;
+        const u4* dummy = nullptr;
+        (void)dummy;
+        for (int slot = tid; slot < kLutBytes / 16; slot += kThreads) {
+            const int e = slot >> 4;  // 16 slots of 16 bytes per entry
+            const uint32_t v = pack_h2(kLutGain * centroid_of_code(e & 15), kLutGain * centroid_of_code(e >> 4));
+            *reinterpret_cast<u4*>(smem + slot * 16) = u4{v, v, v, v};
+        }
     }
 
     if (!BAL && P.tiles_by_request) {
@@ -499,49 +546,27 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         load_tok_ok(tok0);
     }
 
-    // Rotate the query rows now (dead columns are zeroed when they are stored below): the
-    // request lookup and the first KV loads are then not held up behind this wave's VALU work.
-    float q_rot[kColsPerWave][4];
-#pragma unroll
-    for (int c = 0; c < kColsPerWave; ++c) {
-        q_rot[c][0] = TQ::to_f32((uint16_t)(q_raw[c].x & 0xFFFFu));
-        q_rot[c][1] = TQ::to_f32((uint16_t)(q_raw[c].x >> 16));
-        q_rot[c][2] = TQ::to_f32((uint16_t)(q_raw[c].y & 0xFFFFu));
-        q_rot[c][3] = TQ::to_f32((uint16_t)(q_raw[c].y >> 16));
-        // columns of tokens beyond the tile (every second column of a one-token decode tile)
-        // are stored as zeros below: no need to rotate them (wave-uniform branch)
-        const int col = wave + c * kWaves;
-        if (col < 16 * NT && fast_div(col, P.q_group) < rq_end - tok0) {
-#pragma unroll
-            for (int k = 0; k < 4; ++k) q_rot[c][k] = apply_sign(q_rot[c][k], 4 * lane + k);
-            wht256_wave(q_rot[c], lane);
-        }
-    }
-
-    W34_TP(47);
     int tile_tokens = rq_end - tok0;
     if (tile_tokens > P.tok_tile) tile_tokens = P.tok_tile;
 
-    // per-lane column info (one column per N tile)
-    int col_lo[NT], col_hi[NT];
-    bool col_ok[NT];
+    // per-lane column info
+    int col_lo, col_hi;
+    bool col_ok;
     int u_lo = 0x7fffffff, u_hi = -1;  // union of the visible ranges
     int i_lo = 0, i_hi = 0x7fffffff;   // intersection of the visible ranges
-    uint32_t ok_mask[NT];              // bit c: column nt*16+c is live (wave-uniform)
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        const int col = nt * 16 + n;
-        const int t = fast_div(col, P.q_group);
+    uint32_t ok_mask;                  // bit c: column c is live (wave-uniform)
+    {
+        const int t = fast_div(n, P.q_group);
         const int tok = tok0 + t;
-        const bool ok = t < tile_tokens && tok_ok[nt];
+        const bool ok = t < tile_tokens && tok_ok;
         const int q_off = tok - rq_start;
         int mx = (B.mask_mode == WARP34_ATTN_MASK_NONCAUSAL_WINDOW) ? seq_after - 1 : ctx_before + q_off;
         if (mx >= seq_after) mx = seq_after - 1;
         int mn = 0;
         if (B.sliding_window > 0) mn = max(0, ctx_before + q_off - B.sliding_window + 1);
-        col_ok[nt] = ok;
-        col_lo[nt] = ok ? mn : 0;
-        col_hi[nt] = ok ? mx : -1;
+        col_ok = ok;
+        col_lo = ok ? mn : 0;
+        col_hi = ok ? mx : -1;
         if (ok) {
             i_lo = max(i_lo, mn);
             i_hi = min(i_hi, mx);
@@ -550,7 +575,7 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
                 u_hi = max(u_hi, mx);
             }
         }
-        ok_mask[nt] = (uint32_t)(__ballot(ok) & 0xFFFFull);
+        ok_mask = (uint32_t)(__ballot(ok) & 0xFFFFull);
     }
     if (B.valid_token_mask == nullptr && B.sliding_window <= 0) {
         // Common case, no cross-lane traffic: every token of the tile is live, the ranges start
@@ -575,12 +600,7 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
             i_hi = min(i_hi, __shfl_xor(i_hi, off, 64));
         }
     }
-    {
-        uint32_t any = 0;
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) any |= ok_mask[nt];
-        if (any == 0u) return;  // whole tile masked: outputs untouched
-    }
+    if (ok_mask == 0u) return;  // whole tile masked: outputs untouched
     if (u_hi < 0) u_lo = 0;
     u_lo = __builtin_amdgcn_readfirstlane(u_lo);
     u_hi = __builtin_amdgcn_readfirstlane(u_hi);
@@ -601,23 +621,18 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         cu_end = cu_first + g.upc;
         if (cu_end > g.u_first + g.n_units) cu_end = g.u_first + g.n_units;
     }
-    W34_TP(1);
 
     // ---- staging machinery ----------------------------------------------------------------------
     const uint8_t* k_base = reinterpret_cast<const uint8_t*>((uintptr_t)L.k_base) +
                             (size_t)kv_head * L.k_head_stride_bytes;
     const uint8_t* v_base = reinterpret_cast<const uint8_t*>((uintptr_t)L.v_base) +
                             (size_t)kv_head * L.v_head_stride_bytes;
-    uint8_t* stage = stage_all + wave * kStageTq4;  // [K rows 0..31][V rows 0..31], 132 B each
+    const uint32_t stage_addr = (uint32_t)(kLutBytes + wave * kStageTq4);  // LDS byte address (the block starts at 0)
+    uint8_t* stage = stage_all + wave * kStageTq4;
 
-    // A unit is four contiguous runs of 16 rows (2112 B = 132 16-byte pieces): K rows 0-15,
-    // K rows 16-31, V rows 0-15, V rows 16-31.  Pieces 0-127 of every run are two full-wave
-    // loads from a wave-uniform base; the four tails (pieces 128-131) share one load.
-    // The physical page ids of a unit are fetched (scalar loads) one iteration before its data.
     // The physical page ids come from ONE vector load per 64 block-table slots: lane l holds
     // the id of slot slot_base + l, a unit picks its two ids with readlane.  No scalar memory
     // loads remain in the loop (they share the LDS wait counter and would serialise it).
-    u4 pf[9];
     const int32_t* req_blocks = B.block_tables + (size_t)req * B.max_blocks_per_req;
     int slot_base = fast_div(cu_first * kUnit, L.block_size);
     int page_vec;
@@ -627,10 +642,10 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
     };
     // Runs that do not overlap the visible key range, or whose block-table entry is missing,
     // are read from page 0 of the slab instead: every row they deliver is masked, and any
-    // TQ4 bytes dequantise to finite values.  Keeping the loads unconditional lets the
-    // compiler count them statically (s_waitcnt vmcnt(N) instead of vmcnt(0)).
-    auto issue_loads = [&](int unit) {
-        const uint8_t* run_ptr[4];
+    // TQ4 bytes dequantise to finite values.
+    const uint8_t* nk[2];  // run bases of the unit that is loaded next (wave-uniform)
+    const uint8_t* nv[2];
+    auto locate_unit = [&](int unit) {
 #pragma unroll
         for (int gidx = 0; gidx < 2; ++gidx) {
             const int pos = unit * kUnit + 16 * gidx;
@@ -646,415 +661,392 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
             const bool live = pos <= u_hi && pos + 15 >= u_lo && pg >= 0;
             const size_t koff = live ? (size_t)pg * L.k_page_stride_bytes + (size_t)in_page * L.k_token_stride_bytes : 0;
             const size_t voff = live ? (size_t)pg * L.v_page_stride_bytes + (size_t)in_page * L.v_token_stride_bytes : 0;
-            run_ptr[gidx] = k_base + koff;
-            run_ptr[2 + gidx] = v_base + voff;
-        }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            pf[2 * r] = *(global_cu4*)(run_ptr[r] + 16 * lane);
-            pf[2 * r + 1] = *(global_cu4*)(run_ptr[r] + 1024 + 16 * lane);
-        }
-        {
-            const int r = lane >> 2;
-            const uint8_t* base = r == 0 ? run_ptr[0] : r == 1 ? run_ptr[1] : r == 2 ? run_ptr[2] : run_ptr[3];
-            pf[8] = *(global_cu4*)(base + 2048 + 16 * (lane & 3));
+            nk[gidx] = k_base + koff;
+            nv[gidx] = v_base + voff;
         }
     };
-    auto commit_loads = [&]() {
+    // six load instructions per half unit: a 16-row run is 2112 bytes = 132 pieces of 16 bytes, moved
+    // by three instructions of 44 lanes each (the instruction's immediate offset moves the global
+    // AND the LDS address, so the rows arrive contiguous, as they lie in the page)
+    const uint32_t lane16 = (uint32_t)lane * 16u;
+    auto issue_k = [&]() {
+        if (lane < 44) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            *reinterpret_cast<u4*>(stage + r * kRunBytes + 16 * lane) = pf[2 * r];
-            *reinterpret_cast<u4*>(stage + r * kRunBytes + 1024 + 16 * lane) = pf[2 * r + 1];
+            for (int r = 0; r < 2; ++r) {
+                lds_load16<0>(lane16, nk[r], stage_addr + r * kRunBytes);
+                lds_load16<704>(lane16, nk[r], stage_addr + r * kRunBytes);
+                lds_load16<1408>(lane16, nk[r], stage_addr + r * kRunBytes);
+            }
         }
-        if (lane < 16) *reinterpret_cast<u4*>(stage + (lane >> 2) * kRunBytes + 2048 + 16 * (lane & 3)) = pf[8];
     };
+    auto issue_v = [&]() {
+        if (lane < 44) {
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                lds_load16<0>(lane16, nv[r], stage_addr + (2 + r) * kRunBytes);
+                lds_load16<704>(lane16, nv[r], stage_addr + (2 + r) * kRunBytes);
+                lds_load16<1408>(lane16, nv[r], stage_addr + (2 + r) * kRunBytes);
+            }
+        }
+    };
+    constexpr int kLoadsPerHalf = 6;
+
+    // Units are dealt to the waves by a fixed rule, never handed out dynamically: which wave
+    // sums which keys decides the floating-point result, and the output has to be the same bits
+    // on every run and under every page permutation.  The rule deals the units to the four
+    // SIMDs in turn and, inside a SIMD, to its waves in turn (wave w runs on SIMD w mod 4): with
+    // a wave count that is not a multiple of four the SIMDs still get equal shares.
+    const int simd = wave & 3, wslot = wave >> 2;
+    const int simd_waves = (kWaves - simd + 3) / 4;
+    auto nth_unit = [&](int j) -> int { return cu_first + 4 * (wslot + simd_waves * j) + simd; };
 
     // first unit's data goes in flight before the rest of the prologue
-    int unit = cu_first + wave;
+    int unit = nth_unit(0);
     if (slot_base == spec_slot_base) {
         page_vec = spec_vec;
     } else {
         load_page_vec();
     }
-    W34_TP(41);
-    issue_loads(unit);  // harmless for a wave without work: dead runs read page 0
-    W34_TP(42);
+    if (unit < cu_end) {
+        locate_unit(unit);
+        issue_k();
+        issue_v();
+    }
 
-    // ---- prologue: rotated fp16 queries to LDS ---------------------------------------------------
-    // Staged in the (still unused) staging area as [16*NT][264] halves.  All the constant
-    // factors of the scores (softmax scale, log2 e, 1 / table gain) go into Q'.
-    constexpr int kQStride = 264;
-    _Float16* qlds = reinterpret_cast<_Float16*>(stage_all);
+    // ---- prologue: the query operand table ---------------------------------------------------------
+    // B operands of the QK MFMAs, nine per lane (five for the first half-row, four for the second),
+    // in the order the loop reads them: slot (n, b) holds 9 x 16 bytes.  Operand (h, m) of k-block
+    // b pairs with row dword D = tq4_qk_dword(h, m, b); its eight elements (tq4_dword_elem) are
+    // contiguous in the query row: dword D < 16 covers elements 8 D - 4 .. 8 D + 3 (the first four
+    // are scale nibbles for D = 0 and stay zero), dword 16 elements 124 .. 127 and zeros, dword
+    // 17 + k elements 128 + 8 k .. 128 + 8 k + 7.  A lane of the rotating wave holds elements
+    // 4 lane .. 4 lane + 3 of its column, i.e. one half of one operand, and writes it there.
+    // All the constant factors of the scores (softmax scale, log2 e, 1 / table gain) go into Q'.
+    uint8_t* qop = stage_all + kWaves * kStageTq4;
     const float q_scale = B.sm_scale * kLog2e * kLutInvGain;
+    // where this lane's four elements go: operand (k-block, mf) and which half of it
+    int q_kb, q_mf, q_half;
+    {
+        int D, half;
+        if (lane < 32) {
+            D = (lane + 1) >> 1;
+            half = (lane & 1) ? 0 : 1;
+        } else {
+            D = 17 + ((lane - 32) >> 1);
+            half = lane & 1;
+        }
+        const int Dh = D < 17 ? D : D - 17;  // dword inside its half-row
+        const int grp = (Dh >> 2) & 3;       // 4-dword group -> k-block (groups 1 and 2 swapped)
+        q_kb = D == 16 ? 0 : (grp == 1 ? 2 : grp == 2 ? 1 : grp);
+        q_mf = D == 16 ? 4 : (D < 16 ? (Dh & 3) : 5 + (Dh & 3));
+        q_half = half;
+    }
 #pragma unroll
     for (int c = 0; c < kColsPerWave; ++c) {
         const int col = wave + c * kWaves;
-        if (col < 16 * NT) {
-            const bool okc = (ok_mask[(col >> 4) & (NT - 1)] >> (col & 15)) & 1u;
-            const float sc_q = okc ? q_scale : 0.f;
-            uint2 packed;
-            packed.x = pack_h2(q_rot[c][0] * sc_q, q_rot[c][1] * sc_q);
-            packed.y = pack_h2(q_rot[c][2] * sc_q, q_rot[c][3] * sc_q);
-            *reinterpret_cast<uint2*>(qlds + col * kQStride + 4 * lane) = packed;
+        if (col < 16) {  // wave-uniform
+            float q_rot[4];
+            q_rot[0] = TQ::to_f32((uint16_t)(q_raw[c].x & 0xFFFFu));
+            q_rot[1] = TQ::to_f32((uint16_t)(q_raw[c].x >> 16));
+            q_rot[2] = TQ::to_f32((uint16_t)(q_raw[c].y & 0xFFFFu));
+            q_rot[3] = TQ::to_f32((uint16_t)(q_raw[c].y >> 16));
+            const bool okc = (ok_mask >> col) & 1u;
+            uint2 packed = {0u, 0u};
+            if (okc) {  // dead columns stay zero: no need to rotate them
+#pragma unroll
+                for (int k = 0; k < 4; ++k) q_rot[k] = apply_sign(q_rot[k], 4 * lane + k);
+                wht256_wave(q_rot, lane);
+                packed.x = pack_h2(q_rot[0] * q_scale, q_rot[1] * q_scale);
+                packed.y = pack_h2(q_rot[2] * q_scale, q_rot[3] * q_scale);
+            }
+            uint8_t* slot0 = qop + (size_t)(col * 4) * 144;
+            *reinterpret_cast<uint2*>(slot0 + q_kb * 144 + q_mf * 16 + q_half * 8) = packed;
+            // the parts no element maps to: the scale nibbles of dword 0 (k-block 0, operand 0,
+            // first half), the second half of operand 4 in k-block 0, operand 4 of k-blocks 1-3
+            if (lane < 8) {
+                int zkb, zoff;
+                if (lane == 0) {
+                    zkb = 0; zoff = 0;
+                } else if (lane == 1) {
+                    zkb = 0; zoff = 4 * 16 + 8;
+                } else {
+                    zkb = 1 + (lane - 2) / 2; zoff = 4 * 16 + 8 * ((lane - 2) & 1);
+                }
+                *reinterpret_cast<uint2*>(slot0 + zkb * 144 + zoff) = uint2{0u, 0u};
+            }
         }
     }
-    W34_TP(44);
-    __syncthreads();
-    W34_TP(45);
-
-    // B operands of the QK MFMAs: 9 per N tile (5 for the first half-row, 4 for the second).
-    // Operand (h, m) of k-block b pairs with row dword D = tq4_qk_dword(h, m, b); its eight
-    // elements (tq4_dword_elem) are contiguous in the query row, so they are fetched with 64-
-    // and 128-bit reads: dword D < 16 covers elements 8 D - 4 .. 8 D + 3 (the first four are
-    // scale nibbles for D = 0), dword 16 elements 124 .. 127 and two scale nibbles' worth of
-    // zeros, dword 17 + k elements 128 + 8 k .. 128 + 8 k + 7.
-    h8 bq[NT][9];
-    {
-        const int kb = 8 * (b & 1) + 4 * (b >> 1);  // first dword of this k-block
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            const uint8_t* qrow = reinterpret_cast<const uint8_t*>(qlds + (nt * 16 + n) * kQStride);
-#pragma unroll
-            for (int m = 0; m < 4; ++m) {
-                const int D = kb + m;
-                u2v lo = *reinterpret_cast<const u2v*>(qrow + (D > 0 ? 16 * D - 8 : 0));
-                if (D == 0) lo = u2v{0u, 0u};
-                const u2v hi = *reinterpret_cast<const u2v*>(qrow + 16 * D);
-                bq[nt][m] = __builtin_bit_cast(h8, u4{lo[0], lo[1], hi[0], hi[1]});
-            }
-            {
-                u2v lo = *reinterpret_cast<const u2v*>(qrow + 248);
-                if (b != 0) lo = u2v{0u, 0u};
-                bq[nt][4] = __builtin_bit_cast(h8, u4{lo[0], lo[1], 0u, 0u});
-            }
-#pragma unroll
-            for (int m = 0; m < 4; ++m)
-                bq[nt][5 + m] = *reinterpret_cast<const h8*>(qrow + 256 + 16 * (kb + m));
-        }
-    }
-    W34_TP(46);
-    __syncthreads();  // qlds is dead, the staging area may be overwritten; the table is complete
-    W34_TP(2);
+    __syncthreads();  // the pair table and the query operands are complete
 
     // ---- per-wave state -----------------------------------------------------------------------
     const uint32_t lut_lane = (uint32_t)lane << 2;  // byte 0 of every table address
+    const uint8_t* my_qop = qop + (size_t)(n * 4 + b) * 144;
+    h8 bq[9];  // the query operands of this lane stay in registers
+#pragma unroll
+    for (int mf = 0; mf < 9; ++mf) bq[mf] = *reinterpret_cast<const h8*>(my_qop + 16 * mf);
 
-    f4 o_acc[NT][2][8];
-    float m_run[NT], l_run[NT];
+    f4 o_acc[2][8];
+    float m_run = kNegBig, l_run = 0.f;
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        m_run[nt] = kNegBig;
-        l_run[nt] = 0.f;
+    for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int j = 0; j < 8; ++j) o_acc[nt][h][j] = f4{0.f, 0.f, 0.f, 0.f};
-    }
+        for (int j = 0; j < 8; ++j) o_acc[h][j] = f4{0.f, 0.f, 0.f, 0.f};
 
-#ifdef W34_TRACE
-    int trace_it = 0;
-#endif
+    // rows of the staging area: K rows 0-31, then V rows 0-31, 132 bytes each
+    const uint8_t* ka_lo = stage + unit_token(0, n >> 2, n & 3) * kTq4RowBytes;  // A row of sub-tile 0; sub-tile 1: + 8 rows
+    const uint8_t* kt_lo = stage + unit_token(0, b, 0) * kTq4RowBytes;           // token of output row 4b; + 8 s + i rows
+    const uint8_t* vt_lo = kt_lo + 2 * kRunBytes;
+    const uint8_t* kt_n = kt_lo + (n & 3) * kTq4RowBytes;  // the token whose K scales this lane fetches (+ 8 s rows)
+    const uint8_t* vt_n = vt_lo + (8 * ((n >> 2) & 1) + (n & 3)) * kTq4RowBytes;  // ... and V scales: token n & 7
+
     // one 32-token unit.  MASKED = false (wave-uniform) is the interior case: every token of the
     // unit is visible to every live column, so the compares / selects are branched over.
-    auto process_unit = [&](int t0, const bool MASKED) {
-        const uint8_t* k_rows = stage;
-        const uint8_t* v_rows = stage + 2 * kRunBytes;
-
-        // ---- S^T = K Q'^T for the two 16-key sub-tiles ------------------------------------
-        // Phase structure (few, large LDS batches so that one s_waitcnt covers many reads):
-        // all raw K dwords and K scales -> per sub-tile 36 table reads -> 9 MFMAs.
-        float sc[NT][8];
-        uint32_t kw[2][9], ks0[2][4], ks16[2][4];
+    // HAS_NEXT: the wave has another unit, whose two halves are requested as soon as the raw rows of
+    // this unit's halves have been read out of the staging area.
+    auto process_unit = [&](int t0, const bool MASKED, const bool HAS_NEXT) {
+        // ---- raw K dwords and K scales -------------------------------------------------------------
+        wait_vm<kLoadsPerHalf>();  // this unit's K half has landed (its V half may still be in flight)
+        uint32_t kw[2][9], ksc[2][4];
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-            const int arow = unit_token(s, n >> 2, n & 3);  // A row n of sub-tile s
-            const uint32_t* row32 = reinterpret_cast<const uint32_t*>(k_rows + arow * kTq4RowBytes);
+            const uint32_t* row32 = reinterpret_cast<const uint32_t*>(ka_lo + s * 8 * kTq4RowBytes);
 #pragma unroll
             for (int mf = 0; mf < 9; ++mf) kw[s][mf] = row32[tq4_qk_dword(mf < 5 ? 0 : 1, mf < 5 ? mf : mf - 5, b)];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const uint32_t* r32 =
-                    reinterpret_cast<const uint32_t*>(k_rows + unit_token(s, b, i) * kTq4RowBytes);
-                ks0[s][i] = r32[0];
-                ks16[s][i] = r32[16];
-            }
+            // The two scales of token unit_token(s, b, i) in one register, d0 | d1 << 16.  The 16
+            // lanes of a row need the same four tokens: lane n reads token n & 3 and the values
+            // are handed round inside the row.
+            const uint32_t* r32 = reinterpret_cast<const uint32_t*>(kt_n + 8 * s * kTq4RowBytes);
+            const uint32_t mine = __builtin_amdgcn_perm(r32[16], r32[0], 0x07060100u);
+            ksc[s][0] = row_bcast<0>(mine);
+            ksc[s][1] = row_bcast<1>(mine);
+            ksc[s][2] = row_bcast<2>(mine);
+            ksc[s][3] = row_bcast<3>(mine);
         }
-        __builtin_amdgcn_sched_barrier(0);
-#ifdef W34_TRACE
-        if (trace_it < 8) W34_TP(4 + 4 * trace_it + 1);
-#endif
+        wait_lds_reads();
+        if (HAS_NEXT) issue_k();  // nk was located by the caller
+
+        // ---- S^T = K Q'^T for the two 16-key sub-tiles ------------------------------------------
+        // Six batches of three operands (twelve table reads, three MFMAs), software-pipelined: the
+        // table reads of batch k + 1 are requested before the MFMAs of batch k are issued, so the
+        // wave does not sit out the LDS latency of every batch.
+        constexpr int kQkOrder[9] = {0, 5, 1, 6, 2, 7, 3, 8, 4};
+        f4 s_acc[2][2];
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            u4 a[9];
+        for (int s = 0; s < 2; ++s) s_acc[s][0] = s_acc[s][1] = f4{0.f, 0.f, 0.f, 0.f};
+        u4 qa[2][3];
+        auto qk_reads = [&](int bt, u4 (&a)[3]) {
+            const int s = bt / 3;
 #pragma unroll
-            for (int mf = 0; mf < 9; ++mf) {
-                const uint32_t w = kw[s][mf];
-                a[mf][0] = lut_read(w, lut_lane, 0x0c0c0400u);
-                a[mf][1] = lut_read(w, lut_lane, 0x0c0c0500u);
-                a[mf][2] = lut_read(w, lut_lane, 0x0c0c0600u);
-                a[mf][3] = lut_read(w, lut_lane, 0x0c0c0700u);
+            for (int k = 0; k < 3; ++k) {
+                const uint32_t w = kw[s][kQkOrder[3 * (bt % 3) + k]];
+                a[k][0] = lut_read(w, lut_lane, 0x0c0c0400u);
+                a[k][1] = lut_read(w, lut_lane, 0x0c0c0500u);
+                a[k][2] = lut_read(w, lut_lane, 0x0c0c0600u);
+                a[k][3] = lut_read(w, lut_lane, 0x0c0c0700u);
             }
+        };
+        qk_reads(0, qa[0]);
+#pragma unroll
+        for (int bt = 0; bt < 6; ++bt) {
+            if (bt + 1 < 6) qk_reads(bt + 1, qa[(bt + 1) & 1]);
             __builtin_amdgcn_sched_barrier(0);
-            f4 s_acc[NT][2];
+            const int s = bt / 3;
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                s_acc[nt][0] = f4{0.f, 0.f, 0.f, 0.f};
-                s_acc[nt][1] = f4{0.f, 0.f, 0.f, 0.f};
-            }
-#pragma unroll
-            for (int m = 0; m < 5; ++m) {
-                // alternate the two half-row accumulators so consecutive MFMAs are independent
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    if (h == 1 && m == 4) continue;
-                    const int mf = h == 0 ? m : 5 + m;
-                    const h8 av = __builtin_bit_cast(h8, a[mf]);
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) {
-                        s_acc[nt][h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bq[nt][mf], s_acc[nt][h], 0, 0, 0);
-                    }
-                }
-            }
-            // rows 4b+i of the result are tokens unit_token(s, b, i); apply the K scales
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const float d0 = half_lo_to_f32(ks0[s][i]);
-                const float d1 = half_hi_to_f32(ks16[s][i]);
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt) sc[nt][4 * s + i] = d0 * s_acc[nt][0][i] + d1 * s_acc[nt][1][i];
+            for (int k = 0; k < 3; ++k) {
+                const int mf = kQkOrder[3 * (bt % 3) + k];
+                const int h = mf < 5 ? 0 : 1;
+                s_acc[s][h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, qa[bt & 1][k]), bq[mf],
+                                                                    s_acc[s][h], 0, 0, 0);
             }
         }
+        // rows 4b+i of the result are tokens unit_token(s, b, i); apply the K scales
+        float sc[8];
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                sc[4 * s + i] = half_lo_to_f32(ksc[s][i]) * s_acc[s][0][i] + half_hi_to_f32(ksc[s][i]) * s_acc[s][1][i];
         if (MASKED) {
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
                 const int pos = t0 + unit_token(t >> 2, b, t & 3);
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    const bool vis = col_ok[nt] && pos >= col_lo[nt] && pos <= col_hi[nt];
-                    sc[nt][t] = vis ? sc[nt][t] : kNegBig;
-                }
+                const bool vis = col_ok && pos >= col_lo && pos <= col_hi;
+                sc[t] = vis ? sc[t] : kNegBig;
             }
         }
 
         // ---- raw V dwords of this lane's 8 tokens ------------------------------------------
-        uint32_t vd0[8], vd16[8], vwr[8], vw1[8];
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            const int trow = unit_token(t >> 2, b, t & 3);
-            const uint32_t* row32 = reinterpret_cast<const uint32_t*>(v_rows + trow * kTq4RowBytes);
-            vd0[t] = row32[0];
-            vd16[t] = row32[16];
-            vwr[t] = row32[n];  // n == 0 re-reads dword 0
-            vw1[t] = row32[17 + n];
+        if (HAS_NEXT) {
+            wait_vm<kLoadsPerHalf>();  // the V half has landed; the next K half may be in flight
+        } else {
+            wait_vm<0>();
         }
+        // per token: the two scales (d0 | d1 << 16), the dword of the first half-row that holds this
+        // lane's codes (dword n; for n = 0 codes 0-3 and 124-127 are put together from dwords 0 and
+        // 16) and the dword of the second half-row
+        uint32_t vsc[8], vw[2][8];
+        {
+            // lane n reads dwords 0 and 16 of token n & 7 (of the eight this row of lanes works on)
+            // and hands the scale pair and the n = 0 column round inside the row
+            const uint32_t* r32 = reinterpret_cast<const uint32_t*>(vt_n);
+            const uint32_t d0 = r32[0], d16 = r32[16];
+            const uint32_t mine_sc = __builtin_amdgcn_perm(d16, d0, 0x07060100u);
+            const uint32_t mine_c0 = __builtin_amdgcn_alignbit(d16, d0, 16);
+            uint32_t c0[8];
+            vsc[0] = row_bcast<0>(mine_sc); c0[0] = row_bcast<0>(mine_c0);
+            vsc[1] = row_bcast<1>(mine_sc); c0[1] = row_bcast<1>(mine_c0);
+            vsc[2] = row_bcast<2>(mine_sc); c0[2] = row_bcast<2>(mine_c0);
+            vsc[3] = row_bcast<3>(mine_sc); c0[3] = row_bcast<3>(mine_c0);
+            vsc[4] = row_bcast<4>(mine_sc); c0[4] = row_bcast<4>(mine_c0);
+            vsc[5] = row_bcast<5>(mine_sc); c0[5] = row_bcast<5>(mine_c0);
+            vsc[6] = row_bcast<6>(mine_sc); c0[6] = row_bcast<6>(mine_c0);
+            vsc[7] = row_bcast<7>(mine_sc); c0[7] = row_bcast<7>(mine_c0);
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const uint32_t* row32 = reinterpret_cast<const uint32_t*>(vt_lo + (8 * (t >> 2) + (t & 3)) * kTq4RowBytes);
+                vw[0][t] = n == 0 ? c0[t] : row32[n];  // (lane n = 0 reads dword 0 and drops it)
+                vw[1][t] = row32[17 + n];
+            }
+        }
+        wait_lds_reads();
+        if (HAS_NEXT) issue_v();
 
         // ---- online softmax (log2 domain), per lane = per query column --------------------
-        float p[NT][8];
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            float mx = fmaxf(fmaxf(fmaxf(sc[nt][0], sc[nt][1]), fmaxf(sc[nt][2], sc[nt][3])),
-                             fmaxf(fmaxf(sc[nt][4], sc[nt][5]), fmaxf(sc[nt][6], sc[nt][7])));
+        float p[8];
+        {
+            float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
             mx = max_over_rows(mx);
-            const float m_new = fmaxf(m_run[nt], mx);
-            const float alpha = __builtin_amdgcn_exp2f(m_run[nt] - m_new);
-            m_run[nt] = m_new;
+            const float m_new = fmaxf(m_run, mx);
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            m_run = m_new;
             float psum = 0.f;
             // (the MASKED tests sit outside the unrolled loops: one wave-uniform branch per block
             // instead of one per element, and the eight exponentials can overlap)
 #pragma unroll
-            for (int t = 0; t < 8; ++t) p[nt][t] = __builtin_amdgcn_exp2f(sc[nt][t] - m_new);
+            for (int t = 0; t < 8; ++t) p[t] = __builtin_amdgcn_exp2f(sc[t] - m_new);
             if (MASKED) {
 #pragma unroll
-                for (int t = 0; t < 8; ++t) p[nt][t] = sc[nt][t] > 0.5f * kNegBig ? p[nt][t] : 0.f;
+                for (int t = 0; t < 8; ++t) p[t] = sc[t] > 0.5f * kNegBig ? p[t] : 0.f;
             }
 #pragma unroll
-            for (int t = 0; t < 8; ++t) psum += p[nt][t];
-            l_run[nt] = l_run[nt] * alpha + psum;
+            for (int t = 0; t < 8; ++t) psum += p[t];
+            l_run = l_run * alpha + psum;
             if (__ballot(alpha != 1.0f) != 0ull) {
 #pragma unroll
                 for (int h = 0; h < 2; ++h)
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) o_acc[nt][h][j] *= alpha;
+                    for (int j = 0; j < 8; ++j) o_acc[h][j] *= alpha;
             }
         }
 
-#ifdef W34_TRACE
-        if (trace_it < 8) W34_TP(4 + 4 * trace_it + 2);
-#endif
         // ---- O^T += V^T P^T ------------------------------------------------------------------
+        // weights of each half: probability times the half-row scale of the value row, as a high
+        // and a low fp16 operand (split_h2)
+        u4 ph[2], pl[2];
+        uint32_t lo[2][4], hi[2][4];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            // weights of this half: probability times the half-row scale of the value row, as a
-            // high and a low fp16 operand (split_h2)
-            uint32_t pb_hi[NT][4], pb_lo[NT][4];
+            float w[8];
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                float w[8];
+            for (int t = 0; t < 8; ++t) w[t] = p[t] * (h == 0 ? half_lo_to_f32(vsc[t]) : half_hi_to_f32(vsc[t]));
+            if (MASKED) {
+                // masked tokens have p == 0; select instead of multiply so that a garbage scale
+                // (rows beyond the sequence end) cannot inject NaN
 #pragma unroll
-                for (int t = 0; t < 8; ++t)
-                    w[t] = p[nt][t] * (h == 0 ? half_lo_to_f32(vd0[t]) : half_hi_to_f32(vd16[t]));
-                if (MASKED) {
-                    // masked tokens have p == 0; select instead of multiply so that a garbage scale
-                    // (rows beyond the sequence end) cannot inject NaN
-#pragma unroll
-                    for (int t = 0; t < 8; ++t) w[t] = p[nt][t] > 0.f ? w[t] : 0.f;
-                }
-#pragma unroll
-                for (int k = 0; k < 4; ++k) split_h2(w[2 * k], w[2 * k + 1], pb_hi[nt][k], pb_lo[nt][k]);
+                for (int t = 0; t < 8; ++t) w[t] = p[t] > 0.f ? w[t] : 0.f;
             }
-            uint32_t lo[4], hi[4];
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                uint32_t wa, wb;
-                if (h == 0) {
-                    const uint32_t xa = __builtin_amdgcn_alignbit(vd16[2 * k], vd0[2 * k], 16);
-                    const uint32_t xb = __builtin_amdgcn_alignbit(vd16[2 * k + 1], vd0[2 * k + 1], 16);
-                    wa = n == 0 ? xa : vwr[2 * k];
-                    wb = n == 0 ? xb : vwr[2 * k + 1];
-                } else {
-                    wa = vw1[2 * k];
-                    wb = vw1[2 * k + 1];
-                }
+                uint32_t whi, wlo;
+                split_h2(w[2 * k], w[2 * k + 1], whi, wlo);
+                ph[h][k] = whi;
+                pl[h][k] = wlo;
+                const uint32_t wa = vw[h][2 * k], wb = vw[h][2 * k + 1];
                 // byte q of lo / hi = (nibble 2q / 2q+1 of token a) | (same nibble of token b) << 4
-                lo[k] = (wa & 0x0F0F0F0Fu) | ((wb << 4) & 0xF0F0F0F0u);
-                hi[k] = ((wa >> 4) & 0x0F0F0F0Fu) | (wb & 0xF0F0F0F0u);
+                lo[h][k] = (wa & 0x0F0F0F0Fu) | ((wb << 4) & 0xF0F0F0F0u);
+                hi[h][k] = ((wa >> 4) & 0x0F0F0F0Fu) | (wb & 0xF0F0F0F0u);
             }
-            u4 a[8];
+        }
+        // four batches of four value tiles (16 table reads, eight MFMAs), pipelined like the QK batches
+        u4 va[2][4];
+        auto pv_reads = [&](int bt, u4 (&a)[4]) {
+            const int h = bt >> 1;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
+            for (int jj = 0; jj < 4; ++jj) {
+                const int j = 4 * (bt & 1) + jj;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    const uint32_t src = (j & 1) ? hi[k] : lo[k];
+                    const uint32_t src = (j & 1) ? hi[h][k] : lo[h][k];
                     const uint32_t sel = 0x0c0c0400u + ((uint32_t)(j >> 1) << 8);
-                    a[j][k] = lut_read(src, lut_lane, sel);
+                    a[jj][k] = lut_read(src, lut_lane, sel);
                 }
             }
+        };
+        pv_reads(0, va[0]);
+#pragma unroll
+        for (int bt = 0; bt < 4; ++bt) {
+            if (bt + 1 < 4) pv_reads(bt + 1, va[(bt + 1) & 1]);
             __builtin_amdgcn_sched_barrier(0);
+            const int h = bt >> 1;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const h8 av = __builtin_bit_cast(h8, a[j]);
+            for (int jj = 0; jj < 4; ++jj) {
+                const int j = 4 * (bt & 1) + jj;
+                const h8 av = __builtin_bit_cast(h8, va[bt & 1][jj]);
+                o_acc[h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, __builtin_bit_cast(h8, ph[h]), o_acc[h][j], 0, 0, 0);
+            }
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    const u4 ph = {pb_hi[nt][0], pb_hi[nt][1], pb_hi[nt][2], pb_hi[nt][3]};
-                    const u4 pl = {pb_lo[nt][0], pb_lo[nt][1], pb_lo[nt][2], pb_lo[nt][3]};
-                    o_acc[nt][h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                        av, __builtin_bit_cast(h8, ph), o_acc[nt][h][j], 0, 0, 0);
-                    o_acc[nt][h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                        av, __builtin_bit_cast(h8, pl), o_acc[nt][h][j], 0, 0, 0);
-                }
+            for (int jj = 0; jj < 4; ++jj) {
+                const int j = 4 * (bt & 1) + jj;
+                const h8 av = __builtin_bit_cast(h8, va[bt & 1][jj]);
+                o_acc[h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, __builtin_bit_cast(h8, pl[h]), o_acc[h][j], 0, 0, 0);
             }
         }
     };
 
-
-    // Units are dealt to the waves by a fixed rule, never handed out dynamically: which wave
-    // sums which keys decides the floating-point result, and the output has to be the same bits
-    // on every run and under every page permutation.  The rule is round robin with one extra
-    // unit for waves 0-3 after every eight rounds (68 units: nine each for waves 0-3, eight each
-    // for waves 4-7): the SIMD serves its older wave first, which makes waves 0-3 about 10 %
-    // faster per unit, and an even deal leaves them waiting at the merge.
-    auto nth_unit = [&](int j) -> int {  // j-th unit of this wave
-        if constexpr (kWaves == 8) {
-            if (wave < 4) {
-                const int g = j / 9, k = j - 9 * g;
-                return cu_first + 68 * g + (k < 8 ? 8 * k + wave : 64 + wave);
-            }
-            return cu_first + 68 * (j >> 3) + 8 * (j & 7) + wave;
-        } else {
-            return cu_first + j * kWaves + wave;
-        }
-    };
     for (int j = 0; unit < cu_end; ++j) {
-        // the two waves of a SIMD take turns at the higher issue priority, unit by unit
-        if constexpr (kWaves == 8) {
-            if ((j + (wave >> 2)) & 1) {
-                __builtin_amdgcn_s_setprio(1);
-            } else {
-                __builtin_amdgcn_s_setprio(0);
-            }
-        }
-        commit_loads();
-#ifdef W34_TRACE
-        if (trace_it < 8) W34_TP(4 + 4 * trace_it);
-#endif
         const int next_unit = nth_unit(j + 1);
-        if (next_unit < cu_end) issue_loads(next_unit);
+        const bool has_next = next_unit < cu_end;
+        if (has_next) locate_unit(next_unit);
         const int t0 = unit * kUnit;
-        process_unit(t0, !(t0 >= i_lo && t0 + kUnit - 1 <= i_hi));
-#ifdef W34_TRACE
-        if (trace_it < 8) W34_TP(4 + 4 * trace_it + 3);
-        ++trace_it;
-#endif
+        const bool masked = !(t0 >= i_lo && t0 + kUnit - 1 <= i_hi);
+        process_unit(t0, masked, has_next);
         unit = next_unit;
     }
-    __builtin_amdgcn_s_setprio(0);
-    W34_TP(36);
+    wait_vm<0>();  // nothing of this wave may still be on its way into LDS when the areas are reused
 
     // ---- combine the per-lane partial sums of l over the four k-block lanes of a column ------
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) l_run[nt] = sum_over_rows(l_run[nt]);
+    l_run = sum_over_rows(l_run);
 
     // ---- merge the waves' states through LDS ---------------------------------------------------
-    // Every wave publishes (m, l), rescales its O by 2^(m - m_tot) and stores it in its own
-    // region; then the waves split the columns and add the regions up in wave order.
+    // Every wave publishes (m, l); then, for each half of the 16 columns that has a live column,
+    // the waves store their O of those columns, rescaled by 2^(m - m_tot), in their own region, and
+    // waves 0-7 each add the regions of one column up in wave order.  (Two passes because ten
+    // regions of sixteen columns do not fit the LDS; a decode tile has live columns in one half only.)
     // Region layout: column stride 260 dwords; inside a column the four values a lane holds for
     // one MFMA result (rows 4b..4b+3 of (h, j)) are contiguous at ((h*8 + j)*4 + b)*4, so a
     // lane stores them with one 128-bit write, and the 8 lanes of a write pass (8 columns)
     // start 4 banks apart.
     constexpr int kColStride = 260;
-    constexpr int kRegion = NT * 16 * kColStride;
+    constexpr int kRegion = 8 * kColStride;
     float* xbuf = reinterpret_cast<float*>(smem);
-    float* mlbuf = xbuf + kWaves * kRegion;  // [kWaves][NT*16][2], behind the table + staging areas
-    static_assert(kWaves * kRegion + (kWaves + 1) * NT * 16 * 2 == merge_floats_for(NT), "merge layout");
-    static_assert(smem_bytes_for(NT) >= merge_floats_for(NT) * 4, "merge buffer must fit");
-    static_assert(kWaves * kRegion * 4 >= kLutBytes + kWaves * kStageTq4, "(m, l) table must not alias live LDS");
+    // [kWaves][16][2], then (m_tot, l_tot)[16]: in an area of its own, a wave publishes its state
+    // while others are still in their loops
+    float* mlbuf = reinterpret_cast<float*>(smem + ml_offset_for(1));
+    static_assert(kWaves * kRegion == merge_floats_for(1), "merge layout");
     if (b == 0) {
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            mlbuf[(wave * NT * 16 + nt * 16 + n) * 2 + 0] = m_run[nt];
-            mlbuf[(wave * NT * 16 + nt * 16 + n) * 2 + 1] = l_run[nt];
-        }
+        mlbuf[(wave * 16 + n) * 2 + 0] = m_run;
+        mlbuf[(wave * 16 + n) * 2 + 1] = l_run;
     }
-    W34_TP(49);
     __syncthreads();  // every wave is done with the table and with its staging area
-    W34_TP(50);
-    float m_tot[NT], l_tot[NT];
+    float m_tot = kNegBig, l_tot = 0.f;
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        float mt = kNegBig;
+    for (int w = 0; w < kWaves; ++w) m_tot = fmaxf(m_tot, mlbuf[(w * 16 + n) * 2]);
 #pragma unroll
-        for (int w = 0; w < kWaves; ++w) mt = fmaxf(mt, mlbuf[(w * NT * 16 + nt * 16 + n) * 2]);
-        float lt = 0.f;
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w)
-            lt += mlbuf[(w * NT * 16 + nt * 16 + n) * 2 + 1] *
-                  __builtin_amdgcn_exp2f(mlbuf[(w * NT * 16 + nt * 16 + n) * 2] - mt);
-        m_tot[nt] = mt;
-        l_tot[nt] = lt;
-        const float wgt = __builtin_amdgcn_exp2f(m_run[nt] - mt);
-        float* c = xbuf + wave * kRegion + (nt * 16 + n) * kColStride;
-        if (col_ok[nt]) {  // dead columns are never read back
-#pragma unroll
-            for (int h = 0; h < 2; ++h)
-#pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    *reinterpret_cast<f4*>(c + ((h * 8 + j) * 4 + b) * 4) = o_acc[nt][h][j] * wgt;
-        }
-    }
-    // (m_tot, l_tot) of every column for the epilogue, read back by column below
-    float* mltot = mlbuf + kWaves * NT * 16 * 2;
-    if (wave == 0 && b == 0) {
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            mltot[(nt * 16 + n) * 2 + 0] = m_tot[nt];
-            mltot[(nt * 16 + n) * 2 + 1] = l_tot[nt];
-        }
-    }
-    W34_TP(51);
-    __syncthreads();
-    W34_TP(37);
+    for (int w = 0; w < kWaves; ++w)
+        l_tot += mlbuf[(w * 16 + n) * 2 + 1] * __builtin_amdgcn_exp2f(mlbuf[(w * 16 + n) * 2] - m_tot);
+    const float wgt = __builtin_amdgcn_exp2f(m_run - m_tot);
+    float* mltot = mlbuf + kWaves * 16 * 2;
 
-    // ---- epilogue: per column, add the regions, then store the partial or finish the row -------
     int merge_slot[4];  // region slot of element 4*lane + k (inverse of tq4_pv_elem)
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
@@ -1071,54 +1063,71 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         }
         merge_slot[k] = ((h * 8 + j) * 4 + (r >> 2)) * 4 + (r & 3);
     }
-    for (int col = wave; col < 16 * NT; col += kWaves) {
-        const int t = fast_div(col, P.q_group);
-        const int a = col - t * P.q_group;
-        if (!((ok_mask[col >> 4] >> (col & 15)) & 1u)) continue;
-        const size_t row = (size_t)(tok0 + t) * P.num_q_heads + (size_t)(q_head_base + a);
-        float v[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+    for (int half = 0; half < 2; ++half) {
+        if (((ok_mask >> (8 * half)) & 0xFFu) == 0u) continue;  // the same in every wave
+        if (half == 1 && (ok_mask & 0xFFu) != 0u) __syncthreads();  // the first pass has read the regions
+        if ((n >> 3) == half && col_ok) {  // dead columns are never read back
+            float* c = xbuf + wave * kRegion + (n & 7) * kColStride;
 #pragma unroll
-        for (int w = 0; w < kWaves; ++w) {
-            // element e = 4*lane + k is value (h, j, row r) with e = tq4_pv_elem(h, j, r)
-            const float* c = xbuf + w * kRegion + col * kColStride;
+            for (int h = 0; h < 2; ++h)
 #pragma unroll
-            for (int k = 0; k < 4; ++k) v[k] += c[merge_slot[k]];
-        }
-        const float m_col = mltot[col * 2 + 0];
-        const float l_col = mltot[col * 2 + 1];
-        if (BAL ? item.n_chunks > 1 : P.max_chunks > 1) {
-            // un-normalised, rotated, still carrying the table gain; the merge kernel finishes
-            const size_t prow = BAL ? bal_partial_row(item.slot, (int)gridDim.y, kv_sub, col)
-                                    : row * P.max_chunks + chunk;
-            float* dst = P.part_acc + prow * kHeadDim;
-            *reinterpret_cast<f4*>(dst + 4 * lane) = f4{v[0], v[1], v[2], v[3]};
-            if (lane == 0) {
-                // (m, l, number of chunks of this row, -): one record per chunk, every record
-                // carries the count so the merge needs no dependent load
-                *reinterpret_cast<f4*>(P.part_ml + prow * 4) = f4{m_col, l_col, (float)g.n_chunks, 0.f};
+                for (int j = 0; j < 8; ++j) *reinterpret_cast<f4*>(c + ((h * 8 + j) * 4 + b) * 4) = o_acc[h][j] * wgt;
+            if (wave == 0 && b == 0) {
+                mltot[n * 2 + 0] = m_tot;
+                mltot[n * 2 + 1] = l_tot;
             }
-        } else {
-            const float inv = l_col > 0.f ? kLutInvGain / l_col : 0.f;
+        }
+        __syncthreads();
+        const int col = 8 * half + wave;
+        if (wave < 8 && ((ok_mask >> col) & 1u)) {
+            const int t = fast_div(col, P.q_group);
+            const int a = col - t * P.q_group;
+            const size_t row = (size_t)(tok0 + t) * P.num_q_heads + (size_t)(q_head_base + a);
+            float v[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int k = 0; k < 4; ++k) v[k] *= inv;
-            wht256_wave(v, lane);
+            for (int w = 0; w < kWaves; ++w) {
+                // element e = 4*lane + k is value (h, j, row r) with e = tq4_pv_elem(h, j, r)
+                const float* c = xbuf + w * kRegion + wave * kColStride;
 #pragma unroll
-            for (int k = 0; k < 4; ++k) v[k] = apply_sign(v[k], 4 * lane + k);
-            uint2 o;
-            o.x = (uint32_t)TQ::from_f32(v[0]) | ((uint32_t)TQ::from_f32(v[1]) << 16);
-            o.y = (uint32_t)TQ::from_f32(v[2]) | ((uint32_t)TQ::from_f32(v[3]) << 16);
-            *reinterpret_cast<uint2*>(P.out + row * kHeadDim + 4 * lane) = o;
+                for (int k = 0; k < 4; ++k) v[k] += c[merge_slot[k]];
+            }
+            const float m_col = mltot[col * 2 + 0];
+            const float l_col = mltot[col * 2 + 1];
+            if (BAL ? item.n_chunks > 1 : P.max_chunks > 1) {
+                // un-normalised, rotated, still carrying the table gain; the merge kernel finishes
+                const size_t prow = BAL ? bal_partial_row(item.slot, (int)gridDim.y, kv_sub, col)
+                                        : row * P.max_chunks + chunk;
+                float* dst = P.part_acc + prow * kHeadDim;
+                *reinterpret_cast<f4*>(dst + 4 * lane) = f4{v[0], v[1], v[2], v[3]};
+                if (lane == 0) {
+                    // (m, l, number of chunks of this row, -): one record per chunk, every record
+                    // carries the count so the merge needs no dependent load
+                    *reinterpret_cast<f4*>(P.part_ml + prow * 4) = f4{m_col, l_col, (float)g.n_chunks, 0.f};
+                }
+            } else {
+                const float inv = l_col > 0.f ? kLutInvGain / l_col : 0.f;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) v[k] *= inv;
+                wht256_wave(v, lane);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) v[k] = apply_sign(v[k], 4 * lane + k);
+                uint2 o;
+                o.x = (uint32_t)TQ::from_f32(v[0]) | ((uint32_t)TQ::from_f32(v[1]) << 16);
+                o.y = (uint32_t)TQ::from_f32(v[2]) | ((uint32_t)TQ::from_f32(v[3]) << 16);
+                *reinterpret_cast<uint2*>(P.out + row * kHeadDim + 4 * lane) = o;
+            }
         }
     }
-    W34_TP(40);
 }
 
 template <typename TQ, int NT>
-__global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(const AttnParams P) {
+__global__ __launch_bounds__(kTq4Waves * 64, 1) void paged_attn_tq4_kernel(const AttnParams P) {
+    static_assert(NT == 1, "one 16-column tile per workgroup");
     extern __shared__ __align__(16) uint8_t smem[];
     // lut_read() addresses the table absolutely: the dynamic block starts at LDS address 0 because
     // the kernel has no static LDS (checked on the host before the first launch)
-    tq4_tile<TQ, NT, false>(P, smem, BalItem{});
+    tq4_tile<TQ, false>(P, smem, BalItem{});
 }
 
 // Balanced decode: grid = (groups, kv head x q subgroup).  Every wave computes the plan (the
@@ -1127,10 +1136,6 @@ __global__ __launch_bounds__(waves_for(NT) * 64, 1) void paged_attn_tq4_kernel(c
 template <typename TileFn>
 __device__ __forceinline__ void bal_for_each_piece(const AttnParams& P, TileFn&& tile) {
     const int lane = (int)threadIdx.x & 63;
-#ifdef W34_TRACE
-    const int wave = (int)threadIdx.x >> 6;
-#endif
-    W34_TP(60);
     const int num_reqs = P.B.num_reqs;
     // the first 64 requests are loaded once: their lane values serve the total and the search for
     // the first piece (most workgroups have exactly one piece, most batches at most 64 requests)
@@ -1167,7 +1172,6 @@ __device__ __forceinline__ void bal_for_each_piece(const AttnParams& P, TileFn&&
     int base = 0, before = 0, taken = 0;  // group, units before it, pieces of it already done
     BalItem it{};
     int piece_end = 0;
-    W34_TP(59);
     // next piece inside the group whose lane values are (q, incl); false: the group has none left
     auto scan_group = [&](const BalReq& q, int incl) -> bool {
         const int start = before + incl - q.units;  // of the real units, behind the charge
@@ -1215,13 +1219,12 @@ __device__ __forceinline__ void bal_for_each_piece(const AttnParams& P, TileFn&&
         __syncthreads();  // the tile's merge regions alias what the next piece sets up
         have = find_next();
     }
-    W34_TP(61);
 }
 
 template <typename TQ>
-__global__ __launch_bounds__(waves_for(1) * 64, 1) void paged_attn_tq4_balanced_kernel(const AttnParams P) {
+__global__ __launch_bounds__(kTq4Waves * 64, 1) void paged_attn_tq4_balanced_kernel(const AttnParams P) {
     extern __shared__ __align__(16) uint8_t smem[];
-    bal_for_each_piece(P, [&](const BalItem& it) { tq4_tile<TQ, 1, true>(P, smem, it); });
+    bal_for_each_piece(P, [&](const BalItem& it) { tq4_tile<TQ, true>(P, smem, it); });
 }
 
 // Merge for the balanced decode kernel: one workgroup of 1024 threads per (token, q head) row.
@@ -1308,12 +1311,6 @@ __global__ __launch_bounds__(1024) void balanced_merge_kernel(const AttnParams P
     ob.y = (uint32_t)TQ::from_f32(o[2]) | ((uint32_t)TQ::from_f32(o[3]) << 16);
     *reinterpret_cast<uint2*>(P.out + (size_t)row * kHeadDim + 4 * lane) = ob;
 }
-
-#ifdef W34_TRACE
-extern "C" int warp34_debug_read_trace(unsigned long long* dst) {
-    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_trace), sizeof(unsigned long long) * 64 * 64);
-}
-#endif
 
 // Merge of the split-K partials (op_paged_attn.cu:1132-1218): m_tot = max m_s,
 // w_s = 2^(m_s - m_tot), out = sum acc_s w_s / sum l_s w_s, then one inverse rotation.
@@ -1425,66 +1422,6 @@ __global__ __launch_bounds__(1024) void split_merge_kernel(const float* part_acc
     ob.x = (uint32_t)TQ::from_f32(o[0]) | ((uint32_t)TQ::from_f32(o[1]) << 16);
     ob.y = (uint32_t)TQ::from_f32(o[2]) | ((uint32_t)TQ::from_f32(o[3]) << 16);
     *reinterpret_cast<uint2*>(P.out + (size_t)row * kHeadDim + 4 * lane) = ob;
-}
-
-// Tile lookup shared by the kernels that do not split it around other work (see the TQ4
-// decode kernel for the scheme): blockIdx.z counts tiles; request z when no request can have
-// two tiles, a prefix sum over the requests' tile counts otherwise.
-struct TileInfo {
-    bool hit;
-    int req, rq_start, rq_end, seq_after, ctx_before, tile_in_req;
-};
-__device__ __forceinline__ TileInfo locate_tile(const AttnParams& P, int tile_z, int lane) {
-    const warp34_attention_batch& B = P.B;
-    TileInfo t{false, -1, 0, 0, 0, 0, 0};
-    if (P.tiles_by_request) {
-        t.req = tile_z;
-        const int lo = B.query_start_loc[tile_z];
-        const int hi = B.query_start_loc[tile_z + 1];
-        const int sa = B.seq_lens_after[tile_z];
-        const int cb = B.context_lens_before != nullptr ? B.context_lens_before[tile_z] : 0;
-        const int rm = B.valid_req_mask != nullptr ? (int)B.valid_req_mask[tile_z] : 1;
-        t.rq_start = __builtin_amdgcn_readfirstlane(lo);
-        t.rq_end = __builtin_amdgcn_readfirstlane(hi);
-        t.seq_after = __builtin_amdgcn_readfirstlane(sa);
-        t.ctx_before = B.context_lens_before != nullptr ? __builtin_amdgcn_readfirstlane(cb)
-                                                        : t.seq_after - (t.rq_end - t.rq_start);
-        t.hit = __builtin_amdgcn_readfirstlane(rm) != 0 && t.rq_end > t.rq_start;
-        return t;
-    }
-    int tiles_before = 0;
-    for (int base = 0; base < B.num_reqs; base += 64) {
-        const int r = base + lane;
-        const bool inb = r < B.num_reqs;
-        const int lo = inb ? B.query_start_loc[r] : 0;
-        const int hi = inb ? B.query_start_loc[r + 1] : 0;
-        const int sa = inb ? B.seq_lens_after[r] : 0;
-        const int cb = (inb && B.context_lens_before != nullptr) ? B.context_lens_before[r] : 0;
-        const int rm = (inb && B.valid_req_mask != nullptr) ? (int)B.valid_req_mask[r] : 1;
-        const int cnt = hi > lo ? fast_div(hi - lo + P.tok_tile - 1, P.tok_tile) : 0;
-        int incl = cnt;
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const int up = __shfl_up(incl, off, 64);
-            if (lane >= off) incl += up;
-        }
-        const int first = tiles_before + incl - cnt;
-        const unsigned long long hits = __ballot(cnt > 0 && tile_z >= first && tile_z < first + cnt);
-        if (hits != 0ull) {
-            const int src = __builtin_ctzll(hits);
-            t.req = base + src;
-            t.rq_start = __builtin_amdgcn_readlane(lo, src);
-            t.rq_end = __builtin_amdgcn_readlane(hi, src);
-            t.seq_after = __builtin_amdgcn_readlane(sa, src);
-            t.ctx_before = B.context_lens_before != nullptr ? __builtin_amdgcn_readlane(cb, src)
-                                                            : t.seq_after - (t.rq_end - t.rq_start);
-            t.tile_in_req = tile_z - __builtin_amdgcn_readlane(first, src);
-            t.hit = __builtin_amdgcn_readlane(rm, src) != 0;
-            return t;
-        }
-        tiles_before += __builtin_amdgcn_readlane(incl, 63);
-    }
-    return t;
 }
 
 }  // namespace w34

@@ -85,7 +85,6 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     const int b = lane >> 4;
     const warp34_kv_layer_layout& L = P.L;
     const warp34_attention_batch& B = P.B;
-    W34_TP(0);
 
     // ---- tile identification: blockIdx = (tile of the request, kv head x q subgroup, request) ----
     const int req = (int)blockIdx.z;
@@ -685,10 +684,16 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
                 a[j] = (IS_BF16 && h == 0) ? av0[j] : *reinterpret_cast<const h8*>(vb + d * 64 + 16 * (b ^ ((d >> 1) & 3)));
             }
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                o_acc[h][j] = pf_mfma32<IS_BF16>(a[j], __builtin_bit_cast(h8, pb[h]), o_acc[h][j]);
-                if constexpr (IS_BF16) o_acc[h][j] = pf_mfma32<true>(a[j], __builtin_bit_cast(h8, pb_lo), o_acc[h][j]);
-                if constexpr (TQ4F) o_acc[h][j] = pf_mfma32<false>(a[j], __builtin_bit_cast(h8, pb_l2[h]), o_acc[h][j]);
+            for (int j = 0; j < 8; ++j) o_acc[h][j] = pf_mfma32<IS_BF16>(a[j], __builtin_bit_cast(h8, pb[h]), o_acc[h][j]);
+            // the low-order operands in a pass of their own: a tile's two MFMAs are then eight
+            // instructions apart instead of back to back (the second waits for the first's result)
+            if constexpr (IS_BF16) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) o_acc[h][j] = pf_mfma32<true>(a[j], __builtin_bit_cast(h8, pb_lo), o_acc[h][j]);
+            }
+            if constexpr (TQ4F) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) o_acc[h][j] = pf_mfma32<false>(a[j], __builtin_bit_cast(h8, pb_l2[h]), o_acc[h][j]);
             }
         }
     };
@@ -698,21 +703,14 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     const int32_t pg_first = __builtin_amdgcn_readfirstlane(load_page(0));
     int32_t pg_next = load_page(1);
     if (n_units > 0) issue_loads(0, pg_first);
-    W34_TP(1);
     for (int it = -2; it < n_units; ++it) {
         // commit unit it + 2 (loaded during the previous iteration), then start unit it + 3
         if (it + 2 < n_units) commit_loads((it + 2) & 1);
-#ifdef W34_TRACE
-        if (it >= 8 && it < 16) W34_TP(4 + 5 * (it - 8));
-#endif
         // The page id of unit it + 4 is requested BEFORE the key loads of unit it + 3: a
         // write to its register after them would have to wait for all of them to return.
         const int32_t pg_s = __builtin_amdgcn_readfirstlane(pg_next);
         pg_next = load_page(it + 4);
         if (it + 3 < n_units) issue_loads(it + 3, pg_s);
-#ifdef W34_TRACE
-        if (it >= 8 && it < 16) W34_TP(4 + 5 * (it - 8) + 1);
-#endif
         // TQ4 pages: the two waves of a SIMD (w and w + 4) take the two halves of an iteration in
         // opposite order, so that one dequantises (table reads and VALU) while the other
         // multiplies.  Both orders are valid between two barriers: the dequantiser writes buffer
@@ -734,22 +732,12 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
                 dequant_unit((it + 1) & 1, (it + 1) & 1);
             }
         }
-#ifdef W34_TRACE
-        if (it >= 8 && it < 16) W34_TP(4 + 5 * (it - 8) + 2);
-#endif
         if (!compute_first && it >= 0) {
             const int t0 = (u_first + it) * kUnit;
             compute_unit(it & 1, t0, !(t0 >= i_lo && t0 + kUnit - 1 <= i_hi));
         }
-#ifdef W34_TRACE
-        if (it >= 8 && it < 16) W34_TP(4 + 5 * (it - 8) + 3);
-#endif
         __syncthreads();
-#ifdef W34_TRACE
-        if (it >= 8 && it < 16) W34_TP(4 + 5 * (it - 8) + 4);
-#endif
     }
-    W34_TP(50);
 
     // ---- epilogue: normalise, transpose through LDS, rotate back, store ----
     l_run = sum_over_rows(l_run);

@@ -113,7 +113,6 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
     const int kv_head = fast_div(kv_sub, P.q_subgroups);
     const int q_head_base = kv_head * P.gqa + (kv_sub - kv_head * P.q_subgroups) * P.q_group;
 
-    W34_TP(0);
     // ---- this token's list ------------------------------------------------------------------------
     // The counts and the list entries of this wave's first unit are requested together: the first
     // unit is guessed from the list's capacity (exact when the list is full, the common case) and
@@ -155,7 +154,6 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
         for (int k = 0; k < 8; ++k) dst[k] = vv;
     }
 
-    W34_TP(47);
     int n_sel = __builtin_amdgcn_readfirstlane(a_live) != 0 ? __builtin_amdgcn_readfirstlane(a_sel) : 0;
     if (n_sel > P.select_k) n_sel = P.select_k;
     if (n_sel < 0) n_sel = 0;
@@ -245,9 +243,7 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
             load_groups(unit, id_vec, pos_vec);
         }
     }
-    W34_TP(41);
     issue_loads(id_vec);  // harmless for a wave without work
-    W34_TP(42);
 
     // ---- rotated, scaled fp16 queries to LDS, then the B operands of the QK MFMAs -----------------
     constexpr int kQStride = 264;
@@ -268,9 +264,7 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
         packed.y = pack_h2(qv[2] * q_scale, qv[3] * q_scale);
         *reinterpret_cast<uint2*>(qlds + col * kQStride + 4 * lane) = packed;
     }
-    W34_TP(44);
     __syncthreads();
-    W34_TP(45);
     h8 bq[9];
     {
         const int kb = 8 * (b & 1) + 4 * (b >> 1);
@@ -291,9 +285,7 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
 #pragma unroll
         for (int m = 0; m < 4; ++m) bq[5 + m] = *reinterpret_cast<const h8*>(qrow + 256 + 16 * (kb + m));
     }
-    W34_TP(46);
     __syncthreads();  // qlds is dead, the staging area may be overwritten; the table is complete
-    W34_TP(2);
 
     const uint32_t lut_lane = (uint32_t)lane << 2;
     const bool col_ok = n < P.q_group;
@@ -438,18 +430,18 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
             const u4 ph = {pb_hi[0], pb_hi[1], pb_hi[2], pb_hi[3]};
             const u4 pl = {pb_lo[0], pb_lo[1], pb_lo[2], pb_lo[3]};
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
+            for (int j = 0; j < 8; ++j)
                 o_acc[h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a[j]),
                                                                     __builtin_bit_cast(h8, ph), o_acc[h][j], 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < 8; ++j)  // (a pass of its own: a tile's two MFMAs are not back to back)
                 o_acc[h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a[j]),
                                                                     __builtin_bit_cast(h8, pl), o_acc[h][j], 0, 0, 0);
-            }
         }
     };
 
     while (unit < cu_end) {
         commit_loads();
-        W34_TP(4);
         const int cur_pos_vec = pos_vec;
         const int next_unit = unit + kQsaWaves;
         if (next_unit < cu_end) {
@@ -462,12 +454,10 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
         // interior unit: all eight groups present and wholly in front of the token's position
         const bool interior = __ballot(lane < 8 && cur_pos_vec + 3 > seq_pos) == 0ull;
         process_unit(gp0, gp1, !interior);
-        W34_TP(7);
         unit = next_unit;
     }
 
     // ---- merge the waves' states through LDS (layout as in the dense kernel) -------------------------
-    W34_TP(36);
     l_run = sum_over_rows(l_run);
     float* xbuf = reinterpret_cast<float*>(smem);
     float* mlbuf = reinterpret_cast<float*>(smem + (kQsaSmem - kQsaMlBytes));
@@ -475,9 +465,7 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
         mlbuf[(wave * 16 + n) * 2 + 0] = m_run;
         mlbuf[(wave * 16 + n) * 2 + 1] = l_run;
     }
-    W34_TP(49);
     __syncthreads();  // every wave is done with the table and with its staging area
-    W34_TP(50);
     {
         float mt = kNegBig;
 #pragma unroll
@@ -500,9 +488,7 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
             mltot[n * 2 + 1] = lt;
         }
     }
-    W34_TP(51);
     __syncthreads();
-    W34_TP(37);
     const float* mltot = mlbuf + kQsaWaves * 16 * 2;
 
     int merge_slot[4];  // region slot of element 4 lane + k (inverse of tq4_pv_elem)
@@ -549,7 +535,6 @@ __global__ __launch_bounds__(kQsaWaves * 64, 1) void qsa_sparse_tq4_kernel(const
             qsa_finish_row(v, lane, row, true, P.gate != nullptr, g, P.had64 != 0, P.out);
         }
     }
-    W34_TP(40);
 }
 
 // One wave per (token, q head) row: lane s holds the record of split s (n_splits <= 16).
