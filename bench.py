@@ -7,7 +7,9 @@ several layers are allocated and the steps cycle through them, as a decode step 
 would, so that the working set (layers x 69.2 MB) exceeds the 256 MB last-level cache and
 the figure is an HBM figure.  K/V are synthetic bf16 N(0,1) with 1 % outlier channels (x20),
 TQ4-encoded by the library's own quantize-on-append kernel into 64-token pages whose
-physical order is a random permutation.
+physical order is a seeded permutation.  Every input comes from the library's deterministic
+generators (include/warp34_synth.h: SplitMix64 -> Box-Muller -> bf16, Fisher-Yates), so two
+machines build the same bytes.
 
 Prints ONE JSON line.
 """
@@ -57,10 +59,25 @@ WORKLOADS = {
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by
 # a plain copy of known size (profiles/paged_attn_tq4_decode_b1_ctx131072_hbm_traffic.txt); counters cannot
 # be read from inside this process, so workloads without such a profile report null.
-MEASURED_TRAFFIC = {"tq4_decode_b1_ctx131072": 71_824_000}
+MEASURED_TRAFFIC = {
+    # workload: (HBM bytes per launch of the dominant kernel, the profile that holds the counter readings)
+    "tq4_decode_b1_ctx131072": (71_824_000, "profiles/paged_attn_tq4_decode_b1_ctx131072_hbm_traffic.txt"),
+}
 SHARED_PREFIX = {"tq4_verify_16x4_ctx262144_shared200k": 200000}
 VERIFY_Q = {"tq4_verify_16x4_ctx262144_shared200k": 4}
 PREFILL_CHUNK = 2048
+
+
+def dev_bf16(torch, bits):
+    """uint16 bf16 bits (numpy) -> bf16 tensor on the device"""
+    return torch.from_numpy(bits.view(np.int16)).to("cuda:0").view(torch.bfloat16)
+
+
+def synth_normal(torch, ffi, shape, seed, dtype=None):
+    """N(0,1) tensor on the device from the library's generator (bf16 values, optionally cast)."""
+    n = int(np.prod(shape))
+    t = dev_bf16(torch, ffi.synth_normal_bf16(n + (n & 1), seed)[:n]).reshape(shape)
+    return t if dtype is None else t.to(dtype)
 
 
 def parse():
@@ -78,7 +95,6 @@ def parse():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run plain 256 MiB device copies instead of a workload (scale reference for the "
                          "FETCH_SIZE / WRITE_SIZE counters of rocprofv3 --pmc)")
-    ap.add_argument("--cpu-ctx", type=int, default=32768, help="context length of the CPU-oracle sample")
     args = ap.parse_args()
     prefill = "_prefill_" in args.workload
     if args.steps <= 0:
@@ -90,8 +106,10 @@ def parse():
 
 def build_workload(name, seed=0):
     fmt, ctx, pool_tokens = WORKLOADS[name]
-    if ctx is None:
-        ctx = np.random.default_rng(seed).integers(1024, 65537, size=32)
+    if ctx is None:  # 32 context lengths drawn uniformly from 1K .. 64K
+        from warp34_amd import ffi
+
+        ctx = ffi.synth_uniform_i32(32, 1024, 65536, seed)
     return fmt, np.asarray(ctx, dtype=np.int64), pool_tokens
 
 
@@ -110,10 +128,8 @@ class Layer:
         self.layout = ffi.Warp34KvLayerLayout(
             self.k.data_ptr(), self.v.data_ptr(), self.page, self.head, self.tok, self.page, self.head, self.tok,
             0, seed, KV_HEADS, HEAD_DIM, BLOCK, kv_format, kv_format, xf, xf, 0)
-        g = torch.Generator(device=dev)
-        g.manual_seed(1000 + seed)
         pages_per = [(int(c) + BLOCK - 1) // BLOCK for c in ctx]
-        perm = torch.randperm(pool_pages, generator=g, device=dev).to(torch.int32)
+        perm = torch.from_numpy(ffi.synth_permutation(pool_pages, 1000 + seed)).to(dev)
         mb = max(pages_per)
         bt = torch.zeros((len(ctx), mb), dtype=torch.int32, device=dev)
         at = 0
@@ -128,22 +144,24 @@ class Layer:
                 at += n
         self.block_tables = bt
         self.max_blocks = mb
-        # outlier channels: 3 of 256 per kv head scaled x20
-        gain = torch.ones((KV_HEADS, HEAD_DIM), device=dev)
-        for h in range(KV_HEADS):
-            idx = torch.randperm(HEAD_DIM, generator=g, device=dev)[:3]
-            gain[h, idx] = 20.0
+        # K and V rows: one stream per layer and tensor (3 of 256 channels per kv head x20), the
+        # requests' tokens one after the other
+        k_seed, v_seed = 10 * seed + 1, 10 * seed + 2
         stream = torch.cuda.current_stream().cuda_stream
         ex = ffi.Warp34Exec(stream, 0, 0, 0)
         chunk = 2048
         self.tail_k, self.tail_v, self.tail_slots = [], [], []
+        row_at = 0
         for r, c in enumerate(ctx):
             c = int(c)
             first = shared_pages * BLOCK if r > 0 else 0  # shared pages were filled by request 0
+            k_all = dev_bf16(torch, ffi.synth_kv_rows_bf16(c - first, KV_HEADS, HEAD_DIM, k_seed, 3, first_row=row_at))
+            v_all = dev_bf16(torch, ffi.synth_kv_rows_bf16(c - first, KV_HEADS, HEAD_DIM, v_seed, 3, first_row=row_at))
+            row_at += c - first
             for t0 in range(first, c, chunk):
                 n = min(chunk, c - t0)
-                kk = (torch.randn((n, KV_HEADS, HEAD_DIM), generator=g, device=dev) * gain).to(torch.bfloat16)
-                vv = (torch.randn((n, KV_HEADS, HEAD_DIM), generator=g, device=dev) * gain).to(torch.bfloat16)
+                kk = k_all[t0 - first:t0 - first + n]
+                vv = v_all[t0 - first:t0 - first + n]
                 pos = torch.arange(t0, t0 + n, device=dev)
                 slots = (bt[r, (pos // BLOCK)].to(torch.int64) * BLOCK + pos % BLOCK).to(torch.int32)
                 qsl = torch.tensor([0, n], dtype=torch.int32, device=dev)
@@ -161,40 +179,73 @@ class Layer:
                     self.tail_slots.append(slots)
 
 
-def cpu_baseline(ctx_len, threads):
-    """The CPU oracle (port of the reference's scalar path) timed on this host: one decode
-    attention layer at ctx_len tokens, all hardware threads."""
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(torch, sample, threads, min_seconds=1.5):
+    """The CPU oracle (restatement of the reference's scalar path) timed on this host over the SAME
+    workload the GPU leg ran: layer 0's pages as the append kernel wrote them (downloaded),
+    its block table, the same queries; all host threads up to 16.  Also reports how far the GPU
+    output is from the oracle's.  Requests beyond a bound on the total context are left out of
+    the sample (said in `sample`)."""
     import oracle
 
-    n_pages = (ctx_len + BLOCK - 1) // BLOCK
-    pool = oracle.HostPool(n_pages, KV_HEADS, HEAD_DIM, BLOCK, oracle.FMT_TQ4, oracle.XF_WHT256)
-    # encode a small set of rows and tile them: the attention cost does not depend on values
-    rows = 256
-    k = oracle.fill_kv_rows(rows, KV_HEADS, HEAD_DIM, 1, oracle.DT_BF16, 3)
-    v = oracle.fill_kv_rows(rows, KV_HEADS, HEAD_DIM, 2, oracle.DT_BF16, 3)
-    small = oracle.HostPool(rows // BLOCK, KV_HEADS, HEAD_DIM, BLOCK, oracle.FMT_TQ4, oracle.XF_WHT256)
-    bt_s = np.arange(rows // BLOCK, dtype=np.int32).reshape(1, -1)
-    wb = oracle.HostBatch([0, rows], [rows], bt_s, context_lens_before=[0],
-                          write_slot_mapping=oracle.slot_mapping(bt_s[0], 0, rows, BLOCK))
+    L, q, ctx, ql, fmt, got = sample["layer"], sample["q"], sample["ctx"], sample["ql"], sample["fmt"], sample["out"]
+    ofmt = {"tq4": oracle.FMT_TQ4, "bf16": oracle.FMT_BF16, "fp8": oracle.FMT_FP8, "q8_0": oracle.FMT_Q8_0}[fmt]
+    xf = oracle.XF_WHT256 if fmt == "tq4" else oracle.XF_IDENTITY
+    # bounded sample: leading requests up to 262 144 context tokens in total
+    keep, tot = 0, 0
+    for c in ctx:
+        if keep and tot + int(c) > 262144:
+            break
+        keep, tot = keep + 1, tot + int(c)
+    pool_pages = L.k.numel() // L.page
+    pool = oracle.HostPool(pool_pages, KV_HEADS, HEAD_DIM, BLOCK, ofmt, xf)
+    pool.k[:] = L.k.cpu().numpy()
+    pool.v[:] = L.v.cpu().numpy()
+    bt = L.block_tables[:keep].cpu().numpy()
+    qsl = [ql * r for r in range(keep + 1)]
+    seq = [int(c) for c in ctx[:keep]]
+    hb = oracle.HostBatch(qsl, seq, bt, context_lens_before=[c - ql for c in seq])
+    qb = q[:keep * ql].contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+    # append rate: 4 096 rows, single thread
+    rows = 4096
+    kk = oracle.fill_kv_rows(rows // (2 * KV_HEADS), KV_HEADS, HEAD_DIM, 1, oracle.DT_BF16, 3)
+    small = oracle.HostPool(rows // (2 * KV_HEADS) // BLOCK, KV_HEADS, HEAD_DIM, BLOCK, ofmt, xf)
+    bt_s = np.arange(small.k.size // (KV_HEADS * BLOCK * ROW_BYTES[fmt]), dtype=np.int32).reshape(1, -1)
+    n_s = rows // (2 * KV_HEADS)
+    wb = oracle.HostBatch([0, n_s], [n_s], bt_s, context_lens_before=[0],
+                          write_slot_mapping=oracle.slot_mapping(bt_s[0], 0, n_s, BLOCK))
     t0 = time.perf_counter()
-    oracle.kv_cache_write(small, wb, k, v, oracle.DT_BF16)
+    oracle.kv_cache_write(small, wb, kk, kk, oracle.DT_BF16)
     t_append = time.perf_counter() - t0
-    reps = (pool.k.size + small.k.size - 1) // small.k.size
-    pool.k[:] = np.tile(small.k, reps)[:pool.k.size]
-    pool.v[:] = np.tile(small.v, reps)[:pool.v.size]
-    bt = oracle.permutation(n_pages, 3).reshape(1, -1)
-    q = oracle.fill_normal(Q_HEADS * HEAD_DIM, 4, oracle.DT_BF16).reshape(1, Q_HEADS, HEAD_DIM)
-    hb = oracle.HostBatch([0, 1], [ctx_len], bt, context_lens_before=[ctx_len - 1])
-    t0 = time.perf_counter()
-    oracle.paged_attention(pool, hb, q, oracle.DT_BF16, Q_HEADS, n_threads=threads)
-    dt = time.perf_counter() - t0
-    kv_bytes = ctx_len * KV_HEADS * 2 * ROW_BYTES["tq4"]
+    reps, t_total, want = 0, 0.0, None
+    while t_total < min_seconds:
+        t0 = time.perf_counter()
+        want = oracle.paged_attention(pool, hb, qb, oracle.DT_BF16, Q_HEADS, n_threads=threads)
+        t_total += time.perf_counter() - t0
+        reps += 1
+    dt = t_total / reps
+    kv_bytes = tot * KV_HEADS * 2 * ROW_BYTES[fmt]
+    gotf = got[:keep * ql].float().cpu().numpy().astype(np.float64)
+    err = np.abs(gotf - np.asarray(want, dtype=np.float64))
     return {
         "value": round(kv_bytes / dt / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
-        "sample": "CPU oracle (oracle/tq4_oracle.c), 1 layer decode attention, ctx %d tokens, %d pthreads: "
-                  "%.1f ms/layer; append of %d rows single-thread: %.0f rows/s"
-                  % (ctx_len, threads, dt * 1e3, rows * KV_HEADS * 2, rows * KV_HEADS * 2 / t_append),
+        "sample": "CPU oracle (oracle/tq4_oracle.c) over the same workload: layer 0's pages as written by the append "
+                  "kernel, %d of %d requests (%d context tokens), %d query token(s) each, %d pthreads on %s "
+                  "(%d hardware threads): %.1f ms/layer, mean of %d runs; append of %d rows single-thread: %.0f rows/s"
+                  % (keep, len(ctx), tot, ql, threads, cpu_model(), os.cpu_count() or 0, dt * 1e3, reps, rows,
+                     rows / t_append),
         "us_per_layer": round(dt * 1e6, 1),
+        "gpu_vs_oracle": {"max_abs_err": float(err.max()), "max_rel": float(err.max() / max(np.abs(want).max(), 1e-30)),
+                          "worst_excess_over_2e-3_plus_1e-2_want": float((err - (2e-3 + 1e-2 * np.abs(want))).max())},
     }
 
 
@@ -204,9 +255,7 @@ def run_prefill(args, torch, lib, ffi, layers, ctx, n_layers, pool_pages, fmt):
     dev = "cuda:0"
     R, n = len(ctx), PREFILL_CHUNK
     N = R * n
-    g = torch.Generator(device=dev)
-    g.manual_seed(7)
-    q = torch.randn((N, Q_HEADS, HEAD_DIM), generator=g, device=dev).to(torch.bfloat16)
+    q = synth_normal(torch, ffi, (N, Q_HEADS, HEAD_DIM), 7)
     out = torch.zeros_like(q)
     qsl = (torch.arange(0, R + 1, dtype=torch.int32, device=dev) * n).to(torch.int32)
     seq = torch.tensor(ctx, dtype=torch.int32, device=dev)
@@ -283,10 +332,8 @@ def run_gate(args, torch, lib, ffi):
     are cycled so that the 403 MB of a step do not come out of the Infinity Cache."""
     dev = "cuda:0"
     n, dim, sets = 16384, Q_HEADS * HEAD_DIM, 3
-    g = torch.Generator(device=dev)
-    g.manual_seed(5)
-    bufs = [tuple(torch.randn((n, dim), generator=g, device=dev).to(torch.float16) for _ in range(2)) +
-            (torch.empty((n, dim), dtype=torch.float16, device=dev),) for _ in range(sets)]
+    bufs = [tuple(synth_normal(torch, ffi, (n, dim), 50 + 2 * i + j, torch.float16) for j in range(2)) +
+            (torch.empty((n, dim), dtype=torch.float16, device=dev),) for i in range(sets)]
     ex = ffi.Warp34Exec(torch.cuda.current_stream().cuda_stream, 0, 0, 0)
 
     def step(i):
@@ -326,17 +373,16 @@ def run_qsa(args, torch, lib, ffi, layers, ctx_len, n_layers, n_tok, fmt, select
     drawn from the sequence's groups (the last group always among them, as the selector keeps the
     newest keys).  Algorithmic bytes = the selected K and V rows of both kv heads + the gate rows."""
     dev = "cuda:0"
-    g = torch.Generator(device=dev)
-    g.manual_seed(23)
-    q = torch.randn((n_tok, Q_HEADS, HEAD_DIM), generator=g, device=dev).to(torch.float16)
-    gate = torch.randn((n_tok, Q_HEADS, HEAD_DIM), generator=g, device=dev).to(torch.float16)
+    q = synth_normal(torch, ffi, (n_tok, Q_HEADS, HEAD_DIM), 23, torch.float16)
+    gate = synth_normal(torch, ffi, (n_tok, Q_HEADS, HEAD_DIM), 24, torch.float16)
     out = torch.zeros_like(q)
     n_groups = ctx_len // 4
     gpp = BLOCK // 4
     per_layer = []
-    for L in layers:
-        logs = torch.stack([torch.cat([torch.randperm(n_groups - 1, generator=g, device=dev)[:select_k - 1],
-                                       torch.tensor([n_groups - 1], device=dev)]) for _ in range(n_tok)])
+    for li, L in enumerate(layers):
+        logs = torch.stack([torch.cat([
+            torch.from_numpy(ffi.synth_permutation(n_groups - 1, 3000 + 1000 * li + t)[:select_k - 1].astype(np.int64)).to(dev),
+            torch.tensor([n_groups - 1], device=dev)]) for t in range(n_tok)])
         phys = L.block_tables[0, (logs * 4 // BLOCK)].to(torch.int64) * gpp + (logs * 4 % BLOCK) // 4
         per_layer.append((phys.to(torch.int32).contiguous(), logs.to(torch.int32).contiguous()))
     num_sel = torch.full((n_tok,), select_k, dtype=torch.int32, device=dev)
@@ -394,14 +440,12 @@ def run_producer(args, torch, lib, ffi, layers, n, n_layers, fmt):
     into TQ4 pages: the fused entry point against the two-call sequence (operator in place, then
     the strided append).  One step = one layer's producer work for an n-token chunk."""
     dev = "cuda:0"
-    g = torch.Generator(device=dev)
-    g.manual_seed(11)
     row = (Q_HEADS + 2 * KV_HEADS) * HEAD_DIM
-    qkv0 = torch.randn((n, row), generator=g, device=dev).to(torch.bfloat16)
+    qkv0 = synth_normal(torch, ffi, (n, row), 11)
     qkv = qkv0.clone()
     q_out = torch.empty((n, Q_HEADS * HEAD_DIM), dtype=torch.bfloat16, device=dev)
-    qw = (1.0 + 0.1 * torch.randn(HEAD_DIM, generator=g, device=dev)).to(torch.bfloat16)
-    kw = (1.0 + 0.1 * torch.randn(HEAD_DIM, generator=g, device=dev)).to(torch.bfloat16)
+    qw = (1.0 + 0.1 * synth_normal(torch, ffi, (HEAD_DIM,), 12, torch.float32)).to(torch.bfloat16)
+    kw = (1.0 + 0.1 * synth_normal(torch, ffi, (HEAD_DIM,), 13, torch.float32)).to(torch.bfloat16)
     half = HEAD_DIM // 2
     inv_freq = 1.0 / (10000.0 ** (torch.arange(half, device=dev) / half))
     ang = torch.arange(n, device=dev)[:, None] * inv_freq[None, :]
@@ -522,13 +566,15 @@ def main():
         sub.workload, sub.steps, sub.warmup = "tq4_decode_b8_ctx131072", 200, 20
         torch.cuda.empty_cache()
         r8 = run_workload(sub, torch, lib, ffi, dev)
+        r8.pop("_sample")
         result["batch_point"] = {"workload": sub.workload, "us_per_layer": r8["us_per_layer"],
                                  "GBps": r8["value"], "frac": r8["roofline"]["frac"], "steps": sub.steps,
                                  "kv_bytes_per_step": r8["config"]["kv_bytes_per_step"]}
+    sample = result.pop("_sample")
     if not args.no_cpu_baseline:
         import oracle
 
-        result["cpu_baseline"] = cpu_baseline(args.cpu_ctx, min(oracle.hw_threads(), 16))
+        result["cpu_baseline"] = cpu_baseline(torch, sample, min(oracle.hw_threads(), 16))
     print(json.dumps(result))
 
 
@@ -566,9 +612,7 @@ def run_workload(args, torch, lib, ffi, dev):
 
     R = len(ctx)
     ql = VERIFY_Q.get(args.workload, 1)  # query tokens per request (1 = decode)
-    g = torch.Generator(device=dev)
-    g.manual_seed(7)
-    q = torch.randn((R * ql, Q_HEADS, HEAD_DIM), generator=g, device=dev).to(torch.bfloat16)
+    q = synth_normal(torch, ffi, (R * ql, Q_HEADS, HEAD_DIM), 7)
     out = torch.zeros_like(q)
     qsl = (torch.arange(0, R + 1, dtype=torch.int32, device=dev) * ql).to(torch.int32)
     seq = torch.tensor(ctx, dtype=torch.int32, device=dev)
@@ -604,6 +648,9 @@ def run_workload(args, torch, lib, ffi, dev):
     t_wall = time.perf_counter() - t_wall0
     ms_per_step = e0.elapsed_time(e1) / args.steps
     assert torch.isfinite(out.float()).all()
+    step(0)  # layer 0 once more: its output is what the CPU leg checks
+    torch.cuda.synchronize()
+    sample = {"layer": layers[0], "q": q, "ctx": ctx, "ql": ql, "fmt": fmt, "out": out.clone()}
 
     gbs = kv_bytes / (ms_per_step * 1e-3) / 1e9
     result = {
@@ -640,13 +687,15 @@ def run_workload(args, torch, lib, ffi, dev):
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(gbs / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC.get(args.workload),
+            "traffic": MEASURED_TRAFFIC.get(args.workload, (None, None))[0],
+            "traffic_source": MEASURED_TRAFFIC.get(args.workload, (None, None))[1],
             "kernel": "paged_attn_%s_kernel (+ merge kernel, both inside the timed launch)"
                       % (("tq4" if fmt == "tq4" else "rows") + ("_balanced" if R > 1 and ql == 1 else "")),
             "avg_launch_us": round(ms_per_step * 1e3, 3),
             "host_wall_us_per_step": round(t_wall / args.steps * 1e6, 2),
         },
     }
+    result["_sample"] = sample
     return result
 
 

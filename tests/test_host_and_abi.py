@@ -4,7 +4,7 @@ The host tests are a C++ program (tests/host/kv_host_test.cpp) restating the ref
 unit tests for this path (crates/warp34-host/src/cache.rs:628-826, model/graph_io.rs:1286);
 it is compiled with the host compiler, with address and undefined-behaviour sanitizers, and run here.
 The ABI tests check that the shared library loads without a GPU, exports every symbol
-include/warp34_kv.h declares, and that the descriptor structs have the sizes the reference
+the headers under include/ declare, and that the descriptor structs have the sizes the reference
 static_asserts (warp34_cuda.h:57,80,101).  No compute entry point is called.
 """
 import ctypes as C
@@ -32,7 +32,9 @@ def test_host_mirror_cpp(tmp_path):
 
 
 def _declared_symbols():
-    text = open(os.path.join(ROOT, "include", "warp34_kv.h")).read()
+    import glob
+
+    text = "".join(open(h).read() for h in sorted(glob.glob(os.path.join(ROOT, "include", "*.h"))))
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     text = re.sub(r"//[^\n]*", "", text)
     return sorted(set(re.findall(r"\b(warp34_[a-z0-9_]+)\s*\(", text)))

@@ -93,8 +93,13 @@ _EX = C.POINTER(Warp34Exec)
 _LAY = C.POINTER(Warp34KvLayerLayout)
 _BAT = C.POINTER(Warp34AttentionBatch)
 
-# name -> (restype, argtypes); every symbol include/warp34_kv.h declares
+# name -> (restype, argtypes); every symbol the headers under include/ declare
 SIGNATURES = {
+    # deterministic synthetic inputs (include/warp34_synth.h)
+    "warp34_synth_normal_bf16": (None, [C.c_void_p, C.c_size_t, C.c_size_t, C.c_uint64]),
+    "warp34_synth_kv_rows_bf16": (None, [C.c_void_p, C.c_size_t, C.c_size_t, C.c_int, C.c_int, C.c_uint64, C.c_int]),
+    "warp34_synth_permutation": (None, [C.c_void_p, C.c_int, C.c_uint64]),
+    "warp34_synth_uniform_i32": (None, [C.c_void_p, C.c_int, C.c_int32, C.c_int32, C.c_uint64]),
     "warp34_kv_cache_write": (C.c_int, [_EX, _LAY, _BAT, C.c_void_p, C.c_void_p]),
     "warp34_kv_cache_write_strided": (C.c_int, [_EX, _LAY, _BAT, C.c_void_p, C.c_void_p, C.c_int, C.c_int]),
     "warp34_kv_cache_write_bf16": (C.c_int, [_EX, _LAY, _BAT, C.c_void_p, C.c_void_p]),
@@ -185,3 +190,39 @@ class Warp34Error(RuntimeError):
 def check_rc(rc, context):
     if rc != 0:
         raise Warp34Error(rc, context)
+
+
+# ---- deterministic synthetic inputs (include/warp34_synth.h) as numpy arrays ----
+
+def synth_normal_bf16(n, seed, first=0):
+    """Elements first .. first + n of the N(0,1) stream of `seed`, bf16 bits (uint16)."""
+    import numpy as np
+
+    out = np.empty(n, dtype=np.uint16)
+    load().warp34_synth_normal_bf16(out.ctypes.data, first, n, seed)
+    return out
+
+
+def synth_kv_rows_bf16(rows, kv_heads, head_dim, seed, n_outliers=3, first_row=0):
+    """Rows first_row .. first_row + rows of the K / V tensor of `seed`: [rows, kv_heads, head_dim] bf16 bits."""
+    import numpy as np
+
+    out = np.empty((rows, kv_heads, head_dim), dtype=np.uint16)
+    load().warp34_synth_kv_rows_bf16(out.ctypes.data, first_row, rows, kv_heads, head_dim, seed, n_outliers)
+    return out
+
+
+def synth_permutation(n, seed):
+    import numpy as np
+
+    out = np.empty(n, dtype=np.int32)
+    load().warp34_synth_permutation(out.ctypes.data, n, seed)
+    return out
+
+
+def synth_uniform_i32(n, lo, hi, seed):
+    import numpy as np
+
+    out = np.empty(n, dtype=np.int32)
+    load().warp34_synth_uniform_i32(out.ctypes.data, n, lo, hi, seed)
+    return out
