@@ -223,6 +223,42 @@ int warp34_dflash_qk_norm_rope_kv_write_bf16_f32_table(
     const warp34_kv_layer_layout* kv_layout, const int32_t* write_slot_mapping,
     int rows, int q_heads, int kv_heads, int dim, int table_rows, float eps);  /* warp34_cuda.h:625-628 */
 
+/* Producer side of the target model's gated full-attention layers (model/forward.rs:1105-1148):
+ * Gemma RMSNorm (weight 1 + w) over every Q head of q_gate_in ([tokens, q_gate_row_stride], head h
+ * at h * 2 * head_dim: head_dim query elements, then head_dim gate elements) and every K head of
+ * k_in ([tokens, k_row_stride]), interleaved mRoPE over the first rotary_dim elements (pair
+ * (i, i + rotary_dim / 2), position plane i % 3 for i below 3 * s1 / 3 * s2, plane 0 otherwise;
+ * positions = three planes pos_plane_stride apart), and the gate halves copied to gate_out; all
+ * fp16, outputs dense [tokens, heads, head_dim].  Tokens whose valid_token_mask byte is 0 are
+ * skipped (mask may be NULL).  Replaces ops/op_norms_rope_act.cu:524-689,1201-1272.  This build
+ * wants head_dim % 8 == 0 and <= 256, rotary_dim <= 256, strides % 8 == 0 and 16-byte aligned
+ * pointers (hipErrorNotSupported otherwise). */
+int warp34_fused_qk_rmsnorm_rope_gate_strided_f16(
+    const warp34_exec* ex, const void* q_gate_in, const void* k_in, const void* q_norm_w,
+    const void* k_norm_w, const int32_t* positions, const uint8_t* valid_token_mask, void* q_out,
+    void* k_out, void* gate_out, int num_tokens, int pos_plane_stride, int num_q_heads,
+    int num_kv_heads, int head_dim, int rotary_dim, int mrope_s0, int mrope_s1, int mrope_s2,
+    int q_gate_row_stride, int k_row_stride, float rope_theta, float rms_eps); /* warp34_cuda.h:264-287 */
+int warp34_fused_qk_rmsnorm_rope_gate_f16(
+    const warp34_exec* ex, const void* q_gate_in, const void* k_in, const void* q_norm_w,
+    const void* k_norm_w, const int32_t* positions, const uint8_t* valid_token_mask, void* q_out,
+    void* k_out, void* gate_out, int num_tokens, int pos_plane_stride, int num_q_heads,
+    int num_kv_heads, int head_dim, int rotary_dim, int mrope_s0, int mrope_s1, int mrope_s2,
+    float rope_theta, float rms_eps);                                         /* warp34_cuda.h:241-262 */
+/* The same operator fused with the append.  No counterpart in the reference, which runs the
+ * operator and then warp34_kv_cache_write_strided (model/forward.rs:1128-1148): here the finished K
+ * rows and the V rows of v_in ([tokens, v_row_stride], fp16) go straight to the pages of kv_layout
+ * at write_slot_mapping[token] (negative: no cache write for that token), with bits equal to that
+ * sequence's.  k_out may be NULL.  head_dim 256, K and V pages of one format and transform. */
+int warp34_fused_qk_rmsnorm_rope_gate_kv_write_f16(
+    const warp34_exec* ex, const void* q_gate_in, const void* k_in, const void* v_in,
+    const void* q_norm_w, const void* k_norm_w, const int32_t* positions,
+    const uint8_t* valid_token_mask, void* q_out, void* k_out, void* gate_out,
+    const warp34_kv_layer_layout* kv_layout, const int32_t* write_slot_mapping, int num_tokens,
+    int pos_plane_stride, int num_q_heads, int num_kv_heads, int head_dim, int rotary_dim,
+    int mrope_s0, int mrope_s1, int mrope_s2, int q_gate_row_stride, int k_row_stride,
+    int v_row_stride, float rope_theta, float rms_eps);
+
 /* Consumer side of the path: out = attn_out * sigmoid(gate) over fp16 [num_tokens, total_dim]
  * (replaces ops/op_norms_rope_act.cu:742-759,1329-1344; called right after
  * warp34_paged_attention_f16 in the gated layers, model/forward.rs:1192-1211).  Rows whose

@@ -91,6 +91,8 @@ def lib():
         L.tq4o_qk_norm_rope_bf16.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                              C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float,
                                              C.POINTER(Layout), C.c_void_p]
+        L.tq4o_fused_qk_rmsnorm_rope_gate_f16.restype = C.c_int
+        L.tq4o_fused_qk_rmsnorm_rope_gate_f16.argtypes = [C.c_void_p] * 9 + [C.c_int] * 11 + [C.c_float, C.c_float]
         L.tq4o_fill_normal.argtypes = [C.c_void_p, C.c_size_t, C.c_uint64, C.c_int]
         L.tq4o_fill_kv_rows.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_uint64, C.c_int, C.c_int]
         L.tq4o_permutation.argtypes = [C.c_void_p, C.c_int, C.c_uint64]
@@ -332,6 +334,33 @@ def qk_norm_rope_bf16(qkv, positions, qw, kw, table, q_heads, kv_heads, dim, eps
     if rc:
         raise RuntimeError("oracle qk_norm_rope_bf16: rc=%d" % rc)
     return qkv, q_out
+
+
+def fused_qk_rmsnorm_rope_gate_f16(q_gate, k, q_norm_w, k_norm_w, positions, num_q_heads, num_kv_heads, head_dim,
+                                   rotary_dim, mrope, rope_theta, rms_eps, valid_token_mask=None, q_out=None,
+                                   k_out=None, gate_out=None):
+    """ops/op_norms_rope_act.cu:524-689.  q_gate: uint16 (fp16 bits) [tokens, q_gate_row_stride], k: uint16
+    [tokens, k_row_stride] (row strides taken from the arrays), positions: int32 [3, plane_stride],
+    mrope: the three section sizes.  Returns (q_out, k_out, gate_out) as uint16 [tokens, heads, head_dim];
+    buffers passed in keep their bytes where a token is masked."""
+    n = q_gate.shape[0]
+    assert q_gate.dtype == np.uint16 and k.dtype == np.uint16 and q_gate.flags.c_contiguous and k.flags.c_contiguous
+    positions = np.ascontiguousarray(positions, dtype=np.int32)
+    assert positions.ndim == 2 and positions.shape[0] == 3
+    q_out = np.zeros((n, num_q_heads, head_dim), dtype=np.uint16) if q_out is None else q_out
+    k_out = np.zeros((n, num_kv_heads, head_dim), dtype=np.uint16) if k_out is None else k_out
+    gate_out = np.zeros((n, num_q_heads, head_dim), dtype=np.uint16) if gate_out is None else gate_out
+    mask = None if valid_token_mask is None else np.ascontiguousarray(valid_token_mask, dtype=np.uint8)
+    qw = np.ascontiguousarray(q_norm_w, dtype=np.uint16)
+    kw = np.ascontiguousarray(k_norm_w, dtype=np.uint16)
+    rc = lib().tq4o_fused_qk_rmsnorm_rope_gate_f16(
+        q_gate.ctypes.data, k.ctypes.data, qw.ctypes.data, kw.ctypes.data, positions.ctypes.data,
+        None if mask is None else mask.ctypes.data, q_out.ctypes.data, k_out.ctypes.data, gate_out.ctypes.data,
+        n, positions.shape[1], num_q_heads, num_kv_heads, head_dim, rotary_dim, mrope[0], mrope[1], mrope[2],
+        q_gate.shape[1], k.shape[1], rope_theta, rms_eps)
+    if rc:
+        raise RuntimeError("oracle fused_qk_rmsnorm_rope_gate_f16: rc=%d" % rc)
+    return q_out, k_out, gate_out
 
 
 def apply_attn_output_gate_f16(attn_out, gate, out=None, valid_token_mask=None):

@@ -778,6 +778,101 @@ int tq4o_paged_attention_split(const tq4o_layout* L, const tq4o_batch* B, const 
     return 0;
 }
 
+/* ---- ops/op_norms_rope_act.cu:524-689,1201-1246: fused_qk_rmsnorm_rope_gate_f16_kernel, the
+ * producer of the target model's full-attention layers.  Per (token, head): Gemma RMSNorm
+ * (x * rsqrt(mean x^2 + eps) * (1 + w), rounded to fp16), rotation of the pairs (i, i + rotary/2)
+ * of the first `rotary_dim` elements by the angle pos_plane(i) * theta^(-2i/rotary_dim) with
+ * fp16-rounded sine and cosine (:649-657), the other elements copied; the gate half of every Q
+ * head is copied to gate_out (:562-585).  Position planes (:639-645): pair i takes plane 1 if
+ * i % 3 == 1 and i < 3 s1, plane 2 if i % 3 == 2 and i < 3 s2, else plane 0.
+ * Declared numerics: fp32 in source order, no contraction; the sum of squares as the kernel's
+ * 128-thread block forms it for head sizes that are multiples of 8 (thread t adds the eight
+ * squares of elements 8t .. 8t+7 in order, 32-lane xor butterflies, the warps' sums added by a
+ * butterfly over warp 0: :586-604, :28-46); rsqrt, powf, sinf, cosf := the double-precision
+ * result rounded once to fp32. ---- */
+int tq4o_fused_qk_rmsnorm_rope_gate_f16(const uint16_t* q_gate_in, const uint16_t* k_in, const uint16_t* q_norm_w,
+                                        const uint16_t* k_norm_w, const int32_t* positions,
+                                        const uint8_t* valid_token_mask, uint16_t* q_out, uint16_t* k_out,
+                                        uint16_t* gate_out, int num_tokens, int pos_plane_stride, int num_q_heads,
+                                        int num_kv_heads, int head_dim, int rotary_dim, int mrope_s0, int mrope_s1,
+                                        int mrope_s2, int q_gate_row_stride, int k_row_stride, float rope_theta,
+                                        float rms_eps) {
+    (void)mrope_s0;
+    if (!q_gate_in || !k_in || !q_norm_w || !k_norm_w || !positions || !q_out || !k_out || !gate_out) return -1;
+    if (num_tokens <= 0) return 0;
+    if (q_gate_row_stride < num_q_heads * 2 * head_dim || k_row_stride < num_kv_heads * head_dim) return -1;
+    if (head_dim <= 0 || (head_dim & 7) || head_dim > 1024 || rotary_dim < 0 || (rotary_dim & 1) ||
+        rotary_dim > head_dim)
+        return -2; /* the restated summation order is the vectorised one */
+    const int half_rot = rotary_dim / 2;
+    float* normed = (float*)malloc((size_t)head_dim * sizeof(float));
+    for (int tok = 0; tok < num_tokens; ++tok) {
+        if (valid_token_mask && valid_token_mask[tok] == 0) continue;
+        for (int head_idx = 0; head_idx < num_q_heads + num_kv_heads; ++head_idx) {
+            const int is_q = head_idx < num_q_heads;
+            const int local = is_q ? head_idx : head_idx - num_q_heads;
+            const uint16_t* src;
+            const uint16_t* w;
+            uint16_t* dst;
+            if (is_q) {
+                const uint16_t* base = q_gate_in + (size_t)tok * q_gate_row_stride + (size_t)local * 2 * head_dim;
+                src = base;
+                memcpy(gate_out + ((size_t)tok * num_q_heads + local) * head_dim, base + head_dim,
+                       (size_t)head_dim * sizeof(uint16_t));
+                w = q_norm_w;
+                dst = q_out + ((size_t)tok * num_q_heads + local) * head_dim;
+            } else {
+                src = k_in + (size_t)tok * k_row_stride + (size_t)local * head_dim;
+                w = k_norm_w;
+                dst = k_out + ((size_t)tok * num_kv_heads + local) * head_dim;
+            }
+            /* sum of squares: 128 threads, thread t owns vector t (8 elements) when t < head_dim / 8 */
+            float part[128];
+            for (int t = 0; t < 128; ++t) {
+                float acc = 0.0f;
+                if (8 * t < head_dim) {
+                    for (int j = 0; j < 8; ++j) {
+                        const float v = tq4o_f16_to_f32(src[8 * t + j]);
+                        const float sq = v * v;
+                        acc = acc + sq;
+                    }
+                }
+                part[t] = acc;
+            }
+            float warp_sums[32];
+            for (int k = 0; k < 32; ++k) warp_sums[k] = 0.0f;
+            for (int wv = 0; wv < 4; ++wv) warp_sums[wv] = warp_sum32(part + 32 * wv);
+            const float sum_sq = warp_sum32(warp_sums);
+            const float mean = sum_sq / (float)head_dim + rms_eps;
+            const float inv_rms = (float)(1.0 / sqrt((double)mean));
+            for (int i = 0; i < head_dim; ++i) {
+                const float v = tq4o_f16_to_f32(src[i]) * inv_rms;
+                const float wt = 1.0f + tq4o_f16_to_f32(w[i]);
+                normed[i] = tq4o_f16_to_f32(tq4o_f32_to_f16(v * wt));
+            }
+            for (int i = 0; i < half_rot; ++i) {
+                int plane = 0;
+                if ((i % 3) == 1 && i < mrope_s1 * 3) plane = 1;
+                else if ((i % 3) == 2 && i < mrope_s2 * 3) plane = 2;
+                const float pos = (float)positions[(size_t)plane * pos_plane_stride + tok];
+                const float expo = (float)(2 * i) / (float)rotary_dim;
+                const float pw = (float)pow((double)rope_theta, (double)expo);
+                const float inv_freq = 1.0f / pw;
+                const float angle = pos * inv_freq;
+                const float sin_a = tq4o_f16_to_f32(tq4o_f32_to_f16((float)sin((double)angle)));
+                const float cos_a = tq4o_f16_to_f32(tq4o_f32_to_f16((float)cos((double)angle)));
+                const float x1 = normed[i], x2 = normed[i + half_rot];
+                const float a = x1 * cos_a, b = x2 * sin_a, c = x2 * cos_a, d = x1 * sin_a;
+                dst[i] = tq4o_f32_to_f16(a - b);
+                dst[i + half_rot] = tq4o_f32_to_f16(c + d);
+            }
+            for (int i = rotary_dim; i < head_dim; ++i) dst[i] = tq4o_f32_to_f16(normed[i]);
+        }
+    }
+    free(normed);
+    return 0;
+}
+
 /* ---- deterministic synthetic inputs ---- */
 uint64_t tq4o_splitmix64(uint64_t* s) {
     uint64_t z = (*s += 0x9E3779B97F4A7C15ull);

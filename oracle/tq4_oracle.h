@@ -40,6 +40,12 @@
  *                     preserved; V bit-identical; cache rows = append of the rotated K.  The
  *                     reference's golden tensors for this operator are not in its tree (LFS
  *                     pointers only), so exact bf16 bits are "parity unpinned"
+ *   tq4o_fused_qk_rmsnorm_rope_gate  independent fp64 restatement (Gemma norm, plane selection,
+ *                     partial rotation) within one fp16 ulp; position 0 -> the normed row itself;
+ *                     pair norms preserved; un-rotated tail and gate copied bit for bit; text-only
+ *                     positions (three equal planes) = plain RoPE; masked tokens untouched.  No
+ *                     vector of this operator is in the reference tree: exact fp16 bits are
+ *                     "parity unpinned"
  *   tq4o_qsa_sparse   the reference test's known answer (V = 0.25, gate 0 -> 0.125, ple/gpu_tests.rs:677-681);
  *                     all groups of a sequence selected = dense causal attention of the last token;
  *                     brute-force fp64 softmax over independently dequantised rows with skipped groups,
@@ -142,6 +148,20 @@ int tq4o_qk_norm_rope_bf16(uint16_t* qkv, uint16_t* q_out, const int32_t* positi
                            const uint16_t* kw, const void* table, int table_is_f32, int rows, int q_heads,
                            int kv_heads, int dim, int table_rows, float eps, const tq4o_layout* L,
                            const int32_t* write_slot_mapping);
+
+/* ops/op_norms_rope_act.cu:524-689,1201-1246: the fused Gemma RMSNorm + interleaved mRoPE + gate split
+ * of the target model's full-attention layers, fp16.  q_gate_in [tokens, q_gate_row_stride]: per Q
+ * head head_dim query elements then head_dim gate elements; k_in [tokens, k_row_stride]; positions
+ * [3, pos_plane_stride]; outputs contiguous.  Masked tokens are skipped.  Returns -1 for the
+ * arguments the reference rejects, -2 for head sizes outside the restated summation order
+ * (head_dim a multiple of 8, at most 1024). */
+int tq4o_fused_qk_rmsnorm_rope_gate_f16(const uint16_t* q_gate_in, const uint16_t* k_in, const uint16_t* q_norm_w,
+                                        const uint16_t* k_norm_w, const int32_t* positions,
+                                        const uint8_t* valid_token_mask, uint16_t* q_out, uint16_t* k_out,
+                                        uint16_t* gate_out, int num_tokens, int pos_plane_stride, int num_q_heads,
+                                        int num_kv_heads, int head_dim, int rotary_dim, int mrope_s0, int mrope_s1,
+                                        int mrope_s2, int q_gate_row_stride, int k_row_stride, float rope_theta,
+                                        float rms_eps);
 
 /* ops/op_norms_rope_act.cu:742-759: out = attn_out * sigmoid(gate), fp16 [num_tokens, total_dim];
  * rows with a zero mask byte are skipped.  Pinned by the float64 sigmoid within one fp16 ulp,

@@ -24,6 +24,7 @@ SOURCES = [
     (os.path.join(CSRC, "kv_write.hip"), ["-ffp-contract=off"]),
     (os.path.join(CSRC, "qk_norm_rope.hip"), ["-ffp-contract=off"]),
     (os.path.join(CSRC, "attn_output_gate.hip"), ["-ffp-contract=off"]),
+    (os.path.join(CSRC, "fused_qk_norm.hip"), ["-ffp-contract=off"]),
     # leading scalar kernel arguments are preloaded into SGPRs at wave launch (gfx950 feature;
     # firmware without it runs the compatibility prologue the compiler emits)
     (os.path.join(CSRC, "paged_attn.hip"), ["-mllvm", "-amdgpu-kernarg-preload-count=12"]),

@@ -124,6 +124,12 @@ SIGNATURES = {
     "warp34_dflash_qk_norm_rope_kv_write_bf16_f32_table":
         (C.c_int, [_EX, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, _LAY, C.c_void_p,
                    C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float]),
+    "warp34_fused_qk_rmsnorm_rope_gate_strided_f16":
+        (C.c_int, [_EX] + [C.c_void_p] * 9 + [C.c_int] * 11 + [C.c_float, C.c_float]),
+    "warp34_fused_qk_rmsnorm_rope_gate_f16":
+        (C.c_int, [_EX] + [C.c_void_p] * 9 + [C.c_int] * 9 + [C.c_float, C.c_float]),
+    "warp34_fused_qk_rmsnorm_rope_gate_kv_write_f16":
+        (C.c_int, [_EX] + [C.c_void_p] * 10 + [_LAY, C.c_void_p] + [C.c_int] * 12 + [C.c_float, C.c_float]),
     "warp34_apply_attn_output_gate_f16":
         (C.c_int, [_EX, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int]),
     # QSA sparse paged attention over selected 4-token groups (plain, and with the per-64 output transform)
