@@ -267,6 +267,14 @@ int warp34_apply_attn_output_gate_f16(const warp34_exec* ex, const void* attn_ou
                                       void* out, const uint8_t* valid_token_mask,
                                       int num_tokens, int total_dim);             /* warp34_cuda.h:297-300 */
 
+/* warp34_paged_attention_f16 followed by warp34_apply_attn_output_gate_f16 in one call, with the
+ * bits of that sequence; the ungated output never goes to memory.  No counterpart in the reference
+ * (model/forward.rs:1192-1211 makes the two calls).  gate: fp16 [total_tokens, num_q_heads, 256],
+ * 8-byte aligned.  Rows of masked tokens and requests stay untouched. */
+int warp34_paged_attention_gated_f16(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
+                                     const warp34_attention_batch* batch, const void* q_in,
+                                     const void* gate, void* attn_out, int num_q_heads);
+
 /* QSA sparse paged attention: query token t attends over its own list of selected 4-token groups
  * (replaces ops/op_qsa.cu:716-1158,1446-1571,1711-1751).  Group j of token t is rows
  * (phys % (block_size / 4)) * 4 .. + 3 of page phys / (block_size / 4), phys =

@@ -123,8 +123,9 @@ def dev_write(dpool, hbatch, k_bits, v_bits, in_dtype, k_stride=None, v_stride=N
 
 
 def dev_attention(dpool, hbatch, q_bits, q_dtype, num_q_heads, scratch_bytes=0, sentinel=0x5500,
-                  max_seq_len=None, max_q_len=None, force_kernel=None, layout=None):
-    """Paged attention through the C ABI.  Returns (rc, out_bits uint16 [N, H, D], scratch tensor)."""
+                  max_seq_len=None, max_q_len=None, force_kernel=None, layout=None, gate=None):
+    """Paged attention through the C ABI.  Returns (rc, out_bits uint16 [N, H, D], scratch tensor).
+    gate (fp16 bits, the shape of the output): the gated entry point."""
     L = dpool.layout() if layout is None else layout
     db = DevBatch(hbatch, max_q_len=max_q_len, max_seq_len=max_seq_len)
     B = db.struct()
@@ -132,7 +133,12 @@ def dev_attention(dpool, hbatch, q_bits, q_dtype, num_q_heads, scratch_bytes=0, 
     qd = to_dev(q_bits)
     out = torch.full((hbatch.total_tokens, num_q_heads, dpool.h.head_dim), sentinel, dtype=torch.int16, device=DEV)
     l = lib()
-    if force_kernel is not None:
+    if gate is not None:
+        assert q_dtype == oracle.DT_F16 and force_kernel is None
+        gd = to_dev(gate)
+        rc = l.warp34_paged_attention_gated_f16(C.byref(ex), C.byref(L), C.byref(B), ptr(qd), ptr(gd), ptr(out),
+                                                num_q_heads)
+    elif force_kernel is not None:
         rc = l.warp34_paged_attention_f16_force_kernel_for_test(
             C.byref(ex), C.byref(L), C.byref(B), ptr(qd), ptr(out), num_q_heads, force_kernel)
     elif q_dtype == oracle.DT_BF16:

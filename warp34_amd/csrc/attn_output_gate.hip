@@ -32,8 +32,7 @@ __global__ __launch_bounds__(256) void attn_output_gate_kernel(const uint16_t* _
             for (int h = 0; h < 2; ++h) {
                 const float a = F16::to_f32((uint16_t)(aw[k] >> (16 * h)));
                 const float g = F16::to_f32((uint16_t)(gw[k] >> (16 * h)));
-                const float sig = 1.0f / (1.0f + expf(-g));
-                r[h] = a * sig;
+                r[h] = gate_product(a, g);
             }
             ow[k] = (uint32_t)F16::from_f32(r[0]) | ((uint32_t)F16::from_f32(r[1]) << 16);
         }
@@ -41,8 +40,7 @@ __global__ __launch_bounds__(256) void attn_output_gate_kernel(const uint16_t* _
     } else {
         const float a = F16::to_f32(attn_out[idx]);
         const float g = F16::to_f32(gate[idx]);
-        const float sig = 1.0f / (1.0f + expf(-g));
-        out[idx] = F16::from_f32(a * sig);
+        out[idx] = F16::from_f32(gate_product(a, g));
     }
 }
 

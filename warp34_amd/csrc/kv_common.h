@@ -66,6 +66,18 @@ struct BF16 {
     }
 };
 
+// attn * sigmoid(gate) as the gate operator computes it (ops/op_norms_rope_act.cu:742-759): an
+// fp32 product, which the caller then rounds to 16 bits.  The empty asm statement keeps the
+// compiler from folding the multiply and that conversion into one mixed-precision FMA, which
+// rounds once instead of twice and turns a product of -0 into +0.
+__device__ __forceinline__ float gate_product(float attn, float gate) {
+#pragma clang fp contract(off)
+    const float sig = 1.0f / (1.0f + expf(-gate));
+    float r = attn * sig;
+    asm volatile("" : "+v"(r));
+    return r;
+}
+
 // ---- request / visible-key-range lookup (op_kv_cache.cu:385-424) ------------------------
 struct RowRange {
     int req;     // owning request, -1 when the row is skipped

@@ -101,7 +101,32 @@ struct AttnParams {
     int rot_out;           // row-format kernel: V rows are stored rotated, rotate the output back
     int32_t* bal_table;    // balanced decode: per query token {first partial slot, pieces, token of the tile, -}
     uint32_t block_magic;  // floor(2^32 / block_size), see div_block
+    const uint16_t* gate;  // fp16 [tokens, q heads, 256] or null: out = fp16(out) * sigmoid(gate)
 };
+
+// A finished output row leaves the kernels here: lane l holds channels 4 l .. 4 l + 3.  With a gate
+// (the gated full-attention layers, model/forward.rs:1192-1211) the stored value is the attention
+// output rounded to its 16-bit type and then passed through the gate operator's arithmetic
+// (ops/op_norms_rope_act.cu:742-759), so it has the bits of the two calls in sequence.
+template <typename TQ>
+__device__ __forceinline__ void store_out_row(const AttnParams& P, size_t row, int lane, const float (&o)[4]) {
+    uint16_t h[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) h[k] = TQ::from_f32(o[k]);
+    if (P.gate != nullptr) {
+        const uint2 g = *reinterpret_cast<const uint2*>(P.gate + row * kHeadDim + 4 * lane);
+        const uint16_t gb[4] = {(uint16_t)g.x, (uint16_t)(g.x >> 16), (uint16_t)g.y, (uint16_t)(g.y >> 16)};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            h[k] = TQ::from_f32(gate_product(TQ::to_f32(h[k]), F16::to_f32(gb[k])));
+        }
+    }
+    uint2 ob;
+    ob.x = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
+    ob.y = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
+    *reinterpret_cast<uint2*>(P.out + row * kHeadDim + 4 * lane) = ob;
+}
+
 
 // token of k-slot (s, b, i) inside a unit: spreads the four 4-row groups of an MFMA over LDS
 // banks so that neither the K-row reads nor the V-column reads conflict.
@@ -1112,10 +1137,7 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
                 wht256_wave(v, lane);
 #pragma unroll
                 for (int k = 0; k < 4; ++k) v[k] = apply_sign(v[k], 4 * lane + k);
-                uint2 o;
-                o.x = (uint32_t)TQ::from_f32(v[0]) | ((uint32_t)TQ::from_f32(v[1]) << 16);
-                o.y = (uint32_t)TQ::from_f32(v[2]) | ((uint32_t)TQ::from_f32(v[3]) << 16);
-                *reinterpret_cast<uint2*>(P.out + row * kHeadDim + 4 * lane) = o;
+                store_out_row<TQ>(P, row, lane, v);
             }
         }
     }
@@ -1247,7 +1269,8 @@ __global__ __launch_bounds__(1024) void balanced_merge_kernel(const AttnParams P
     const int n_chunks = entry.y;
     if (n_chunks < 0 || n_chunks == 1) return;  // masked, or finished by the attention kernel
     if (n_chunks == 0) {                        // no visible key: zeros
-        if (grp == 0) *reinterpret_cast<uint2*>(P.out + (size_t)row * kHeadDim + 4 * lane) = uint2{0u, 0u};
+        const float zero[4] = {0.f, 0.f, 0.f, 0.f};
+        if (grp == 0) store_out_row<TQ>(P, (size_t)row, lane, zero);
         return;
     }
     const int col = entry.z * P.q_group + head % P.q_group;
@@ -1306,10 +1329,7 @@ __global__ __launch_bounds__(1024) void balanced_merge_kernel(const AttnParams P
 #pragma unroll
         for (int k = 0; k < 4; ++k) o[k] = apply_sign(o[k], 4 * lane + k);
     }
-    uint2 ob;
-    ob.x = (uint32_t)TQ::from_f32(o[0]) | ((uint32_t)TQ::from_f32(o[1]) << 16);
-    ob.y = (uint32_t)TQ::from_f32(o[2]) | ((uint32_t)TQ::from_f32(o[3]) << 16);
-    *reinterpret_cast<uint2*>(P.out + (size_t)row * kHeadDim + 4 * lane) = ob;
+    store_out_row<TQ>(P, (size_t)row, lane, o);
 }
 
 // Merge of the split-K partials (op_paged_attn.cu:1132-1218): m_tot = max m_s,
@@ -1418,10 +1438,7 @@ __global__ __launch_bounds__(1024) void split_merge_kernel(const float* part_acc
 #pragma unroll
         for (int k = 0; k < 4; ++k) o[k] = apply_sign(o[k], 4 * lane + k);
     }
-    uint2 ob;
-    ob.x = (uint32_t)TQ::from_f32(o[0]) | ((uint32_t)TQ::from_f32(o[1]) << 16);
-    ob.y = (uint32_t)TQ::from_f32(o[2]) | ((uint32_t)TQ::from_f32(o[3]) << 16);
-    *reinterpret_cast<uint2*>(P.out + (size_t)row * kHeadDim + 4 * lane) = ob;
+    store_out_row<TQ>(P, (size_t)row, lane, o);
 }
 
 }  // namespace w34
@@ -1523,13 +1540,14 @@ static int balanced_groups(int q_subgroups) {
 template <typename TQ>
 static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
                       const warp34_attention_batch* batch, const void* q, void* out, int num_q_heads,
-                      int force_single) {
+                      int force_single, const void* gate) {
     AttnParams P{};
     P.L = *layout;
     P.B = *batch;
     P.block_magic = block_magic_for(layout->block_size);
     P.q = (const uint16_t*)q;
     P.out = (uint16_t*)out;
+    P.gate = (const uint16_t*)gate;
     P.num_q_heads = num_q_heads;
     P.gqa = num_q_heads / layout->local_kv_heads;
     int q_group = P.gqa;
@@ -1616,13 +1634,14 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
 template <typename TQ, int KVF>
 static int launch_rows(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
                        const warp34_attention_batch* batch, const void* q, void* out, int num_q_heads,
-                       int force_single) {
+                       int force_single, const void* gate) {
     AttnParams P{};
     P.L = *layout;
     P.B = *batch;
     P.block_magic = block_magic_for(layout->block_size);
     P.q = (const uint16_t*)q;
     P.out = (uint16_t*)out;
+    P.gate = (const uint16_t*)gate;
     P.num_q_heads = num_q_heads;
     P.gqa = num_q_heads / layout->local_kv_heads;
     int q_group = P.gqa;
@@ -1717,13 +1736,15 @@ static bool prefill_tq4_applicable(const warp34_kv_layer_layout* layout, const w
 
 template <typename TQ, int KVF>
 static int launch_prefill_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
-                              const warp34_attention_batch* batch, const void* q, void* out, int num_q_heads) {
+                              const warp34_attention_batch* batch, const void* q, void* out, int num_q_heads,
+                              const void* gate) {
     AttnParams P{};
     P.L = *layout;
     P.B = *batch;
     P.block_magic = block_magic_for(layout->block_size);
     P.q = (const uint16_t*)q;
     P.out = (uint16_t*)out;
+    P.gate = (const uint16_t*)gate;
     P.part_acc = nullptr;
     P.part_ml = nullptr;
     P.num_q_heads = num_q_heads;
@@ -1807,7 +1828,7 @@ static int common_checks(const warp34_exec* ex, const warp34_kv_layer_layout* la
 template <typename TQ>
 static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
                            const warp34_attention_batch* batch, const void* q, void* out, int num_q_heads,
-                           int force_single) {
+                           int force_single, const void* gate = nullptr) {
     if (layout->local_kv_heads <= 0 || num_q_heads % layout->local_kv_heads != 0 || batch->num_reqs <= 0 ||
         !batch->query_start_loc || !batch->seq_lens_after || !batch->block_tables ||
         batch->max_blocks_per_req <= 0 || batch->sliding_window < 0 ||
@@ -1821,8 +1842,8 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
         const bool many_rows = batch->max_q_len >= 32 &&
                                (long long)batch->total_tokens * num_q_heads >= 128ll * kPfRows;
         if ((force_single || many_rows) && prefill_tq4_applicable(layout, batch, num_q_heads))
-            return launch_prefill_tq4<TQ, WARP34_KV_FORMAT_TQ4>(ex, layout, batch, q, out, num_q_heads);
-        return launch_tq4<TQ>(ex, layout, batch, q, out, num_q_heads, force_single);
+            return launch_prefill_tq4<TQ, WARP34_KV_FORMAT_TQ4>(ex, layout, batch, q, out, num_q_heads, gate);
+        return launch_tq4<TQ>(ex, layout, batch, q, out, num_q_heads, force_single, gate);
     }
     // 16-bit pages: the storage type must be the query type (FP16 pages with the f16 entry
     // point, BF16 pages with the bf16 one, as in the reference)
@@ -1833,8 +1854,8 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
         const bool many_rows = batch->max_q_len >= 32 &&
                                (long long)batch->total_tokens * num_q_heads >= 128ll * kPfRows;
         if (!force_single && many_rows && prefill_tq4_applicable(layout, batch, num_q_heads))
-            return launch_prefill_tq4<TQ, TQ::kStorageFormat>(ex, layout, batch, q, out, num_q_heads);
-        return launch_rows<TQ, TQ::kStorageFormat>(ex, layout, batch, q, out, num_q_heads, force_single);
+            return launch_prefill_tq4<TQ, TQ::kStorageFormat>(ex, layout, batch, q, out, num_q_heads, gate);
+        return launch_rows<TQ, TQ::kStorageFormat>(ex, layout, batch, q, out, num_q_heads, force_single, gate);
     }
     // 8-bit pages (the tail layers of the default TQ4 policy, cache.rs:87-109)
     if (is_kv8(layout, WARP34_KV_FORMAT_FP8_E4M3)) {
@@ -1843,16 +1864,16 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
         const bool many_rows = batch->max_q_len >= 32 &&
                                (long long)batch->total_tokens * num_q_heads >= 128ll * kPfRows;
         if ((force_single || many_rows) && prefill_tq4_applicable(layout, batch, num_q_heads))
-            return launch_prefill_tq4<TQ, WARP34_KV_FORMAT_FP8_E4M3>(ex, layout, batch, q, out, num_q_heads);
-        return launch_rows<TQ, WARP34_KV_FORMAT_FP8_E4M3>(ex, layout, batch, q, out, num_q_heads, force_single);
+            return launch_prefill_tq4<TQ, WARP34_KV_FORMAT_FP8_E4M3>(ex, layout, batch, q, out, num_q_heads, gate);
+        return launch_rows<TQ, WARP34_KV_FORMAT_FP8_E4M3>(ex, layout, batch, q, out, num_q_heads, force_single, gate);
     }
     if (is_kv8(layout, WARP34_KV_FORMAT_Q8_0)) {
         if (!kv8_geometry_ok(layout, q, out, 272)) return (int)hipErrorNotSupported;
         const bool many_rows = batch->max_q_len >= 32 &&
                                (long long)batch->total_tokens * num_q_heads >= 128ll * kPfRows;
         if ((force_single || many_rows) && prefill_tq4_applicable(layout, batch, num_q_heads))
-            return launch_prefill_tq4<TQ, WARP34_KV_FORMAT_Q8_0>(ex, layout, batch, q, out, num_q_heads);
-        return launch_rows<TQ, WARP34_KV_FORMAT_Q8_0>(ex, layout, batch, q, out, num_q_heads, force_single);
+            return launch_prefill_tq4<TQ, WARP34_KV_FORMAT_Q8_0>(ex, layout, batch, q, out, num_q_heads, gate);
+        return launch_rows<TQ, WARP34_KV_FORMAT_Q8_0>(ex, layout, batch, q, out, num_q_heads, force_single, gate);
     }
     return (int)hipErrorNotSupported;
 }
@@ -1987,6 +2008,26 @@ extern "C" int warp34_paged_attention_f16(const warp34_exec* ex, const warp34_kv
     }
     if (batch->total_tokens <= 0 || num_q_heads <= 0) return 0;
     return attention_entry<F16>(ex, layout, batch, q_in, attn_out, num_q_heads, 0);
+}
+
+// warp34_paged_attention_f16 with the output gate of the gated full-attention layers applied as
+// the rows leave the kernels (no counterpart in the reference, which calls
+// warp34_apply_attn_output_gate_f16 afterwards, model/forward.rs:1192-1211): attn_out receives the
+// bits of that sequence, the ungated output never goes to memory.  gate: fp16
+// [total_tokens, num_q_heads, 256], 8-byte aligned; rows the attention leaves untouched (masked
+// tokens and requests) stay untouched.
+extern "C" int warp34_paged_attention_gated_f16(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
+                                                const warp34_attention_batch* batch, const void* q_in,
+                                                const void* gate, void* attn_out, int num_q_heads) {
+    const int rc = common_checks(ex, layout, batch, q_in, attn_out, num_q_heads);
+    if (rc) return rc;
+    if (gate == nullptr) return (int)hipErrorInvalidValue;
+    if (layout->k_format == WARP34_KV_FORMAT_FP8_E4M3 || layout->v_format == WARP34_KV_FORMAT_FP8_E4M3) {
+        if (layout->head_dim != 256) return (int)hipErrorInvalidValue;
+    }
+    if (batch->total_tokens <= 0 || num_q_heads <= 0) return 0;
+    if ((((uintptr_t)gate) & 7u) != 0) return (int)hipErrorNotSupported;
+    return attention_entry<F16>(ex, layout, batch, q_in, attn_out, num_q_heads, 0, gate);
 }
 
 // op_kv_cache.cu:1192-1241

@@ -680,10 +680,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
 #pragma unroll
                 for (int k = 0; k < 4; ++k) v[k] = apply_sign(v[k], 4 * lane + k);
             }
-            uint2 o;
-            o.x = (uint32_t)TQ::from_f32(v[0]) | ((uint32_t)TQ::from_f32(v[1]) << 16);
-            o.y = (uint32_t)TQ::from_f32(v[2]) | ((uint32_t)TQ::from_f32(v[3]) << 16);
-            *reinterpret_cast<uint2*>(P.out + row * kHeadDim + 4 * lane) = o;
+            store_out_row<TQ>(P, row, lane, v);
         }
     }
 }

@@ -763,11 +763,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
 #pragma unroll
             for (int k = 0; k < 4; ++k) o[k] = apply_sign(o[k], 4 * lane + k);
         }
-        uint2 ob;
-        ob.x = (uint32_t)TQ::from_f32(o[0]) | ((uint32_t)TQ::from_f32(o[1]) << 16);
-        ob.y = (uint32_t)TQ::from_f32(o[2]) | ((uint32_t)TQ::from_f32(o[3]) << 16);
         const size_t row = (size_t)(tok0 + t) * P.num_q_heads + (size_t)(q_head_base + a);
-        *reinterpret_cast<uint2*>(P.out + row * kHeadDim + 4 * lane) = ob;
+        store_out_row<TQ>(P, row, lane, o);
     }
 }
 

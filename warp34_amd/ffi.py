@@ -109,6 +109,7 @@ SIGNATURES = {
     "warp34_paged_attention_f16_force_kernel_for_test":
         (C.c_int, [_EX, _LAY, _BAT, C.c_void_p, C.c_void_p, C.c_int, C.c_int]),
     "warp34_paged_attention_scratch_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int]),
+    "warp34_paged_attention_gated_f16": (C.c_int, [_EX, _LAY, _BAT, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]),
     "warp34_paged_attention_bf16_static_scratch": (C.c_int, [_EX, _LAY, _BAT, C.c_void_p, C.c_void_p, C.c_int]),
     "warp34_paged_attention_scratch_bytes_for_layout": (C.c_size_t, [_LAY, C.c_int, C.c_int, C.c_int, C.c_int]),
     # QK RMSNorm + RoPE on packed bf16 rows, optionally fused with the paged KV write
