@@ -30,6 +30,7 @@ SOURCES = [
     (os.path.join(CSRC, "paged_attn.hip"), ["-mllvm", "-amdgpu-kernarg-preload-count=12"]),
     (os.path.join(CSRC, "runtime.hip"), []),
     (os.path.join(HOST, "kv_host.cpp"), []),
+    (os.path.join(HOST, "prefix_cache.cpp"), []),
     (os.path.join(HOST, "kv_host_runtime.cpp"), []),
     (os.path.join(HOST, "synth.cpp"), ["-pthread"]),
 ]

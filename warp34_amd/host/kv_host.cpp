@@ -260,137 +260,7 @@ warp34_attention_batch StepMeta::batch_at(uint64_t dev_base, int mask_mode, floa
     return b;
 }
 
-// ---- prefix-shared pages ----------------------------------------------------------------------
-PrefixPageCache::PrefixPageCache(size_t page_size) : page_size_(page_size) {
-    nodes_.emplace_back();  // root
-    nodes_[0].live = true;
-}
-
-PrefixMatch PrefixPageCache::match_prefix(const std::vector<int32_t>& token_ids) {
-    PrefixMatch m;
-    const size_t aligned = (token_ids.size() / page_size_) * page_size_;
-    int cur = 0;
-    ++clock_;
-    for (size_t off = 0; off < aligned; off += page_size_) {
-        const std::vector<int32_t> key(token_ids.begin() + (long)off, token_ids.begin() + (long)(off + page_size_));
-        auto it = nodes_[cur].children.find(key);
-        if (it == nodes_[cur].children.end()) break;
-        cur = it->second;
-        nodes_[cur].last_use = clock_;
-        m.kv_pages.push_back(nodes_[cur].page);
-    }
-    m.matched_tokens = m.kv_pages.size() * page_size_;
-    m.last_node = cur;
-    return m;
-}
-
-void PrefixPageCache::inc_lock_ref(int node) {
-    for (int n = node; n > 0; n = nodes_[n].parent) ++nodes_[n].lock_ref;
-}
-
-void PrefixPageCache::dec_lock_ref(int node) {
-    for (int n = node; n > 0; n = nodes_[n].parent)
-        if (nodes_[n].lock_ref > 0) --nodes_[n].lock_ref;
-}
-
-int PrefixPageCache::insert(const std::vector<int32_t>& token_ids, const std::vector<int32_t>& kv_pages,
-                            std::vector<int32_t>* duplicate_pages) {
-    const size_t whole = std::min(token_ids.size() / page_size_, kv_pages.size());
-    int cur = 0;
-    ++clock_;
-    for (size_t p = 0; p < whole; ++p) {
-        const std::vector<int32_t> key(token_ids.begin() + (long)(p * page_size_),
-                                       token_ids.begin() + (long)((p + 1) * page_size_));
-        auto it = nodes_[cur].children.find(key);
-        if (it != nodes_[cur].children.end()) {
-            const int child = it->second;
-            if (nodes_[child].page != kv_pages[p] && duplicate_pages != nullptr)
-                duplicate_pages->push_back(kv_pages[p]);
-            nodes_[child].last_use = clock_;
-            cur = child;
-            continue;
-        }
-        int id;
-        if (!free_ids_.empty()) {
-            id = free_ids_.back();
-            free_ids_.pop_back();
-            nodes_[id] = Node();
-        } else {
-            id = (int)nodes_.size();
-            nodes_.emplace_back();
-        }
-        Node& n = nodes_[id];
-        n.parent = cur;
-        n.key = key;
-        n.page = kv_pages[p];
-        n.last_use = clock_;
-        n.live = true;
-        nodes_[cur].children.emplace(key, id);
-        ++live_nodes_;
-        cur = id;
-    }
-    return cur;
-}
-
-EvictResult PrefixPageCache::evict_full_pages(size_t num_pages) {
-    EvictResult r;
-    while (r.freed_kv_pages.size() < num_pages) {
-        int victim = -1;
-        for (int i = 1; i < (int)nodes_.size(); ++i) {
-            const Node& n = nodes_[i];
-            if (!n.live || n.lock_ref > 0 || !n.children.empty()) continue;
-            if (victim < 0 || n.last_use < nodes_[victim].last_use ||
-                (n.last_use == nodes_[victim].last_use && i > victim))  // deeper pages of one insert first
-                victim = i;
-        }
-        if (victim < 0) break;
-        Node& v = nodes_[victim];
-        r.freed_kv_pages.push_back(v.page);
-        nodes_[v.parent].children.erase(v.key);
-        v.live = false;
-        v.children.clear();
-        free_ids_.push_back(victim);
-        --live_nodes_;
-    }
-    return r;
-}
-
-size_t PrefixPageCache::full_evictable_pages() const {
-    size_t n = 0;
-    for (size_t i = 1; i < nodes_.size(); ++i)
-        if (nodes_[i].live && nodes_[i].lock_ref == 0) ++n;
-    return n;
-}
-
-size_t PrefixPageCache::full_protected_pages() const {
-    size_t n = 0;
-    for (size_t i = 1; i < nodes_.size(); ++i)
-        if (nodes_[i].live && nodes_[i].lock_ref > 0) ++n;
-    return n;
-}
-
-void RequestPages::restore_prefix_hit(PrefixPageCache& cache, const std::vector<int32_t>& prompt_tokens,
-                                      const PrefixMatch& m) {
-    if (m.matched_tokens == 0) return;
-    cache.inc_lock_ref(m.last_node);
-    token_ids.assign(prompt_tokens.begin(), prompt_tokens.begin() + (long)m.matched_tokens);
-    kv_pages = m.kv_pages;
-    protected_pages = kv_pages.size();
-    last_locked_node = m.last_node;
-    page_size = cache.page_size();
-}
-
-std::vector<int32_t> RequestPages::rollback_uncommitted_kv_pages() {
-    size_t needed = page_size ? (token_ids.size() + page_size - 1) / page_size : kv_pages.size();
-    needed = std::max(needed, protected_pages);
-    std::vector<int32_t> freed;
-    if (kv_pages.size() > needed) {
-        freed.assign(kv_pages.begin() + (long)needed, kv_pages.end());
-        kv_pages.resize(needed);
-    }
-    return freed;
-}
-
+// ---- page reservation (model/batch.rs:57-103); the prefix tree itself lives in prefix_cache.cpp ----
 bool reserve_kv_pages_from(KvPool& pool, PrefixPageCache& cache, std::vector<int32_t>* dst, size_t target_pages) {
     if (dst->size() >= target_pages) return true;
     const size_t missing = target_pages - dst->size();

@@ -166,59 +166,135 @@ StepMeta pack_step_meta(const std::vector<int32_t>& tokens, const std::vector<in
                         size_t block_size, int32_t state_in_slot = -1, int32_t state_out_slot = -1,
                         bool has_initial_state = false);
 
-// ---- prefix-shared pages (radix.rs page side) -------------------------------------------------
+// ---- prefix-shared pages (radix.rs:1-1041, 1129-1157, 1234-1245) -------------------------------
+// A radix tree over token ids whose edges are whole pages: a node holds a run of pages (key =
+// tokens, value = physical page ids, optionally the draft model's pages beside them) and,
+// optionally, the handle of a recurrent-state snapshot taken at the end of its key.  The handle
+// is opaque here (the state pools are not part of this library); what the tree does with it is
+// what keeps the page side correct: a prefix only counts as a hit up to the deepest node that
+// still has a snapshot, internal nodes may lose theirs (tombstones) while their pages stay for
+// longer descendants, leaves never are tombstones.
+//
+// Two lock counts per node: full_lock_ref pins the pages of every node on [node .. root),
+// state_lock_ref pins the snapshot of the locked node alone (full >= state everywhere).  Two
+// recency orders: a hit refreshes the page order along the whole path and the snapshot order on
+// the hit node only.  Both orders are intrusive doubly linked lists through the node arena, so a
+// touch is O(1).
 struct PrefixMatch {
-    size_t matched_tokens = 0;       // whole pages only
-    std::vector<int32_t> kv_pages;   // shared physical pages, in sequence order
-    int last_node = 0;               // 0 = root (nothing matched)
+    size_t kv_matched_tokens = 0;    // whole-page prefix present in the tree, snapshot or not
+    size_t matched_tokens = 0;       // usable prefix: up to last_node (multiple of page_size)
+    std::vector<int32_t> kv_pages;   // matched_tokens / page_size shared pages, in sequence order
+    std::vector<int32_t> draft_pages;
+    bool has_state = false;          // false only when nothing matched
+    int32_t state_slot = -1;
+    int last_node = 0;               // deepest matched node with a snapshot; 0 = root
+    size_t state_branching_seqlen = 0;  // > 0: pages matched past last_node; chunk-aligned length
+};
+struct PrefixInsertResult {
+    size_t existing_prefix_tokens = 0;   // tokens of the insert that were in the tree already
+    bool state_already_existed = false;  // true: the caller keeps (frees) the handle it offered
+    std::vector<int32_t> freed_duplicate_kv_pages;  // caller's pages superseded by tree pages
+    std::vector<int32_t> freed_duplicate_draft_pages;
+    int terminal_node = 0;
 };
 struct EvictResult {
     std::vector<int32_t> freed_kv_pages;
+    std::vector<int32_t> freed_draft_pages;
+    std::vector<int32_t> freed_state_slots;
 };
 
-// Page-granular prefix tree over token ids: each node owns exactly one full page.  Nodes on a
-// locked path are never evicted; eviction removes least-recently-used unlocked leaves.
 class PrefixPageCache {
 public:
-    explicit PrefixPageCache(size_t page_size);
+    // state_chunk_tokens: spacing of snapshots, a multiple of page_size (0 = page_size).
+    explicit PrefixPageCache(size_t page_size, size_t state_chunk_tokens = 0);
+    void reset();
     size_t page_size() const { return page_size_; }
-    // Longest whole-page prefix of token_ids already cached (radix.rs:383-490); refreshes LRU.
+    size_t state_chunk_tokens() const { return chunk_; }
+    bool disable = false;  // every call becomes a no-op / miss (radix.rs:392,497,563)
+
+    // Longest whole-page prefix of token_ids that ends in a node with a snapshot
+    // (radix.rs:383-490).  A partial match of a node splits it.  Refreshes both recency orders.
     PrefixMatch match_prefix(const std::vector<int32_t>& token_ids);
-    // Locks / unlocks the path [node .. root) (radix.rs:494-550).
+    // radix.rs:494-550.  dec on a count of zero throws std::logic_error.
     void inc_lock_ref(int node);
     void dec_lock_ref(int node);
-    // Donates the whole pages of (token_ids, kv_pages) to the tree.  Pages whose prefix is
-    // already cached under another physical page are returned as duplicates for the caller to
-    // free; returns the node of the last whole page.
-    int insert(const std::vector<int32_t>& token_ids, const std::vector<int32_t>& kv_pages,
-               std::vector<int32_t>* duplicate_pages);
-    // Evicts up to num_pages unlocked leaf pages, least recently used first (radix.rs:950-981).
+    // Donates page-aligned (token_ids, kv_pages[, draft_pages], state_slot) (radix.rs:552-699).
+    // The first prev_protected_pages pages are the tree's own (the request got them from a hit);
+    // pages behind them whose tokens are already cached are returned as duplicates.
+    // Throws std::invalid_argument on lengths that do not fit.
+    PrefixInsertResult insert(const std::vector<int32_t>& token_ids, const std::vector<int32_t>& kv_pages,
+                              const std::vector<int32_t>& draft_pages, int32_t state_slot,
+                              size_t prev_protected_pages);
+    // Deletes unlocked leaves, least recently used first, decode tails before anything else, until
+    // at least num_pages pages are free; tombstone ancestors that become leaves go with them
+    // (radix.rs:701-756, 950-981).
     EvictResult evict_full_pages(size_t num_pages);
-    size_t full_evictable_pages() const;
-    size_t full_protected_pages() const;
-    size_t cached_pages() const { return live_nodes_; }
+    // Frees snapshots (radix.rs:907-948): superseded single-child internal nodes first (no page
+    // freed), then reclaimable decode-tail leaves, then snapshot recency order.
+    EvictResult evict_state_slots(size_t num_slots);
+    bool has_evictable_internal_state() const;
+    // Drops every node's claim on `slot` (radix.rs:856-886); `slot` itself is not reported back.
+    EvictResult invalidate_state_slot(int32_t slot);
+    // radix.rs:772-776: the leaf holds generated tokens nobody has verified yet.
+    void mark_node_decode_tail(int node);
+    bool can_recycle_locked_state(int node) const;  // radix.rs:838-844
+    // Takes the snapshot handle of an unlocked-state internal node (radix.rs:888-899); -1 if none.
+    int32_t reclaim_internal_state(int node);
+    void set_node_state(int node, int32_t slot);  // a live node without a snapshot gets one
+    std::vector<int32_t> collect_node_kv_pages(int node) const;  // radix.rs:180-193
+
+    size_t full_evictable_pages() const { return full_evictable_pages_; }
+    size_t full_protected_pages() const { return full_protected_pages_; }
+    size_t state_evictable_slots() const { return state_evictable_slots_; }
+    size_t state_protected_slots() const { return state_protected_slots_; }
+    size_t cached_pages() const { return full_evictable_pages_ + full_protected_pages_; }
+    bool node_alive(int node) const { return node >= 0 && (size_t)node < nodes_.size() && nodes_[node].alive; }
+    size_t arena_size() const { return nodes_.size(); }
+    uint64_t total_lookups = 0, total_lookup_tokens = 0, total_hit_tokens = 0, total_state_hits = 0;
+    double hit_rate() const { return total_lookup_tokens ? (double)total_hit_tokens / (double)total_lookup_tokens : 0.0; }
+    // Recomputes the four counters and checks the lock / tombstone / list invariants
+    // (radix.rs:983-1041); on failure returns false and says why.
+    bool sanity_check(std::string* why = nullptr) const;
 
 private:
     struct Node {
         int parent = -1;
-        std::vector<int32_t> key;  // page_size tokens
-        int32_t page = -1;
-        int lock_ref = 0;
-        uint64_t last_use = 0;
-        std::map<std::vector<int32_t>, int> children;
-        bool live = false;
+        std::map<std::vector<int32_t>, int> children;  // keyed by the child's first page
+        std::vector<int32_t> key, pages, draft_pages;
+        bool has_state = false;
+        int32_t state_slot = -1;
+        size_t full_lock_ref = 0, state_lock_ref = 0;
+        bool decode_tail = false, alive = false;
+        int lru_prev[2] = {-1, -1}, lru_next[2] = {-1, -1};  // [0] page order, [1] snapshot order
+        bool in_lru[2] = {false, false};
     };
+    enum { kFull = 0, kState = 1 };
+    int alloc_node();
+    void retire(int id);
+    void lru_push_mru(int which, int id);
+    void lru_remove(int which, int id);
+    void lru_touch(int which, int id);
+    void touch_path(int node);
+    size_t common_pages(const std::vector<int32_t>& key, const int32_t* rest, size_t rest_len) const;
+    int split_node(int child, size_t split_tokens);
+    void delete_leaf(int leaf, EvictResult* out);
+    bool has_verified_state_below(int node) const;
+    bool superseded_linear_internal(int node) const;
+    bool reclaimable_decode_tail_leaf(int node) const;
+
     std::vector<Node> nodes_;
     std::vector<int> free_ids_;
-    size_t page_size_;
-    size_t live_nodes_ = 0;
-    uint64_t clock_ = 0;
+    int lru_head_[2] = {-1, -1}, lru_tail_[2] = {-1, -1};  // head = least recently used
+    size_t page_size_, chunk_;
+    size_t full_evictable_pages_ = 0, full_protected_pages_ = 0;
+    size_t state_evictable_slots_ = 0, state_protected_slots_ = 0;
 };
 
 // A request's page list: shared prefix pages first (protected), private pages behind them.
 struct RequestPages {
     std::vector<int32_t> token_ids;  // committed tokens
     std::vector<int32_t> kv_pages;
+    std::vector<int32_t> draft_pages;
     size_t protected_pages = 0;
     int last_locked_node = 0;
     size_t page_size = 0;
@@ -229,6 +305,18 @@ struct RequestPages {
     // Drops private tail pages beyond ceil(committed / page_size); never a protected page
     // (radix.rs:1234-1245).  Returns the pages to hand back to the pool.
     std::vector<int32_t> rollback_uncommitted_kv_pages();
+    // The page side of a donation (radix.rs:1247-1380): the first cache_len committed tokens
+    // (page-aligned, beyond the protected prefix) and their pages go to the tree with the snapshot
+    // handle state_slot; pages the tree already had are swapped for the tree's and the request's
+    // copies returned; the lock moves to the new terminal node, or is dropped when the request
+    // finishes, in which case the private tail pages are returned as well and a leaf that extends
+    // a protected prompt is marked as an unverified decode tail.
+    struct Donation {
+        size_t donated_seq_len = 0;
+        bool state_already_existed = false;
+        std::vector<int32_t> freed_kv_pages, freed_draft_pages;
+    };
+    Donation donate_pages(PrefixPageCache& cache, size_t cache_len, int32_t state_slot, bool finish_req);
 };
 
 // Grows dst to target_pages: evicts the deficit from the prefix cache in one batch, then takes
