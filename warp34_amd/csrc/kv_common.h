@@ -32,12 +32,28 @@ __device__ __constant__ constexpr uint32_t kSignMask[8] = {
     0xba639274u, 0xe2eb25d0u, 0xfde0ee14u, 0x36b5bda1u,
 };
 
+// Word w (0..7) of the mask for an index that differs between lanes, picked from the eight
+// immediates with three levels of selects.  A lookup in the constant array would be a vector
+// memory load: a round trip on the spot, and a wait that also waits for every load issued before it.
+__device__ __forceinline__ uint32_t sign_word(int w) {
+    const uint32_t a = (w & 1) ? 0x48974752u : 0x29e1d357u;
+    const uint32_t b = (w & 1) ? 0xf1297e2au : 0xeebc0de4u;
+    const uint32_t c = (w & 1) ? 0xe2eb25d0u : 0xba639274u;
+    const uint32_t d = (w & 1) ? 0x36b5bda1u : 0xfde0ee14u;
+    const uint32_t ab = (w & 2) ? b : a;
+    const uint32_t cd = (w & 2) ? d : c;
+    return (w & 4) ? cd : ab;
+}
+static_assert(kSignMask[0] == 0x29e1d357u && kSignMask[1] == 0x48974752u && kSignMask[2] == 0xeebc0de4u &&
+                  kSignMask[3] == 0xf1297e2au && kSignMask[4] == 0xba639274u && kSignMask[5] == 0xe2eb25d0u &&
+                  kSignMask[6] == 0xfde0ee14u && kSignMask[7] == 0x36b5bda1u,
+              "sign_word() repeats the mask");
 __device__ __forceinline__ bool sign_is_negative(int i) {
-    return (kSignMask[i >> 5] >> (i & 31)) & 1u;
+    return (sign_word(i >> 5) >> (i & 31)) & 1u;
 }
 // multiply by the +-1 sign of element i (exact: flips the sign bit)
 __device__ __forceinline__ float apply_sign(float v, int i) {
-    return __uint_as_float(__float_as_uint(v) ^ (((kSignMask[i >> 5] >> (i & 31)) & 1u) << 31));
+    return __uint_as_float(__float_as_uint(v) ^ (((sign_word(i >> 5) >> (i & 31)) & 1u) << 31));
 }
 
 constexpr int kHeadDim = 256;

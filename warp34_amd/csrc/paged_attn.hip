@@ -71,7 +71,7 @@ __host__ __device__ constexpr int ml_offset_for(int nt) {  // (m, l) tables of t
 __host__ __device__ constexpr int smem_bytes_for(int nt) {
     return ml_offset_for(nt) + (waves_for(nt) + 1) * nt * 16 * 2 * 4;
 }
-static_assert(merge_floats_for(1) * 4 <= kLutBytes + waves_for(1) * kStageTq4, "merge regions alias the table and the staging areas only");
+static_assert(merge_floats_for(1) * 4 <= waves_for(1) * kStageTq4, "merge regions alias the staging areas only");
 static_assert(smem_bytes_for(1) <= 160 * 1024, "decode LDS budget");
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kNegBig = -1.0e30f;  // "minus infinity" that stays finite under subtraction
@@ -102,6 +102,9 @@ struct AttnParams {
     int32_t* bal_table;    // balanced decode: per query token {first partial slot, pieces, token of the tile, -}
     uint32_t block_magic;  // floor(2^32 / block_size), see div_block
     const uint16_t* gate;  // fp16 [tokens, q heads, 256] or null: out = fp16(out) * sigmoid(gate)
+    // chunk geometry of a tile whose keys are exactly [0, max_seq_len): worked out on the host, so a
+    // request that is as long as the host's bound needs no division on the device (TQ4 decode kernel)
+    int spec_units, spec_upc, spec_chunks;
 };
 
 // A finished output row leaves the kernels here: lane l holds channels 4 l .. 4 l + 3.  With a gate
@@ -442,7 +445,7 @@ __device__ __forceinline__ void wait_lds_reads() { asm volatile("s_waitcnt lgkmc
 // A staging area holds one 32-token unit as it lies in the pages, written by LDS-direct loads:
 // K rows 0-31, then V rows 0-31, 132 bytes each (four runs of 16 rows = 2112 bytes).
 template <typename TQ, bool BAL>
-__device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, const BalItem& item) {
+__device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, const BalItem& item, bool build_table) {
     constexpr int kWaves = kTq4Waves;
     uint8_t* stage_all = smem + kLutBytes;
 
@@ -465,10 +468,56 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
     const int q_head_base = kv_head * P.gqa + (kv_sub - kv_head * P.q_subgroups) * P.q_group;
     const int chunk = BAL ? 0 : (int)blockIdx.x;
 
-    // Work that depends on nothing goes first so that it overlaps the request lookup below:
-    // the raw query rows of this wave's columns and the table.  The first token of the tile is
-    // guessed (exact when every request has a whole number of tiles); a wrong guess is
-    // corrected after the lookup.
+    // The request lookup goes first: its loads head the longest dependency chain of the prologue
+    // (lengths -> chunk geometry -> page ids -> the first K / V loads).
+    bool req_hit = false;
+    int req = -1, rq_start = 0, rq_end = 0, seq_after = 0, ctx_before = 0, tile_in_req = 0;
+    int spec_slot_base = -1, spec_vec = -1;
+    int a_lo = 0, a_hi = 0, a_sa = 0, a_cb = 0, a_rm = 0;
+    if constexpr (BAL) {
+        req = item.req;
+        rq_start = item.rq_start;
+        rq_end = item.rq_end;
+        seq_after = item.seq_after;
+        ctx_before = item.ctx_before;
+        req_hit = true;
+        // the piece's first unit is known: its block-table slice is requested together with the
+        // query rows
+        spec_slot_base = div_block(item.u_begin * kUnit, P);
+        const int slot = spec_slot_base + lane;
+        if (slot < B.max_blocks_per_req) spec_vec = B.block_tables[(size_t)req * B.max_blocks_per_req + slot];
+    } else if (P.tiles_by_request) {
+        req = tile_z;  // < num_reqs by the launch geometry
+        // Speculative block-table load, in flight together with the request's lengths: it
+        // assumes that the request's length is the host's bound max_seq_len.  When the guess is
+        // wrong the ids are fetched again below, so it changes the latency only, never the result.
+        if (B.sliding_window <= 0 && B.max_seq_len > 0) {
+            spec_slot_base = div_block(chunk * P.spec_upc * kUnit, P);
+            const int slot = spec_slot_base + lane;
+            if (slot < B.max_blocks_per_req)
+                spec_vec = B.block_tables[(size_t)req * B.max_blocks_per_req + slot];
+        }
+        // one vector load per array (all lanes the same address), no scalar-cache round trip;
+        // the values are made scalar after the table has been built, so that the build overlaps
+        // the round trip
+        a_lo = B.query_start_loc[req];
+        a_hi = B.query_start_loc[req + 1];
+        a_sa = B.seq_lens_after[req];
+        a_cb = B.context_lens_before != nullptr ? B.context_lens_before[req] : 0;
+        a_rm = B.valid_req_mask != nullptr ? (int)B.valid_req_mask[req] : 1;
+    } else {
+        const TileInfo ti = locate_tile(P, tile_z, lane);
+        req = ti.req;
+        rq_start = ti.rq_start;
+        rq_end = ti.rq_end;
+        seq_after = ti.seq_after;
+        ctx_before = ti.ctx_before;
+        tile_in_req = ti.tile_in_req;
+        req_hit = ti.hit;
+    }
+    // While the request's lengths are on their way: the raw query rows of this wave's columns and
+    // the table.  The first token of the tile is guessed (exact when every request has a whole
+    // number of tiles); a wrong guess is corrected after the lookup.
     const int tok_guess = BAL ? item.rq_start
                               : min(P.tiles_by_request ? tile_z : tile_z * P.tok_tile, B.total_tokens - 1);
     constexpr int kColsPerWave = (16 + kWaves - 1) / kWaves;
@@ -497,62 +546,20 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
     };
     load_tok_ok(tok_guess);
 
-    bool req_hit = false;
-    int req = -1, rq_start = 0, rq_end = 0, seq_after = 0, ctx_before = 0, tile_in_req = 0;
-    int spec_slot_base = -1, spec_vec = -1;
-    int a_lo = 0, a_hi = 0, a_sa = 0, a_cb = 0, a_rm = 0;
-    if constexpr (BAL) {
-        req = item.req;
-        rq_start = item.rq_start;
-        rq_end = item.rq_end;
-        seq_after = item.seq_after;
-        ctx_before = item.ctx_before;
-        req_hit = true;
-        // the piece's first unit is known: its block-table slice is requested together with the
-        // query rows
-        spec_slot_base = fast_div(item.u_begin * kUnit, L.block_size);
-        const int slot = spec_slot_base + lane;
-        if (slot < B.max_blocks_per_req) spec_vec = B.block_tables[(size_t)req * B.max_blocks_per_req + slot];
-    } else if (P.tiles_by_request) {
-        req = tile_z;  // < num_reqs by the launch geometry
-        // Speculative block-table load, in flight together with the request's lengths: it
-        // assumes that the request's length is the host's bound max_seq_len.  When the guess is
-        // wrong the ids are fetched again below, so it changes the latency only, never the result.
-        if (B.sliding_window <= 0 && B.max_seq_len > 0) {
-            const ChunkGeom sg = chunk_geom(0, B.max_seq_len - 1, P.max_chunks, P.min_upc);
-            spec_slot_base = fast_div((sg.u_first + chunk * sg.upc) * kUnit, L.block_size);
-            const int slot = spec_slot_base + lane;
-            if (slot < B.max_blocks_per_req)
-                spec_vec = B.block_tables[(size_t)req * B.max_blocks_per_req + slot];
-        }
-        // one vector load per array (all lanes the same address), no scalar-cache round trip;
-        // the values are made scalar after the table has been built, so that the build overlaps
-        // the round trip
-        a_lo = B.query_start_loc[req];
-        a_hi = B.query_start_loc[req + 1];
-        a_sa = B.seq_lens_after[req];
-        a_cb = B.context_lens_before != nullptr ? B.context_lens_before[req] : 0;
-        a_rm = B.valid_req_mask != nullptr ? (int)B.valid_req_mask[req] : 1;
-    } else {
-        const TileInfo ti = locate_tile(P, tile_z, lane);
-        req = ti.req;
-        rq_start = ti.rq_start;
-        rq_end = ti.rq_end;
-        seq_after = ti.seq_after;
-        ctx_before = ti.ctx_before;
-        tile_in_req = ti.tile_in_req;
-        req_hit = ti.hit;
-    }
-    {
-        // entry e = (gain*centroid[e & 15], gain*centroid[e >> 4]) as packed fp16, 64 copies:
-        // 16 KB per pass of 1024 "slots" of 16 bytes each
-        constexpr int kThreads = kWaves * 64;
-        const u4* dummy = nullptr;
-        (void)dummy;
-        for (int slot = tid; slot < kLutBytes / 16; slot += kThreads) {
-            const int e = slot >> 4;  // 16 slots of 16 bytes per entry
-            const uint32_t v = pack_h2(kLutGain * centroid_of_code(e & 15), kLutGain * centroid_of_code(e >> 4));
-            *reinterpret_cast<u4*>(smem + slot * 16) = u4{v, v, v, v};
+    if (build_table) {
+        // entry e = (gain*centroid[e & 15], gain*centroid[e >> 4]) as packed fp16, 64 copies of 4 bytes.
+        // Thread t writes the 16-byte slots t + 512 i (conflict-free), i.e. entries (t >> 4) + 32 i:
+        // their low code (t >> 4) & 15 is the thread's own, their high code (t >> 8) + 2 i is the
+        // same in the whole wave.  Lane j < 16 computes centroid j once; everything else is lane
+        // traffic, so the build costs a few dozen instructions per wave.
+        static_assert(kWaves == 8, "table build: 512 threads");
+        const uint32_t c_bits = (uint32_t)F16::from_f32(kLutGain * centroid_of_code(lane & 15));
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute(((tid >> 4) & 15) << 2, (int)c_bits);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)c_bits, (wave >> 2) + 2 * i);
+            const uint32_t v = lo | (hi << 16);
+            *reinterpret_cast<u4*>(smem + (tid + 512 * i) * 16) = u4{v, v, v, v};
         }
     }
 
@@ -574,13 +581,18 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
     int tile_tokens = rq_end - tok0;
     if (tile_tokens > P.tok_tile) tile_tokens = P.tok_tile;
 
-    // per-lane column info
-    int col_lo, col_hi;
-    bool col_ok;
+    // Column info: per lane (= per query column) the visible key range, and for the tile the union
+    // and the intersection of the ranges.  Without a token mask and a window -- the common case --
+    // the tile-wide values follow from scalars (every token of the tile is live, the ranges start
+    // at 0 and their ends grow with the token: the union is the last token's range, the
+    // intersection the first one's), and the per-lane part waits until the first loads are out.
+    int col_lo = 0, col_hi = -1;
+    bool col_ok = false;
     int u_lo = 0x7fffffff, u_hi = -1;  // union of the visible ranges
     int i_lo = 0, i_hi = 0x7fffffff;   // intersection of the visible ranges
-    uint32_t ok_mask;                  // bit c: column c is live (wave-uniform)
-    {
+    uint32_t ok_mask = 0u;             // bit c: column c is live (wave-uniform)
+    const bool simple = B.valid_token_mask == nullptr && B.sliding_window <= 0;
+    auto column_info = [&](bool accumulate) {
         const int t = fast_div(n, P.q_group);
         const int tok = tok0 + t;
         const bool ok = t < tile_tokens && tok_ok;
@@ -592,7 +604,7 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         col_ok = ok;
         col_lo = ok ? mn : 0;
         col_hi = ok ? mx : -1;
-        if (ok) {
+        if (accumulate && ok) {
             i_lo = max(i_lo, mn);
             i_hi = min(i_hi, mx);
             if (mn <= mx) {
@@ -601,11 +613,9 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
             }
         }
         ok_mask = (uint32_t)(__ballot(ok) & 0xFFFFull);
-    }
-    if (B.valid_token_mask == nullptr && B.sliding_window <= 0) {
-        // Common case, no cross-lane traffic: every token of the tile is live, the ranges start
-        // at 0 and their ends grow with the token, so the union is the last token's range and
-        // the intersection the first one's.
+    };
+    if (simple) {
+        if (tok0 >= B.total_tokens) return;  // no live column
         const int q_off0 = tok0 - rq_start;
         const bool window = B.mask_mode == WARP34_ATTN_MASK_NONCAUSAL_WINDOW;
         int hi_first = window ? seq_after - 1 : ctx_before + q_off0;
@@ -617,6 +627,7 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         i_lo = 0;
         i_hi = hi_first;
     } else {
+        column_info(true);
 #pragma unroll
         for (int off = 1; off < 16; off <<= 1) {
             u_lo = min(u_lo, __shfl_xor(u_lo, off, 64));
@@ -624,8 +635,8 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
             i_lo = max(i_lo, __shfl_xor(i_lo, off, 64));
             i_hi = min(i_hi, __shfl_xor(i_hi, off, 64));
         }
+        if (ok_mask == 0u) return;  // whole tile masked: outputs untouched
     }
-    if (ok_mask == 0u) return;  // whole tile masked: outputs untouched
     if (u_hi < 0) u_lo = 0;
     u_lo = __builtin_amdgcn_readfirstlane(u_lo);
     u_hi = __builtin_amdgcn_readfirstlane(u_hi);
@@ -640,7 +651,11 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         cu_first = item.u_begin;
         cu_end = item.u_end;
     } else {
-        g = chunk_geom(u_lo, u_hi, P.max_chunks, P.min_upc);
+        if (u_lo == 0 && B.max_seq_len > 0 && u_hi == B.max_seq_len - 1) {
+            g = ChunkGeom{0, P.spec_units, P.spec_upc, P.spec_chunks};  // as long as the host's bound
+        } else {
+            g = chunk_geom(u_lo, u_hi, P.max_chunks, P.min_upc);
+        }
         if (chunk >= g.n_chunks) return;
         cu_first = g.u_first + chunk * g.upc;
         cu_end = cu_first + g.upc;
@@ -659,7 +674,7 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
     // the id of slot slot_base + l, a unit picks its two ids with readlane.  No scalar memory
     // loads remain in the loop (they share the LDS wait counter and would serialise it).
     const int32_t* req_blocks = B.block_tables + (size_t)req * B.max_blocks_per_req;
-    int slot_base = fast_div(cu_first * kUnit, L.block_size);
+    int slot_base = div_block(cu_first * kUnit, P);
     int page_vec;
     auto load_page_vec = [&]() {
         const int slot = slot_base + lane;
@@ -732,11 +747,17 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
     } else {
         load_page_vec();
     }
+    // The raw query rows are consumed after the first K / V loads have gone out.  Loads return in
+    // order, so a wait for them placed behind those loads would wait for the K / V data as well:
+    // the (empty) statement makes the compiler finish its own loads here, where they have long landed.
+#pragma unroll
+    for (int c = 0; c < kColsPerWave; ++c) asm volatile("" ::"v"(q_raw[c].x), "v"(q_raw[c].y));
     if (unit < cu_end) {
         locate_unit(unit);
         issue_k();
         issue_v();
     }
+    if (simple) column_info(false);
 
     // ---- prologue: the query operand table ---------------------------------------------------------
     // B operands of the QK MFMAs, nine per lane (five for the first half-row, four for the second),
@@ -1053,7 +1074,7 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
     // start 4 banks apart.
     constexpr int kColStride = 260;
     constexpr int kRegion = 8 * kColStride;
-    float* xbuf = reinterpret_cast<float*>(smem);
+    float* xbuf = reinterpret_cast<float*>(stage_all);  // the staging areas are idle now; the table stays
     // [kWaves][16][2], then (m_tot, l_tot)[16]: in an area of its own, a wave publishes its state
     // while others are still in their loops
     float* mlbuf = reinterpret_cast<float*>(smem + ml_offset_for(1));
@@ -1149,7 +1170,7 @@ __global__ __launch_bounds__(kTq4Waves * 64, 1) void paged_attn_tq4_kernel(const
     extern __shared__ __align__(16) uint8_t smem[];
     // lut_read() addresses the table absolutely: the dynamic block starts at LDS address 0 because
     // the kernel has no static LDS (checked on the host before the first launch)
-    tq4_tile<TQ, false>(P, smem, BalItem{});
+    tq4_tile<TQ, false>(P, smem, BalItem{}, true);
 }
 
 // Balanced decode: grid = (groups, kv head x q subgroup).  Every wave computes the plan (the
@@ -1246,7 +1267,12 @@ __device__ __forceinline__ void bal_for_each_piece(const AttnParams& P, TileFn&&
 template <typename TQ>
 __global__ __launch_bounds__(kTq4Waves * 64, 1) void paged_attn_tq4_balanced_kernel(const AttnParams P) {
     extern __shared__ __align__(16) uint8_t smem[];
-    bal_for_each_piece(P, [&](const BalItem& it) { tq4_tile<TQ, true>(P, smem, it); });
+    // the pair table survives a piece (the merge regions lie in the staging areas): built once
+    bool first = true;
+    bal_for_each_piece(P, [&](const BalItem& it) {
+        tq4_tile<TQ, true>(P, smem, it, first);
+        first = false;
+    });
 }
 
 // Merge for the balanced decode kernel: one workgroup of 1024 threads per (token, q head) row.
@@ -1583,6 +1609,16 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     // tile's count is limited by its own units first) and keeps the partial records, and what
     // the merge kernel loads ahead of knowing the count, as small as the bound allows.
     P.max_chunks = grid_x;
+    if (batch->max_seq_len > 0) {  // = chunk_geom(0, max_seq_len - 1, max_chunks, min_upc)
+        P.spec_units = ((batch->max_seq_len - 1) >> 5) + 1;
+        int nc = (P.spec_units + P.min_upc - 1) / P.min_upc;
+        if (nc > P.max_chunks) nc = P.max_chunks;
+        if (nc < 1) nc = 1;
+        P.spec_upc = (P.spec_units + nc - 1) / nc;
+        if (P.spec_upc < 1) P.spec_upc = 1;
+        P.spec_chunks = (P.spec_units + P.spec_upc - 1) / P.spec_upc;
+        if (P.spec_chunks < 1) P.spec_chunks = 1;
+    }
     if (P.max_chunks > 1) {
         uint8_t* ws = reinterpret_cast<uint8_t*>((uintptr_t)ex->scratch_ptr);
         P.part_acc = reinterpret_cast<float*>(ws);
