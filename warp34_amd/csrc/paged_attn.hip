@@ -427,6 +427,10 @@ __device__ __forceinline__ void lds_load16(uint32_t voffset, const uint8_t* sbas
                  : "memory");
 }
 // lane L of every row of 16 lanes, in all lanes of that row (one VALU move)
+// value of the lane eight places on inside the row of 16 lanes (DPP row_ror:8)
+__device__ __forceinline__ float row_ror8(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xF, 0xF, true));
+}
 template <int L>
 __device__ __forceinline__ uint32_t row_bcast(uint32_t v) {
     return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x150 + L, 0xF, 0xF, true);  // row_newbcast:L
@@ -539,11 +543,12 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
     load_q(tok_guess);
     // validity of the token of this lane's column
     bool tok_ok;
-    auto load_tok_ok = [&](int tokbase) {
-        const int tok = tokbase + fast_div(n, P.q_group);
+    auto load_tok_ok_col = [&](int tokbase, int column) {
+        const int tok = tokbase + fast_div(column, P.q_group);
         tok_ok = tok < B.total_tokens &&
                  (B.valid_token_mask == nullptr || B.valid_token_mask[min(tok, B.total_tokens - 1)] != 0);
     };
+    auto load_tok_ok = [&](int tokbase) { load_tok_ok_col(tokbase, n); };
     load_tok_ok(tok_guess);
 
     if (build_table) {
@@ -581,6 +586,15 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
     int tile_tokens = rq_end - tok0;
     if (tile_tokens > P.tok_tile) tile_tokens = P.tok_tile;
 
+    // A tile with at most eight columns (a decode step of up to eight query heads per kv head) runs
+    // "packed": columns 8-15 repeat columns 0-7 -- same query, same scores, same probabilities -- and
+    // carry the LOW-order fp16 part of the value weights where columns 0-7 carry the high-order
+    // part, so one MFMA per value tile does the work of two.  The two halves are added up before
+    // the waves merge.
+    const bool pack = tile_tokens * P.q_group <= 8;  // wave-uniform
+    const int ncol = pack ? (n & 7) : n;             // the query column this lane works for
+    if (pack && ncol != n) load_tok_ok_col(tok0, ncol);
+
     // Column info: per lane (= per query column) the visible key range, and for the tile the union
     // and the intersection of the ranges.  Without a token mask and a window -- the common case --
     // the tile-wide values follow from scalars (every token of the tile is live, the ranges start
@@ -593,7 +607,7 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
     uint32_t ok_mask = 0u;             // bit c: column c is live (wave-uniform)
     const bool simple = B.valid_token_mask == nullptr && B.sliding_window <= 0;
     auto column_info = [&](bool accumulate) {
-        const int t = fast_div(n, P.q_group);
+        const int t = fast_div(ncol, P.q_group);
         const int tok = tok0 + t;
         const bool ok = t < tile_tokens && tok_ok;
         const int q_off = tok - rq_start;
@@ -612,7 +626,7 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
                 u_hi = max(u_hi, mx);
             }
         }
-        ok_mask = (uint32_t)(__ballot(ok) & 0xFFFFull);
+        ok_mask = (uint32_t)(__ballot(ok) & (pack ? 0xFFull : 0xFFFFull));  // mirror columns produce no output
     };
     if (simple) {
         if (tok0 >= B.total_tokens) return;  // no live column
@@ -787,6 +801,8 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         q_mf = D == 16 ? 4 : (D < 16 ? (Dh & 3) : 5 + (Dh & 3));
         q_half = half;
     }
+    static_assert(kColsPerWave == 2 && kWaves == 8, "a packed tile's mirror column col + 8 belongs to the wave of col");
+    uint2 packed_prev = {0u, 0u};
 #pragma unroll
     for (int c = 0; c < kColsPerWave; ++c) {
         const int col = wave + c * kWaves;
@@ -798,13 +814,16 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
             q_rot[3] = TQ::to_f32((uint16_t)(q_raw[c].y >> 16));
             const bool okc = (ok_mask >> col) & 1u;
             uint2 packed = {0u, 0u};
-            if (okc) {  // dead columns stay zero: no need to rotate them
+            if (pack && c == 1) {  // mirror column: the operands of column col - 8
+                packed = packed_prev;
+            } else if (okc) {  // dead columns stay zero: no need to rotate them
 #pragma unroll
                 for (int k = 0; k < 4; ++k) q_rot[k] = apply_sign(q_rot[k], 4 * lane + k);
                 wht256_wave(q_rot, lane);
                 packed.x = pack_h2(q_rot[0] * q_scale, q_rot[1] * q_scale);
                 packed.y = pack_h2(q_rot[2] * q_scale, q_rot[3] * q_scale);
             }
+            packed_prev = packed;
             uint8_t* slot0 = qop + (size_t)(col * 4) * 144;
             *reinterpret_cast<uint2*>(slot0 + q_kb * 144 + q_mf * 16 + q_half * 8) = packed;
             // the parts no element maps to: the scale nibbles of dword 0 (k-block 0, operand 0,
@@ -1005,7 +1024,7 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
             for (int k = 0; k < 4; ++k) {
                 uint32_t whi, wlo;
                 split_h2(w[2 * k], w[2 * k + 1], whi, wlo);
-                ph[h][k] = whi;
+                ph[h][k] = (pack && (n & 8)) ? wlo : whi;  // packed: the mirror columns take the low-order part
                 pl[h][k] = wlo;
                 const uint32_t wa = vw[h][2 * k], wb = vw[h][2 * k + 1];
                 // byte q of lo / hi = (nibble 2q / 2q+1 of token a) | (same nibble of token b) << 4
@@ -1040,11 +1059,13 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
                 const h8 av = __builtin_bit_cast(h8, va[bt & 1][jj]);
                 o_acc[h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, __builtin_bit_cast(h8, ph[h]), o_acc[h][j], 0, 0, 0);
             }
+            if (!pack) {
 #pragma unroll
-            for (int jj = 0; jj < 4; ++jj) {
-                const int j = 4 * (bt & 1) + jj;
-                const h8 av = __builtin_bit_cast(h8, va[bt & 1][jj]);
-                o_acc[h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, __builtin_bit_cast(h8, pl[h]), o_acc[h][j], 0, 0, 0);
+                for (int jj = 0; jj < 4; ++jj) {
+                    const int j = 4 * (bt & 1) + jj;
+                    const h8 av = __builtin_bit_cast(h8, va[bt & 1][jj]);
+                    o_acc[h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, __builtin_bit_cast(h8, pl[h]), o_acc[h][j], 0, 0, 0);
+                }
             }
         }
     };
@@ -1059,6 +1080,16 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         unit = next_unit;
     }
     wait_vm<0>();  // nothing of this wave may still be on its way into LDS when the areas are reused
+
+    // ---- packed tile: column n += its mirror column n + 8 (the low-order share of the weights) ----
+    if (pack) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) o_acc[h][j][k] += row_ror8(o_acc[h][j][k]);
+    }
 
     // ---- combine the per-lane partial sums of l over the four k-block lanes of a column ------
     l_run = sum_over_rows(l_run);
