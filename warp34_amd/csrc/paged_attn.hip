@@ -1076,9 +1076,17 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         if (has_next) locate_unit(next_unit);
         const int t0 = unit * kUnit;
         const bool masked = !(t0 >= i_lo && t0 + kUnit - 1 <= i_hi);
+        // The two waves of a SIMD take turns at the higher issue priority, unit by unit: left alone,
+        // the arbiter favours the older wave every time and the younger one finishes its units late.
+        if ((j + wslot) & 1) {
+            __builtin_amdgcn_s_setprio(1);
+        } else {
+            __builtin_amdgcn_s_setprio(0);
+        }
         process_unit(t0, masked, has_next);
         unit = next_unit;
     }
+    __builtin_amdgcn_s_setprio(0);
     wait_vm<0>();  // nothing of this wave may still be on its way into LDS when the areas are reused
 
     // ---- packed tile: column n += its mirror column n + 8 (the low-order share of the weights) ----
