@@ -45,6 +45,8 @@ WORKLOADS = {
     "q8_0_prefill_8x2048_ctx16384": ("q8_0", [18432] * 8, 0),
     # producer side: QK RMSNorm + RoPE fused with the TQ4 append of an 8 192-token chunk
     "tq4_norm_rope_append_8192": ("tq4", [8192], 0),
+    # the target model's producer: Gemma RMSNorm + interleaved mRoPE + gate split fused with the TQ4 append
+    "tq4_fused_qk_gate_append_8192": ("tq4", [8192], 0),
     # consumer side: out = attn_out * sigmoid(gate) over the rows of a 16 384-token prefill step
     "attn_output_gate_16384x4096": ("tq4", [64], 0),
     # QSA sparse attention: 1, 16 or 256 query tokens, each over its own 513 selected 4-token groups (2 052 keys)
@@ -518,6 +520,91 @@ def run_producer(args, torch, lib, ffi, layers, n, n_layers, fmt):
     }))
 
 
+def run_fused_qk_gate(args, torch, lib, ffi, layers, n, n_layers, fmt):
+    """The target model's Q/K producer (Gemma RMSNorm + interleaved mRoPE + gate split) over the fp16 rows of
+    one fused projection [n, 16 * 512 + 2 * 2 * 256], with the K / V rows written into the pages: the fused
+    entry point against the reference's two calls (operator, then the strided append).  One step = one
+    layer's producer work for an n-token chunk."""
+    dev = "cuda:0"
+    qg_w, kv_w = Q_HEADS * 2 * HEAD_DIM, KV_HEADS * HEAD_DIM
+    row = qg_w + 2 * kv_w
+    proj = synth_normal(torch, ffi, (n, row), 21).to(torch.float16)
+    q_out = torch.empty((n, Q_HEADS * HEAD_DIM), dtype=torch.float16, device=dev)
+    gate_out = torch.empty_like(q_out)
+    k_out = torch.empty((n, kv_w), dtype=torch.float16, device=dev)
+    qw = (0.1 * synth_normal(torch, ffi, (HEAD_DIM,), 22, torch.float32)).to(torch.float16)
+    kw = (0.1 * synth_normal(torch, ffi, (HEAD_DIM,), 23, torch.float32)).to(torch.float16)
+    pos = torch.arange(n, dtype=torch.int32, device=dev).repeat(3, 1).contiguous()
+    ex = ffi.Warp34Exec(torch.cuda.current_stream().cuda_stream, 0, 0, 0)
+    per_layer = []
+    posn = torch.arange(0, n, device=dev)
+    for L in layers:
+        slots = (L.block_tables[0, (posn // BLOCK)].to(torch.int64) * BLOCK + posn % BLOCK).to(torch.int32)
+        qsl = torch.tensor([0, n], dtype=torch.int32, device=dev)
+        seq = torch.tensor([n], dtype=torch.int32, device=dev)
+        batch = ffi.Warp34AttentionBatch(qsl.data_ptr(), None, seq.data_ptr(), L.block_tables.data_ptr(),
+                                         slots.data_ptr(), None, None, 1, n, L.max_blocks, n, n, 0, 0, 0.0625, 0)
+        per_layer.append((L, slots, batch, qsl, seq))
+    at = lambda off: C.c_void_p(proj.data_ptr() + 2 * off)
+    vp = lambda t: C.c_void_p(t.data_ptr())
+    rot, mrope, theta, eps = 64, (11, 11, 10), 1.0e7, 1.0e-6
+
+    def fused(i):
+        L, slots, _, _, _ = per_layer[i % n_layers]
+        rc = lib.warp34_fused_qk_rmsnorm_rope_gate_kv_write_f16(
+            C.byref(ex), at(0), at(qg_w), at(qg_w + kv_w), vp(qw), vp(kw), vp(pos), None, vp(q_out), None,
+            vp(gate_out), C.byref(L.layout), vp(slots), n, n, Q_HEADS, KV_HEADS, HEAD_DIM, rot, mrope[0], mrope[1],
+            mrope[2], row, row, row, theta, eps)
+        if rc:
+            raise RuntimeError("fused producer rc=%d" % rc)
+
+    def two_calls(i):
+        L, slots, batch, _, _ = per_layer[i % n_layers]
+        rc = lib.warp34_fused_qk_rmsnorm_rope_gate_strided_f16(
+            C.byref(ex), at(0), at(qg_w), vp(qw), vp(kw), vp(pos), None, vp(q_out), vp(k_out), vp(gate_out), n, n,
+            Q_HEADS, KV_HEADS, HEAD_DIM, rot, mrope[0], mrope[1], mrope[2], row, row, theta, eps)
+        rc = rc or lib.warp34_kv_cache_write_strided(C.byref(ex), C.byref(L.layout), C.byref(batch), vp(k_out),
+                                                     at(qg_w + kv_w), kv_w, row)
+        if rc:
+            raise RuntimeError("operator + append rc=%d" % rc)
+
+    def timed(step):
+        for i in range(args.warmup):
+            step(i)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(args.steps):
+            step(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    ms_fused = timed(fused)
+    ms_two = timed(two_calls)
+    # algorithmic bytes: the projection row is read once, Q and the gate are written once, one K and one V
+    # row per kv head go to the pages
+    bytes_step = n * (row * 2 + 2 * Q_HEADS * HEAD_DIM * 2 + 2 * KV_HEADS * ROW_BYTES[fmt]) + 3 * n * 4
+    gbs = bytes_step / (ms_fused * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "Gemma RMSNorm + mRoPE + gate split fused with the %s append: us/layer + achieved HBM GB/s" % fmt.upper(),
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_fused, 6), "us_per_layer": round(ms_fused * 1e3, 2),
+        "us_per_layer_operator_then_append": round(ms_two * 1e3, 2),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32 arithmetic on fp16 rows, %s rows written" % fmt.upper(), "data": "synthetic",
+        "config": {"workload": args.workload, "tokens": n, "q_heads": Q_HEADS, "kv_heads": KV_HEADS,
+                   "head_dim": HEAD_DIM, "rotary_dim": rot, "page_tokens": BLOCK,
+                   "kv_format": "tq4+wht256" if fmt == "tq4" else fmt, "kv_pools_cycled": n_layers,
+                   "bytes_per_step": bytes_step},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "fused_qk_norm_rope_gate_kernel (cache write fused)",
+                     "avg_launch_us": round(ms_fused * 1e3, 2)},
+    }))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -605,6 +692,9 @@ def run_workload(args, torch, lib, ffi, dev):
         return None
     if "_qsa_sparse_" in args.workload:
         run_qsa(args, torch, lib, ffi, layers, int(ctx[0]), n_layers, int(args.workload.split("_")[3].split("x")[0]), fmt)
+        return None
+    if "_fused_qk_gate_append_" in args.workload:
+        run_fused_qk_gate(args, torch, lib, ffi, layers, int(ctx[0]), n_layers, fmt)
         return None
     if "_norm_rope_append_" in args.workload:
         run_producer(args, torch, lib, ffi, layers, int(ctx[0]), n_layers, fmt)
