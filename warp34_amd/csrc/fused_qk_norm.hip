@@ -8,10 +8,10 @@
 // counterpart in the reference; its result equals operator + warp34_kv_cache_write_strided bit
 // for bit (the same row encoders).
 //
-// Mapping: one workgroup (4 waves) per token.  Wave 0 first computes the token's sine / cosine
+// Mapping: one workgroup (4 waves) per token.  The last wave computes the token's sine / cosine
 // values (they depend on the token's three positions and on the pair index only, not on the
-// head) in double precision and leaves them in LDS, fp16-rounded as the reference does.  Then
-// every wave takes items in turn, one item per wave, the two 32-lane halves of the wave each
+// head) in double precision and leaves them in LDS, fp16-rounded as the reference does, while
+// the other waves normalise their first rows.  Every wave takes items in turn, one item per wave, the two 32-lane halves of the wave each
 // playing the part of the reference's vector lanes: a Q item is two Q heads, a KV item is one K
 // head (lanes 0-31) and, when the cache is written, the V row of the same kv head (lanes 32-63).
 // Lane t of a half owns elements 8t .. 8t+7 (one 16-byte load), which is the reference's
@@ -62,7 +62,10 @@ __global__ __launch_bounds__(256) void fused_qk_norm_rope_gate_kernel(const Fuse
     const int l32 = lane & 31;
     const int hd = P.head_dim, half_rot = P.rotary_dim >> 1;
 
-    if (wave == 0) {
+    // The token's sine / cosine values: the last wave computes them (it has the fewest items),
+    // the others go ahead with the first half of their first item and meet it at the barrier
+    // in front of the first rotation.
+    if (wave == 3) {
         for (int i = lane; i < half_rot; i += 64) {
             int plane = 0;
             if ((i % 3) == 1 && i < P.s1 * 3) {
@@ -72,11 +75,11 @@ __global__ __launch_bounds__(256) void fused_qk_norm_rope_gate_kernel(const Fuse
             }
             const float pos = (float)P.positions[(size_t)plane * P.pos_plane_stride + tok];
             const float angle = pos * P.inv_freq[i];
-            s_sin[i] = F16::to_f32(F16::from_f32((float)sin((double)angle)));
-            s_cos[i] = F16::to_f32(F16::from_f32((float)cos((double)angle)));
+            s_sin[i] = F16::to_f32(F16::from_f32_of_fp32_result((float)sin((double)angle)));
+            s_cos[i] = F16::to_f32(F16::from_f32_of_fp32_result((float)cos((double)angle)));
         }
     }
-    __syncthreads();
+    bool trig_ready = false;  // wave-uniform: this wave has passed the barrier behind the sine / cosine values
 
     const bool to_cache_any = P.write_slot_mapping != nullptr;
     const int slot = to_cache_any ? P.write_slot_mapping[tok] : -1;
@@ -114,32 +117,43 @@ __global__ __launch_bounds__(256) void fused_qk_norm_rope_gate_kernel(const Fuse
             raw = *reinterpret_cast<const uint4*>(src + 8 * l32);
             wraw = *reinterpret_cast<const uint4*>(w + 8 * l32);
         }
-        const uint16_t* h = reinterpret_cast<const uint16_t*>(&raw);
-        const uint16_t* wh = reinterpret_cast<const uint16_t*>(&wraw);
+        // (halves taken out and put together with shifts: indexing the vectors through a pointer
+        // would move them to scratch memory)
+        const uint32_t rw[4] = {raw.x, raw.y, raw.z, raw.w};
+        const uint32_t ww[4] = {wraw.x, wraw.y, wraw.z, wraw.w};
         float x[8];
         float acc = 0.0f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            x[j] = F16::to_f32(h[j]);
+            x[j] = F16::to_f32((uint16_t)(rw[j >> 1] >> (16 * (j & 1))));
             const float sq = x[j] * x[j];
             acc = acc + sq;
         }
         const float sum_sq = half_wave_sum(acc, lane);
         const float mean = sum_sq / (float)hd + P.eps;
         const float inv_rms = (float)(1.0 / sqrt((double)mean));
-        uint4 nrm;
-        uint16_t* nh = reinterpret_cast<uint16_t*>(&nrm);
+        uint32_t nw[4];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const float v = x[j] * inv_rms;
-            const float wt = 1.0f + F16::to_f32(wh[j]);
-            nh[j] = F16::from_f32(v * wt);
+        for (int k = 0; k < 4; ++k) {
+            uint32_t packed = 0u;
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh) {
+                const int j = 2 * k + hh;
+                const float v = x[j] * inv_rms;
+                const float wt = 1.0f + F16::to_f32((uint16_t)(ww[k] >> (16 * hh)));
+                packed |= (uint32_t)F16::from_f32_of_fp32_result(v * wt) << (16 * hh);
+            }
+            nw[k] = is_v_half ? rw[k] : packed;  // the V half keeps its row as it is
         }
-        // the V half keeps its row as it is
-        if (owns_vec) *reinterpret_cast<uint4*>(row + 8 * l32) = is_v_half ? raw : nrm;
-        __atomic_signal_fence(__ATOMIC_SEQ_CST);
-        __builtin_amdgcn_wave_barrier();
-        __atomic_signal_fence(__ATOMIC_SEQ_CST);
+        if (owns_vec) *reinterpret_cast<uint4*>(row + 8 * l32) = uint4{nw[0], nw[1], nw[2], nw[3]};
+        if (!trig_ready) {  // (also orders the row buffer: a workgroup barrier includes the wave's own)
+            __syncthreads();
+            trig_ready = true;
+        } else {
+            __atomic_signal_fence(__ATOMIC_SEQ_CST);
+            __builtin_amdgcn_wave_barrier();
+            __atomic_signal_fence(__ATOMIC_SEQ_CST);
+        }
 
         // ---- rotation of the pairs (i, i + rotary / 2), in place ----
         if (!is_v_half) {
@@ -147,8 +161,8 @@ __global__ __launch_bounds__(256) void fused_qk_norm_rope_gate_kernel(const Fuse
                 const float x1 = F16::to_f32(row[i]), x2 = F16::to_f32(row[i + half_rot]);
                 const float c = s_cos[i], s = s_sin[i];
                 const float a = x1 * c, b = x2 * s, cc = x2 * c, d = x1 * s;
-                row[i] = F16::from_f32(a - b);
-                row[i + half_rot] = F16::from_f32(cc + d);
+                row[i] = F16::from_f32_of_fp32_result(a - b);
+                row[i + half_rot] = F16::from_f32_of_fp32_result(cc + d);
             }
         }
         __atomic_signal_fence(__ATOMIC_SEQ_CST);
@@ -187,6 +201,7 @@ __global__ __launch_bounds__(256) void fused_qk_norm_rope_gate_kernel(const Fuse
         __builtin_amdgcn_wave_barrier();
         __atomic_signal_fence(__ATOMIC_SEQ_CST);
     }
+    if (!trig_ready) __syncthreads();  // a wave without items: every wave of the workgroup meets the barrier once
 }
 
 static int launch_fused_qk(const warp34_exec* ex, const void* q_gate_in, const void* k_in, const void* v_in,

@@ -69,6 +69,14 @@ struct F16 {
     __device__ static __forceinline__ uint16_t from_f32(float f) {
         return __half_as_ushort(__float2half_rn(f));
     }
+    // The same conversion for results whose bits are part of a contract: the value passes through
+    // an empty asm statement, so the compiler cannot fold the fp32 operation that produced it and
+    // the conversion into one mixed-precision FMA (which rounds once where the reference rounds
+    // twice, to fp32 and then to fp16).
+    __device__ static __forceinline__ uint16_t from_f32_of_fp32_result(float f) {
+        asm("" : "+v"(f));
+        return __half_as_ushort(__float2half_rn(f));
+    }
 };
 struct BF16 {
     static constexpr int kStorageFormat = WARP34_KV_FORMAT_BF16;
