@@ -59,11 +59,20 @@ WORKLOADS = {
     "tq4_verify_16x4_ctx262144_shared200k": ("tq4", [262144] * 16, 0),
 }
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by
-# a plain copy of known size (profiles/paged_attn_tq4_decode_b1_ctx131072_hbm_traffic.txt); counters cannot
+# a plain copy of known size (the scale is stated in each profile); counters cannot
 # be read from inside this process, so workloads without such a profile report null.
 MEASURED_TRAFFIC = {
     # workload: (HBM bytes per launch of the dominant kernel, the profile that holds the counter readings)
-    "tq4_decode_b1_ctx131072": (71_824_000, "profiles/paged_attn_tq4_decode_b1_ctx131072_hbm_traffic.txt"),
+    "tq4_decode_b1_ctx131072": (71_834_000, "profiles/paged_attn_tq4_decode_b1_ctx131072.txt"),
+    "tq4_decode_b8_ctx131072": (558_377_000, "profiles/paged_attn_tq4_decode_b8_ctx131072.txt"),
+    "tq4_decode_b32_ctx1k_64k": (586_269_000, "profiles/paged_attn_tq4_decode_b32_ctx1k_64k.txt"),
+    "bf16_decode_b1_ctx32768": (70_596_000, "profiles/paged_attn_rows_bf16_decode_b1_ctx32768.txt"),
+    "fp8_decode_b32_ctx1k_64k": (1_192_010_000, "profiles/paged_attn_rows_fp8_decode_b32_ctx1k_64k.txt"),
+    "tq4_verify_16x4_ctx262144_shared200k": (736_353_000, "profiles/paged_attn_tq4_verify_16x4_ctx262144_shared200k.txt"),
+    "tq4_prefill_8x2048_ctx16384": (1_134_522_000, "profiles/paged_prefill_tq4_8x2048_ctx16384.txt"),
+    "tq4_qsa_sparse_16x513_ctx131072": (23_417_000, "profiles/qsa_sparse_tq4_16x513_ctx131072.txt"),
+    "tq4_norm_rope_append_8192": (183_326_000, "profiles/qk_norm_rope_tq4_append_8192.txt"),
+    "tq4_fused_qk_gate_append_8192": (289_050_000, "profiles/fused_qk_norm_rope_gate_tq4_append_8192.txt"),
 }
 SHARED_PREFIX = {"tq4_verify_16x4_ctx262144_shared200k": 200000}
 VERIFY_Q = {"tq4_verify_16x4_ctx262144_shared200k": 4}
@@ -323,7 +332,8 @@ def run_prefill(args, torch, lib, ffi, layers, ctx, n_layers, pool_pages, fmt):
                    "pool_pages": pool_pages,
                    "attention_flops_per_step": flops, "rows_appended_per_step": N * KV_HEADS * 2},
         "roofline": {"bound": "mfma", "achieved": round(tf_attn, 1), "peak": peak, "unit": "TFLOP/s",
-                     "frac": round(tf_attn / peak, 4), "traffic": None,
+                     "frac": round(tf_attn / peak, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, (None, None))[0],
+                     "traffic_source": MEASURED_TRAFFIC.get(args.workload, (None, None))[1],
                      "kernel": "paged_prefill_tq4_kernel (attention-only launches)",
                      "avg_launch_us": round(ms_attn * 1e3, 1)},
     }))
@@ -365,7 +375,8 @@ def run_gate(args, torch, lib, ffi):
         "dtype": "f32 arithmetic on f16 rows", "data": "synthetic",
         "config": {"workload": args.workload, "tokens": n, "total_dim": dim, "bytes_per_step": nbytes},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "attn_output_gate_kernel<true>",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, (None, None))[0],
+                     "traffic_source": MEASURED_TRAFFIC.get(args.workload, (None, None))[1], "kernel": "attn_output_gate_kernel<true>",
                      "avg_launch_us": round(ms * 1e3, 2)},
     }))
 
@@ -430,7 +441,8 @@ def run_qsa(args, torch, lib, ffi, layers, ctx_len, n_layers, n_tok, fmt, select
                    "head_dim": HEAD_DIM, "page_tokens": BLOCK, "kv_format": "tq4+wht256" if fmt == "tq4" else fmt,
                    "kv_pools_cycled": n_layers, "bytes_per_step": nbytes},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, (None, None))[0],
+                     "traffic_source": MEASURED_TRAFFIC.get(args.workload, (None, None))[1],
                      "kernel": ("qsa_sparse_tq4_kernel" if fmt == "tq4" else "qsa_sparse_rows_kernel") +
                                " + qsa_sparse_merge_kernel (whole call)",
                      "avg_launch_us": round(ms * 1e3, 2)},
@@ -514,7 +526,8 @@ def run_producer(args, torch, lib, ffi, layers, n, n_layers, fmt):
                    "head_dim": HEAD_DIM, "page_tokens": BLOCK, "kv_format": "tq4+wht256" if fmt == "tq4" else fmt,
                    "kv_pools_cycled": n_layers, "bytes_per_step": bytes_step},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, (None, None))[0],
+                     "traffic_source": MEASURED_TRAFFIC.get(args.workload, (None, None))[1],
                      "kernel": "qk_norm_rope_kernel<true, true> (fused cache write)",
                      "avg_launch_us": round(ms_fused * 1e3, 2)},
     }))
@@ -599,7 +612,8 @@ def run_fused_qk_gate(args, torch, lib, ffi, layers, n, n_layers, fmt):
                    "kv_format": "tq4+wht256" if fmt == "tq4" else fmt, "kv_pools_cycled": n_layers,
                    "bytes_per_step": bytes_step},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, (None, None))[0],
+                     "traffic_source": MEASURED_TRAFFIC.get(args.workload, (None, None))[1],
                      "kernel": "fused_qk_norm_rope_gate_kernel (cache write fused)",
                      "avg_launch_us": round(ms_fused * 1e3, 2)},
     }))
