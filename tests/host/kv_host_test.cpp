@@ -9,6 +9,7 @@
 #include <stdexcept>
 #include <string>
 
+#include "../../warp34_amd/host/graph_io.h"
 #include "../../warp34_amd/host/kv_host.h"
 
 using namespace warp34_host;
@@ -601,6 +602,136 @@ static void test_radix_random_walk() {
     std::puts("ok radix_random_walk");
 }
 
+// ---- step descriptors of captured steps (model/graph_io.rs) ----
+static StepSlice spec_slice(std::vector<int32_t> tokens) {  // the fixture of graph_io.rs:1262-1274
+    StepSlice s;
+    s.tokens = std::move(tokens);
+    s.ctx_len_before = 15;
+    s.block_table = {7, 3};
+    s.state_in_slot = 2;
+    s.state_out_slot = 5;
+    s.has_initial_state = true;
+    s.spec_slots = {8, 9};
+    s.checkpoints = {{1, 6}};
+    return s;
+}
+
+static void test_spec_verify_meta() {  // graph_io.rs:1276-1317
+    using M = SpecVerifyMeta;
+    const size_t n = M::T, cp = M::CP;
+    M m;
+    CHECK(pack_spec_verify_meta(spec_slice({41, 42}), kBaseModelLoraId, 16, &m));
+    const auto& w = m.words;
+    CHECK(w[0] == 41 && w[1] == 42);
+    CHECK(w[n] == 15 && w[n + 1] == 16);
+    CHECK(w[2 * n] == 7 * 16 + 15 && w[2 * n + 1] == 3 * 16);  // the second token crosses into the next page
+    CHECK(w[3 * n] == 8 && w[3 * n + 1] == 9);
+    CHECK(w[4 * n] == 6 && w[4 * n + cp] == 1);
+    const int32_t q[6] = {0, 2, 15, 17, 2, 5};
+    for (int i = 0; i < 6; ++i) CHECK(w[4 * n + 2 * cp + i] == q[i]);
+    for (size_t i = 0; i < n; ++i) CHECK(w[4 * n + 2 * cp + 6 + i] == -1);
+    M ml;
+    CHECK(pack_spec_verify_meta(spec_slice({41, 42}), 3, 16, &ml));
+    CHECK(ml.words[4 * n + 2 * cp + 6] == 3 && ml.words[4 * n + 2 * cp + 7] == 3);
+    for (size_t i = 2; i < n; ++i) CHECK(ml.words[4 * n + 2 * cp + 6 + i] == kBaseModelLoraId);
+    for (size_t base : {size_t(0), n, 2 * n, 3 * n})
+        for (size_t i = 2; i < n; ++i) CHECK(w[base + i] == -1);
+    for (size_t i = 1; i < cp; ++i) CHECK(w[4 * n + i] == -1);
+    // capacity and table checks
+    CHECK(!pack_spec_verify_meta(spec_slice(std::vector<int32_t>(n + 1, 1)), -1, 16, &m));
+    CHECK(!pack_spec_verify_meta(spec_slice({}), -1, 16, &m));
+    StepSlice s = spec_slice({1, 2});
+    s.block_table = {7};
+    CHECK(!pack_spec_verify_meta(s, -1, 16, &m));
+    s.ctx_len_before = ~size_t(0);
+    CHECK(!pack_spec_verify_meta(s, -1, 16, &m));
+    // other page sizes: position 15 + 1 stays inside a 64-token page
+    s = spec_slice({5, 6});
+    CHECK(pack_spec_verify_meta(s, -1, 64, &m) && m.words[2 * n] == 7 * 64 + 15 && m.words[2 * n + 1] == 7 * 64 + 16);
+    const warp34_attention_batch b = M::batch_at(0x1000, 0x2000, 2, 8, 4096, 0, 0.0625f);
+    CHECK((uint64_t)(uintptr_t)b.query_start_loc == 0x1000 + 4 * M::kQStartLoc && b.total_tokens == 2 && b.num_reqs == 1);
+    CHECK((uint64_t)(uintptr_t)b.write_slot_mapping == 0x1000 + 4 * 2 * n && b.max_q_len == 2 && b.max_seq_len == 4096);
+    std::puts("ok spec_verify_meta");
+}
+
+static void test_batched_decode_meta() {  // graph_io.rs:585-595, 789-871
+    CHECK(!decode_graph_bucket(0) && *decode_graph_bucket(1) == 1 && *decode_graph_bucket(2) == 2);
+    CHECK(*decode_graph_bucket(3) == 4 && *decode_graph_bucket(4) == 4 && *decode_graph_bucket(5) == 8);
+    CHECK(*decode_graph_bucket(8) == 8 && *decode_graph_bucket(9) == 16 && *decode_graph_bucket(16) == 16);
+    CHECK(!decode_graph_bucket(17));
+    using M = BatchedDecodeMeta;
+    static_assert(M::kWords == 177 && M::kMasksByteOffset == 768 && M::kBlobBytes == 816, "blob layout");
+    std::vector<StepSlice> sl(3);
+    for (int r = 0; r < 3; ++r) {
+        sl[r].tokens = {100 + r};
+        sl[r].ctx_len_before = (size_t)(15 + 16 * r);   // positions 15, 31, 47: the last slot of a page each
+        sl[r].block_table = {7, 3, 9, 4};
+        sl[r].state_in_slot = r;
+        sl[r].state_out_slot = 10 + r;
+        sl[r].has_initial_state = r != 1;
+    }
+    sl[2].checkpoints = {{1, 6}};
+    M m;
+    CHECK(pack_batched_decode_meta(sl, {0, 5}, {}, 2, 16, &m));
+    const auto& w = m.words;
+    CHECK(w[M::kTokenIds] == 100 && w[M::kTokenIds + 2] == 102 && w[M::kTokenIds + 3] == 0);
+    CHECK(w[M::kPositions] == 15 && w[M::kPositions + 1] == 31 + 5 && w[M::kPositions + 2] == 47);
+    CHECK(w[M::kWriteSlots] == 7 * 16 + 15 && w[M::kWriteSlots + 1] == 3 * 16 + 15 && w[M::kWriteSlots + 2] == 9 * 16 + 15);
+    for (size_t r = 3; r < M::N; ++r) CHECK(w[M::kWriteSlots + r] == -1 && w[M::kStateOut + r] == -1 && w[M::kLoraIds + r] == -1);
+    for (size_t i = 0; i <= M::N; ++i) CHECK(w[M::kQStartLoc + i] == (int32_t)i);
+    CHECK(w[M::kCtxBefore + 1] == 31 && w[M::kSeqAfter + 1] == 32 && w[M::kCtxBefore + 3] == 0 && w[M::kSeqAfter + 3] == 0);
+    CHECK(w[M::kStateIn + 2] == 2 && w[M::kStateOut + 2] == 12 && w[M::kCheckpointDst + 2] == 6 && w[M::kCheckpointOffset + 2] == 1);
+    CHECK(w[M::kCheckpointDst] == -1 && w[M::kLoraIds] == 2 && w[M::kLoraIds + 2] == 2);
+    CHECK(m.masks[M::kHasInitialState] == 1 && m.masks[M::kHasInitialState + 1] == 0 && m.masks[M::kValidReq + 2] == 1);
+    CHECK(m.masks[M::kValidReq + 3] == 0 && m.masks[M::kValidToken + 2] == 1 && m.masks[M::kValidToken + 3] == 0);
+    const auto blob = m.blob();
+    CHECK(blob.size() == 816 && blob[M::kMasksByteOffset + M::kValidReq] == 1 && blob[4 * M::kTokenIds] == 100);
+    // a decode row has one token, no speculative slots, and a table that reaches its position
+    sl[0].tokens = {1, 2};
+    CHECK(!pack_batched_decode_meta(sl, {}, {}, -1, 16, &m));
+    sl[0].tokens = {1};
+    sl[0].block_table = {};
+    CHECK(!pack_batched_decode_meta(sl, {}, {}, -1, 16, &m));
+    sl[0].block_table = {7};
+    CHECK(pack_batched_decode_meta(sl, {}, {}, -1, 16, &m));        // position 15 is in the first page
+    sl[0].ctx_len_before = 16;
+    CHECK(!pack_batched_decode_meta(sl, {}, {}, -1, 16, &m));       // position 16 is not
+    CHECK(pack_batched_decode_meta(sl, {}, {}, -1, 64, &m) && m.words[M::kWriteSlots] == 7 * 64 + 16);
+    CHECK(!pack_batched_decode_meta({}, {}, {}, -1, 16, &m));
+    CHECK(!pack_batched_decode_meta(std::vector<StepSlice>(17, sl[1]), {}, {}, -1, 16, &m));
+    const warp34_attention_batch b = M::batch_at(0x10000, 0x20000, 4, 32, 8192, 0, 0.0625f);
+    CHECK(b.num_reqs == 4 && b.total_tokens == 4 && b.max_q_len == 1 && b.max_blocks_per_req == 32);
+    CHECK((uint64_t)(uintptr_t)b.valid_req_mask == 0x10000 + 768 + 16 && (uint64_t)(uintptr_t)b.seq_lens_after == 0x10000 + 4 * 81);
+    std::puts("ok batched_decode_meta");
+}
+
+static void test_block_table_mirror() {  // graph_io.rs:886-1010
+    BlockTableMirror mir(8);
+    std::vector<StepSlice> sl(2);
+    sl[0].block_table = {5, 6};
+    sl[1].block_table = {9};
+    auto sp = mir.dirty_spans(sl);
+    CHECK(sp && sp->size() == 2 && (*sp)[0].row == 0 && (*sp)[0].start == 0 && (*sp)[0].entries == std::vector<int32_t>({5, 6}));
+    CHECK((*sp)[1].dst_byte_offset == 8 * 4);
+    sp = mir.dirty_spans(sl);
+    CHECK(sp && sp->empty());                                     // nothing changed: nothing to copy
+    sl[0].block_table = {5, 6, 7};                                // grew: only the tail
+    sp = mir.dirty_spans(sl);
+    CHECK(sp && sp->size() == 1 && (*sp)[0].start == 2 && (*sp)[0].entries == std::vector<int32_t>({7}) &&
+          (*sp)[0].dst_byte_offset == 2 * 4);
+    sl[1].block_table = {4, 9};                                   // another request took the row: the whole row
+    sp = mir.dirty_spans(sl);
+    CHECK(sp && sp->size() == 1 && (*sp)[0].row == 1 && (*sp)[0].start == 0 && (*sp)[0].entries.size() == 2);
+    mir.invalidate(*sp);                                          // the copy failed: next time the whole row again
+    sp = mir.dirty_spans(sl);
+    CHECK(sp && sp->size() == 1 && (*sp)[0].row == 1 && (*sp)[0].start == 0);
+    sp = mir.dirty_spans(sl, false);
+    CHECK(sp && sp->empty());
+    sl[0].block_table.assign(9, 1);
+    CHECK(!mir.dirty_spans(sl));                                  // a row longer than the device row
+    std::puts("ok block_table_mirror");
+}
+
 int main() {
     test_row_bytes();
     test_policy_resolution();
@@ -621,6 +752,9 @@ int main() {
     test_radix_recycle_and_invalidate();
     test_radix_dual_lock_dual_lru_tombstone_and_split();
     test_radix_random_walk();
+    test_spec_verify_meta();
+    test_batched_decode_meta();
+    test_block_table_mirror();
     std::puts("all host tests passed");
     return 0;
 }

@@ -187,3 +187,104 @@ def test_qsa_sparse_attention_replays_with_new_selections():
         vmax = np.abs(oracle.bits_to_f32(v, DT_F16)).max(axis=0)
         scale = np.broadcast_to(np.maximum(1.0, np.repeat(vmax, heads // 2, axis=0))[None], (n_tok, heads, 256))
         G.assert_close(got, DT_F16, oracle.f16_bits_to_f32(ref), what="replay %d vs oracle" % t, scale=scale)
+
+
+def test_bucketed_decode_graph_serves_any_live_count():
+    """One captured step per bucket (graph_io.rs:585-595): the graph of bucket 8 reads its lengths, slots, masks
+    and block tables from the fixed-shape device blob of BatchedDecodeGraphIo (graph_io.rs:647-871), so batches
+    of 5, 8 and 6 live requests replay the same graph; rows behind the live ones are masked out and untouched."""
+    import torch
+
+    import gpu_harness as G
+    from warp34_amd import ffi
+
+    lib = G.lib()
+    bs, q_heads, kv_heads, B = 64, 16, 2, 8
+    seqs = [700, 65, 1290, 31, 2049, 130, 999, 64]
+    pool, bt, k, v, _, _, _ = make_case(FMT_TQ4, bs, [s + 1 for s in seqs], [1] * B, 77, DT_BF16,
+                                        kv_heads=kv_heads, q_heads=q_heads)
+    starts = np.concatenate([[0], np.cumsum([s + 1 for s in seqs])])
+    host = oracle.HostPool(pool.num_pages, kv_heads, 256, bs, FMT_TQ4, oracle.XF_WHT256)
+    for r, s in enumerate(seqs):
+        wb = oracle.HostBatch([0, s], [s], bt[r:r + 1], context_lens_before=[0],
+                              write_slot_mapping=oracle.slot_mapping(bt[r], 0, s, bs))
+        oracle.kv_cache_write(host, wb, k[starts[r]:starts[r] + s], v[starts[r]:starts[r] + s], DT_BF16)
+    dpool = G.DevPool(host)
+    dpool.upload()
+    L = dpool.layout()
+    max_blocks = bt.shape[1]
+
+    assert lib.warp34_host_decode_graph_bucket(5) == B and lib.warp34_host_decode_graph_bucket(17) == 0
+    blob_bytes = 816
+    blob = torch.zeros(blob_bytes, dtype=torch.uint8, device=G.DEV)
+    btd = torch.zeros((16, max_blocks), dtype=torch.int32, device=G.DEV)
+    k_in = torch.zeros((B, kv_heads, 256), dtype=torch.int16, device=G.DEV)
+    v_in = torch.zeros_like(k_in)
+    q_in = torch.zeros((B, q_heads, 256), dtype=torch.int16, device=G.DEV)
+    out = torch.zeros_like(q_in)
+    scratch = torch.zeros(16 << 20, dtype=torch.uint8, device=G.DEV)
+    batch = ffi.Warp34AttentionBatch()
+    lib.warp34_host_batched_decode_batch_at(blob.data_ptr(), btd.data_ptr(), B, max_blocks, 4096, 0, 0.0625, C.byref(batch))
+    assert batch.num_reqs == B and batch.total_tokens == B and batch.max_q_len == 1
+
+    def step_calls():
+        ex = ffi.Warp34Exec(torch.cuda.current_stream().cuda_stream, scratch.data_ptr(), scratch.numel(), 0)
+        assert lib.warp34_kv_cache_write_bf16(C.byref(ex), C.byref(L), C.byref(batch), C.c_void_p(k_in.data_ptr()),
+                                              C.c_void_p(v_in.data_ptr())) == 0
+        assert lib.warp34_paged_attention_bf16(C.byref(ex), C.byref(L), C.byref(batch), C.c_void_p(q_in.data_ptr()),
+                                               C.c_void_p(out.data_ptr()), q_heads) == 0
+
+    def set_state(live, seed):
+        """The blob and the inputs of a step over the requests `live` (row i of the batch = request live[i])."""
+        n = len(live)
+        tokens = np.arange(n, dtype=np.int32)
+        ctxs = np.array([seqs[r] for r in live], dtype=np.int32)
+        tables = np.ascontiguousarray(bt[live], dtype=np.int32)
+        lens = np.array([(seqs[r] + 1 + bs - 1) // bs for r in live], dtype=np.int32)
+        host_blob = np.zeros(blob_bytes, np.uint8)
+        rc = lib.warp34_host_pack_batched_decode_blob(tokens.ctypes.data, ctxs.ctypes.data, tables.ctypes.data,
+                                                      lens.ctypes.data, max_blocks, n, bs, host_blob.ctypes.data)
+        assert rc == 0
+        blob.copy_(torch.from_numpy(host_blob).to(G.DEV))
+        btd.zero_()
+        btd[:n].copy_(torch.from_numpy(tables).to(G.DEV))
+        rows = [starts[r] + seqs[r] for r in live]
+        kk, vv = np.zeros((B, kv_heads, 256), np.uint16), np.zeros((B, kv_heads, 256), np.uint16)
+        kk[:n], vv[:n] = k[rows], v[rows]
+        k_in.copy_(G.to_dev(kk))
+        v_in.copy_(G.to_dev(vv))
+        q_in.copy_(G.to_dev(oracle.fill_normal(B * q_heads * 256, seed, DT_BF16).reshape(B, q_heads, 256)))
+        out.fill_(0x5500)
+
+    snap_k, snap_v = dpool.k.clone(), dpool.v.clone()
+    set_state(list(range(B)), 1)
+    step_calls()  # eager warm-up
+    torch.cuda.synchronize()
+    dpool.k.copy_(snap_k)
+    dpool.v.copy_(snap_v)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        step_calls()
+
+    for it, live in enumerate(([0, 2, 4, 5, 7], list(range(B)), [6, 1, 3, 0, 2, 4])):
+        dpool.k.copy_(snap_k)
+        dpool.v.copy_(snap_v)
+        set_state(live, 900 + it)
+        g.replay()
+        torch.cuda.synchronize()
+        got = out.cpu().numpy().view(np.uint16).copy()
+        n = len(live)
+        assert (got[n:] == 0x5500).all(), "rows behind the live requests must stay untouched"
+        # the oracle on a host pool that receives the same appended rows
+        hk, hv = dpool.download()
+        ref_pool = oracle.HostPool(pool.num_pages, kv_heads, 256, bs, FMT_TQ4, oracle.XF_WHT256)
+        ref_pool.k[:], ref_pool.v[:] = host.k, host.v
+        cur = [seqs[r] for r in live]
+        slots = np.array([oracle.slot_mapping(bt[r], seqs[r], 1, bs)[0] for r in live], dtype=np.int32)
+        wb = oracle.HostBatch(np.arange(n + 1), [c + 1 for c in cur], bt[live], context_lens_before=cur,
+                              write_slot_mapping=slots)
+        rows = [starts[r] + seqs[r] for r in live]
+        oracle.kv_cache_write(ref_pool, wb, k[rows], v[rows], DT_BF16)
+        assert hk.tobytes() == ref_pool.k.tobytes() and hv.tobytes() == ref_pool.v.tobytes(), "replay %d: pool bytes" % it
+        ref = oracle.paged_attention(ref_pool, wb, q_in.cpu().numpy().view(np.uint16)[:n], DT_BF16, q_heads, n_threads=4)
+        G.assert_close(got[:n], DT_BF16, ref, what="bucket replay %d (%d live) vs oracle" % (it, n))

@@ -15,7 +15,7 @@ import subprocess
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-EXPECTED_HOST_TESTS = 19  # "ok <name>" lines of tests/host/kv_host_test.cpp
+EXPECTED_HOST_TESTS = 22  # "ok <name>" lines of tests/host/kv_host_test.cpp
 
 
 def test_host_mirror_cpp(tmp_path):
@@ -25,7 +25,8 @@ def test_host_mirror_cpp(tmp_path):
            "-static-libasan", "-static-libubsan",
            os.path.join(ROOT, "tests", "host", "kv_host_test.cpp"),
            os.path.join(ROOT, "warp34_amd", "host", "kv_host.cpp"),
-           os.path.join(ROOT, "warp34_amd", "host", "prefix_cache.cpp"), "-o", exe]
+           os.path.join(ROOT, "warp34_amd", "host", "prefix_cache.cpp"),
+           os.path.join(ROOT, "warp34_amd", "host", "graph_io.cpp"), "-o", exe]
     subprocess.run(cmd, check=True)
     p = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     assert p.returncode == 0, p.stdout

@@ -31,6 +31,7 @@ SOURCES = [
     (os.path.join(CSRC, "runtime.hip"), []),
     (os.path.join(HOST, "kv_host.cpp"), []),
     (os.path.join(HOST, "prefix_cache.cpp"), []),
+    (os.path.join(HOST, "graph_io.cpp"), []),
     (os.path.join(HOST, "kv_host_runtime.cpp"), []),
     (os.path.join(HOST, "synth.cpp"), ["-pthread"]),
 ]

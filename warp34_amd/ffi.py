@@ -131,6 +131,11 @@ SIGNATURES = {
         (C.c_int, [_EX] + [C.c_void_p] * 9 + [C.c_int] * 9 + [C.c_float, C.c_float]),
     "warp34_fused_qk_rmsnorm_rope_gate_kv_write_f16":
         (C.c_int, [_EX] + [C.c_void_p] * 10 + [_LAY, C.c_void_p] + [C.c_int] * 12 + [C.c_float, C.c_float]),
+    "warp34_host_decode_graph_bucket": (C.c_int, [C.c_int]),
+    "warp34_host_pack_batched_decode_blob":
+        (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
+    "warp34_host_batched_decode_batch_at":
+        (None, [C.c_uint64, C.c_uint64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, _BAT]),
     "warp34_apply_attn_output_gate_f16":
         (C.c_int, [_EX, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int]),
     # QSA sparse paged attention over selected 4-token groups (plain, and with the per-64 output transform)
