@@ -103,7 +103,7 @@ struct AttnParams {
     uint32_t block_magic;  // floor(2^32 / block_size), see div_block
     const uint16_t* gate;  // fp16 [tokens, q heads, 256] or null: out = fp16(out) * sigmoid(gate)
     // chunk geometry of a tile whose keys are exactly [0, max_seq_len): worked out on the host, so a
-    // request that is as long as the host's bound needs no division on the device (TQ4 decode kernel)
+    // request that is as long as the host's bound needs no division on the device
     int spec_units, spec_upc, spec_chunks;
 };
 
@@ -1602,6 +1602,19 @@ static int balanced_groups(int q_subgroups) {
     return groups < 1 ? 1 : groups;
 }
 
+// P.spec_* = chunk_geom(0, max_seq_len - 1, P.max_chunks, P.min_upc), worked out on the host
+static void fill_spec_geometry(AttnParams& P, int max_seq_len) {
+    if (max_seq_len <= 0) return;
+    P.spec_units = ((max_seq_len - 1) >> 5) + 1;
+    int nc = (P.spec_units + P.min_upc - 1) / P.min_upc;
+    if (nc > P.max_chunks) nc = P.max_chunks;
+    if (nc < 1) nc = 1;
+    P.spec_upc = (P.spec_units + nc - 1) / nc;
+    if (P.spec_upc < 1) P.spec_upc = 1;
+    P.spec_chunks = (P.spec_units + P.spec_upc - 1) / P.spec_upc;
+    if (P.spec_chunks < 1) P.spec_chunks = 1;
+}
+
 template <typename TQ>
 static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
                       const warp34_attention_batch* batch, const void* q, void* out, int num_q_heads,
@@ -1648,16 +1661,7 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     // tile's count is limited by its own units first) and keeps the partial records, and what
     // the merge kernel loads ahead of knowing the count, as small as the bound allows.
     P.max_chunks = grid_x;
-    if (batch->max_seq_len > 0) {  // = chunk_geom(0, max_seq_len - 1, max_chunks, min_upc)
-        P.spec_units = ((batch->max_seq_len - 1) >> 5) + 1;
-        int nc = (P.spec_units + P.min_upc - 1) / P.min_upc;
-        if (nc > P.max_chunks) nc = P.max_chunks;
-        if (nc < 1) nc = 1;
-        P.spec_upc = (P.spec_units + nc - 1) / nc;
-        if (P.spec_upc < 1) P.spec_upc = 1;
-        P.spec_chunks = (P.spec_units + P.spec_upc - 1) / P.spec_upc;
-        if (P.spec_chunks < 1) P.spec_chunks = 1;
-    }
+    fill_spec_geometry(P, batch->max_seq_len);
     if (P.max_chunks > 1) {
         uint8_t* ws = reinterpret_cast<uint8_t*>((uintptr_t)ex->scratch_ptr);
         P.part_acc = reinterpret_cast<float*>(ws);
@@ -1747,6 +1751,7 @@ static int launch_rows(const warp34_exec* ex, const warp34_kv_layer_layout* layo
     // tile's count is limited by its own units first) and keeps the partial records, and what
     // the merge kernel loads ahead of knowing the count, as small as the bound allows.
     P.max_chunks = grid_x;
+    fill_spec_geometry(P, batch->max_seq_len);
     if (P.max_chunks > 1) {
         uint8_t* ws = reinterpret_cast<uint8_t*>((uintptr_t)ex->scratch_ptr);
         P.part_acc = reinterpret_cast<float*>(ws);

@@ -174,12 +174,11 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
     int spec_slot_base = -1, spec_vec = -1;
     if constexpr (BAL) {
         // the piece's first unit is known: its block-table slice is requested with the query rows
-        spec_slot_base = fast_div(item.u_begin * kUnit, L.block_size);
+        spec_slot_base = div_block(item.u_begin * kUnit, P);
         const int slot = spec_slot_base + lane;
         if (slot < B.max_blocks_per_req) spec_vec = B.block_tables[(size_t)tile_z * B.max_blocks_per_req + slot];
     } else if (P.tiles_by_request && B.sliding_window <= 0 && B.max_seq_len > 0) {
-        const ChunkGeom sg = chunk_geom(0, B.max_seq_len - 1, P.max_chunks, P.min_upc);
-        spec_slot_base = fast_div((sg.u_first + chunk * sg.upc) * kUnit, L.block_size);
+        spec_slot_base = div_block(chunk * P.spec_upc * kUnit, P);
         const int slot = spec_slot_base + lane;
         if (slot < B.max_blocks_per_req)
             spec_vec = B.block_tables[(size_t)tile_z * B.max_blocks_per_req + slot];
@@ -220,6 +219,9 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
     int tile_tokens = rq_end - tok0;
     if (tile_tokens > P.tok_tile) tile_tokens = P.tok_tile;
 
+    // Column info (per lane = per query column: visible key range; tile-wide: union and intersection
+    // of the ranges).  Without a token mask and a window the tile-wide values follow from scalars
+    // and the per-lane part waits until the first rows have been requested (see the TQ4 kernel).
     int col_lo[NT], col_hi[NT];
     bool col_ok[NT];
     int u_lo = 0x7fffffff, u_hi = -1;
@@ -227,39 +229,64 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
     uint32_t ok_mask[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-        const int col = nt * 16 + n;
-        const int t = fast_div(col, P.q_group);
-        const int tok = tok0 + t;
-        const bool ok = t < tile_tokens && tok_ok[nt];
-        const int q_off = tok - rq_start;
-        int mx = (B.mask_mode == WARP34_ATTN_MASK_NONCAUSAL_WINDOW) ? seq_after - 1 : ctx_before + q_off;
-        if (mx >= seq_after) mx = seq_after - 1;
-        int mn = 0;
-        if (B.sliding_window > 0) mn = max(0, ctx_before + q_off - B.sliding_window + 1);
-        col_ok[nt] = ok;
-        col_lo[nt] = ok ? mn : 0;
-        col_hi[nt] = ok ? mx : -1;
-        if (ok) {
-            i_lo = max(i_lo, mn);
-            i_hi = min(i_hi, mx);
-            if (mn <= mx) {
-                u_lo = min(u_lo, mn);
-                u_hi = max(u_hi, mx);
+        col_lo[nt] = 0;
+        col_hi[nt] = -1;
+        col_ok[nt] = false;
+        ok_mask[nt] = 0u;
+    }
+    const bool simple = B.valid_token_mask == nullptr && B.sliding_window <= 0;
+    auto column_info = [&](bool accumulate) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int col = nt * 16 + n;
+            const int t = fast_div(col, P.q_group);
+            const int tok = tok0 + t;
+            const bool ok = t < tile_tokens && tok_ok[nt];
+            const int q_off = tok - rq_start;
+            int mx = (B.mask_mode == WARP34_ATTN_MASK_NONCAUSAL_WINDOW) ? seq_after - 1 : ctx_before + q_off;
+            if (mx >= seq_after) mx = seq_after - 1;
+            int mn = 0;
+            if (B.sliding_window > 0) mn = max(0, ctx_before + q_off - B.sliding_window + 1);
+            col_ok[nt] = ok;
+            col_lo[nt] = ok ? mn : 0;
+            col_hi[nt] = ok ? mx : -1;
+            if (ok) {
+                if (accumulate) {
+                    i_lo = max(i_lo, mn);
+                    i_hi = min(i_hi, mx);
+                    if (mn <= mx) {
+                        u_lo = min(u_lo, mn);
+                        u_hi = max(u_hi, mx);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int m = 0; m < 8; ++m) bq[nt][m] = u4{0u, 0u, 0u, 0u};
             }
-        } else {
-#pragma unroll
-            for (int m = 0; m < 8; ++m) bq[nt][m] = u4{0u, 0u, 0u, 0u};
+            ok_mask[nt] = (uint32_t)(__ballot(ok) & 0xFFFFull);
         }
-        ok_mask[nt] = (uint32_t)(__ballot(ok) & 0xFFFFull);
-    }
+    };
+    if (simple) {
+        if (tok0 >= B.total_tokens) return;  // no live column
+        const int q_off0 = tok0 - rq_start;
+        const bool window = B.mask_mode == WARP34_ATTN_MASK_NONCAUSAL_WINDOW;
+        int hi_first = window ? seq_after - 1 : ctx_before + q_off0;
+        int hi_last = window ? seq_after - 1 : ctx_before + q_off0 + tile_tokens - 1;
+        if (hi_first >= seq_after) hi_first = seq_after - 1;
+        if (hi_last >= seq_after) hi_last = seq_after - 1;
+        u_lo = 0;
+        u_hi = hi_last >= 0 ? hi_last : -1;
+        i_lo = 0;
+        i_hi = hi_first;
+    } else {
+        column_info(true);
 #pragma unroll
-    for (int off = 1; off < 16; off <<= 1) {
-        u_lo = min(u_lo, __shfl_xor(u_lo, off, 64));
-        u_hi = max(u_hi, __shfl_xor(u_hi, off, 64));
-        i_lo = max(i_lo, __shfl_xor(i_lo, off, 64));
-        i_hi = min(i_hi, __shfl_xor(i_hi, off, 64));
-    }
-    {
+        for (int off = 1; off < 16; off <<= 1) {
+            u_lo = min(u_lo, __shfl_xor(u_lo, off, 64));
+            u_hi = max(u_hi, __shfl_xor(u_hi, off, 64));
+            i_lo = max(i_lo, __shfl_xor(i_lo, off, 64));
+            i_hi = min(i_hi, __shfl_xor(i_hi, off, 64));
+        }
         uint32_t any = 0;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) any |= ok_mask[nt];
@@ -279,7 +306,11 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
         cu_first = item.u_begin;
         cu_end = item.u_end;
     } else {
-        g = chunk_geom(u_lo, u_hi, P.max_chunks, P.min_upc);
+        if (u_lo == 0 && B.max_seq_len > 0 && u_hi == B.max_seq_len - 1) {
+            g = ChunkGeom{0, P.spec_units, P.spec_upc, P.spec_chunks};  // as long as the host's bound
+        } else {
+            g = chunk_geom(u_lo, u_hi, P.max_chunks, P.min_upc);
+        }
         if (chunk >= g.n_chunks) return;
         cu_first = g.u_first + chunk * g.upc;
         cu_end = cu_first + g.upc;
@@ -292,7 +323,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
                             (size_t)kv_head * L.v_head_stride_bytes;
     uint8_t* stage = smem + wave * kKv16Stage;  // [K rows 0..15][V rows 0..15], kRowStride each
     const int32_t* req_blocks = B.block_tables + (size_t)req * B.max_blocks_per_req;
-    int slot_base = fast_div(cu_first * kUnit, L.block_size);
+    int slot_base = div_block(cu_first * kUnit, P);
     int page_vec;
     auto load_page_vec = [&]() {
         const int slot = slot_base + lane;
@@ -574,6 +605,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
     static_assert(kWaves == 8, "unit deal assumes two waves per SIMD");
     int hidx = 2 * unit, unit_no = 0;
     issue_half(hidx);
+    if (simple) column_info(false);
     while (unit < cu_end) {
         commit_half(hidx);
         int next_h = hidx + 1, next_unit = unit;
