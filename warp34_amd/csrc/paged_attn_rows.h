@@ -604,6 +604,14 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
     };
     static_assert(kWaves == 8, "unit deal assumes two waves per SIMD");
     int hidx = 2 * unit, unit_no = 0;
+    // The query operands are touched again after the first rows have been requested (dead columns
+    // are zeroed).  Loads return in order: a wait for them placed behind the row loads would wait
+    // for the rows too, so the compiler is made to finish them here, where they have long landed.
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int m = 0; m < 8; ++m)
+            asm volatile("" ::"v"(bq[nt][m][0]), "v"(bq[nt][m][1]), "v"(bq[nt][m][2]), "v"(bq[nt][m][3]));
     issue_half(hidx);
     if (simple) column_info(false);
     while (unit < cu_end) {
