@@ -66,8 +66,10 @@ MEASURED_TRAFFIC = {
     "tq4_decode_b1_ctx131072": (71_834_000, "profiles/paged_attn_tq4_decode_b1_ctx131072.txt"),
     "tq4_decode_b8_ctx131072": (558_377_000, "profiles/paged_attn_tq4_decode_b8_ctx131072.txt"),
     "tq4_decode_b32_ctx1k_64k": (586_269_000, "profiles/paged_attn_tq4_decode_b32_ctx1k_64k.txt"),
-    "bf16_decode_b1_ctx32768": (70_596_000, "profiles/paged_attn_rows_bf16_decode_b1_ctx32768.txt"),
-    "fp8_decode_b32_ctx1k_64k": (1_192_010_000, "profiles/paged_attn_rows_fp8_decode_b32_ctx1k_64k.txt"),
+    "bf16_decode_b1_ctx32768": (69_550_000, "profiles/paged_attn_rows_bf16_decode_b1_ctx32768.txt"),
+    "fp8_decode_b32_ctx1k_64k": (1_190_730_000, "profiles/paged_attn_rows_fp8_decode_b32_ctx1k_64k.txt"),
+    "fp8_decode_b1_ctx131072": (140_920_000, "profiles/paged_attn_rows_fp8_decode_b1_ctx131072.txt"),
+    "q8_0_decode_b1_ctx131072": (145_110_000, "profiles/paged_attn_rows_q8_0_decode_b1_ctx131072.txt"),
     "tq4_verify_16x4_ctx262144_shared200k": (736_353_000, "profiles/paged_attn_tq4_verify_16x4_ctx262144_shared200k.txt"),
     "tq4_prefill_8x2048_ctx16384": (1_134_522_000, "profiles/paged_prefill_tq4_8x2048_ctx16384.txt"),
     "tq4_qsa_sparse_16x513_ctx131072": (23_417_000, "profiles/qsa_sparse_tq4_16x513_ctx131072.txt"),

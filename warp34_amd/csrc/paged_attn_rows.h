@@ -91,8 +91,14 @@ __device__ __forceinline__ f4 mfma_x16(u2v a, u2v b, f4 c) {
 // a BF16 query is converted once.
 // BAL: the tile and its unit range come from `item` (balanced decode, see bal_for_each_piece)
 // instead of blockIdx.
-template <typename TQ, int NT, int KVF, bool BAL>
+// VRES (8-bit rows stored rotated): the value operand fp16(d * code) is followed by a second
+// operand holding its rounding residual, and every P V tile takes a second MFMA.  A scale block
+// of a rotated row with large entries holds few distinct codes, so part of the fp16 rounding of
+// d * code is common to the block, and the inverse rotation of the finished row would gather
+// that common part into a single channel.
+template <typename TQ, int NT, int KVF, bool BAL, bool VRES = false>
 __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, const BalItem& item) {
+    static_assert(!VRES || KVF == WARP34_KV_FORMAT_FP8_E4M3 || KVF == WARP34_KV_FORMAT_Q8_0, "residual operand: 8-bit rows");
     constexpr bool K8 = KVF == WARP34_KV_FORMAT_FP8_E4M3 || KVF == WARP34_KV_FORMAT_Q8_0;
     constexpr bool FP8 = KVF == WARP34_KV_FORMAT_FP8_E4M3;
     static_assert(K8 || KVF == TQ::kStorageFormat, "16-bit pages are read in the query type");
@@ -424,6 +430,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
         for (int nt = 0; nt < NT; ++nt) s_acc[nt] = f4{0.f, 0.f, 0.f, 0.f};
         // V operands of the 16 P V MFMAs: a_v[h][j] = element 128 h + 8 n + j of tokens 4b..4b+3
         u2v a_v[2][8];
+        u2v a_vr[VRES ? 2 : 1][VRES ? 8 : 1];  // residuals of a_v
         if constexpr (K8) {
             // Codes of row n, elements 32 m + 8 b .. + 7, widened to fp16; one partial score per
             // scale block (FP8: 2 blocks of 128 = m / 4; Q8_0: 4 blocks of 64 = m / 2), combined
@@ -486,8 +493,17 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
                     }
                 }
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    a_v[h][j] = u2v{pack_h2(vf[0][j], vf[1][j]), pack_h2(vf[2][j], vf[3][j])};
+                for (int j = 0; j < 8; ++j) {
+                    if constexpr (VRES) {
+                        uint32_t hi0, lo0, hi1, lo1;
+                        split_h2(vf[0][j], vf[1][j], hi0, lo0);
+                        split_h2(vf[2][j], vf[3][j], hi1, lo1);
+                        a_v[h][j] = u2v{hi0, hi1};
+                        a_vr[h][j] = u2v{lo0, lo1};
+                    } else {
+                        a_v[h][j] = u2v{pack_h2(vf[0][j], vf[1][j]), pack_h2(vf[2][j], vf[3][j])};
+                    }
+                }
             }
         } else {
             u4 ka[8];
@@ -581,6 +597,13 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
                     o_acc[nt][h][j] = mfma_x16<IS_BF16>(a, pb_hi[nt], o_acc[nt][h][j]);
                     if constexpr (IS_BF16) o_acc[nt][h][j] = mfma_x16<IS_BF16>(a, pb_lo[nt], o_acc[nt][h][j]);
                 }
+            }
+            if constexpr (VRES) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+                        o_acc[nt][h][j] = mfma_x16<false>(a_vr[h][j], pb_hi[nt], o_acc[nt][h][j]);
             }
         }
     };
@@ -725,16 +748,16 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
     }
 }
 
-template <typename TQ, int NT, int KVF>
+template <typename TQ, int NT, int KVF, bool VRES>
 __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_rows_kernel(const AttnParams P) {
     extern __shared__ __align__(16) uint8_t smem[];
-    rows_tile<TQ, NT, KVF, false>(P, smem, BalItem{});
+    rows_tile<TQ, NT, KVF, false, VRES>(P, smem, BalItem{});
 }
 
-template <typename TQ, int KVF>
+template <typename TQ, int KVF, bool VRES>
 __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_rows_balanced_kernel(const AttnParams P) {
     extern __shared__ __align__(16) uint8_t smem[];
-    bal_for_each_piece(P, [&](const BalItem& it) { rows_tile<TQ, 1, KVF, true>(P, smem, it); });
+    bal_for_each_piece(P, [&](const BalItem& it) { rows_tile<TQ, 1, KVF, true, VRES>(P, smem, it); });
 }
 
 }  // namespace w34
