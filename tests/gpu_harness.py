@@ -188,13 +188,17 @@ def assert_close(got_bits, dtype, want_f32, atol=2e-3, rtol=1e-2, what="", scale
 
     `plain_excess` (default 0) is an absolute allowance on top of the plain bound for the few
     cases that sit on the floor of fp16 operand arithmetic with x20 outlier inputs; a test that
-    passes one says which mechanism it is for.  Two exist.  (1) The dequantisation table holds
+    passes one says which mechanism it is for.  Three exist.  (1) The dequantisation table holds
     fp16 centroids (relative error up to 9.4e-5, the same for every element with the same code);
     a rotated row with outlier channels has elements of magnitude ~|V_c| / 16 everywhere, and
     the inverse rotation turns that code-wise error into single plain channels (c1 ^ c2 ^ c3 of
     the outlier channels): a few 1e-4 in rows that one key dominates.  (2) fp16 probability and
     value operands, as in the reference's MMA kernels: up to 2 * 2^-11 * sum_t p_t |V[t, c]|,
-    which passes 2e-3 when large values of opposite sign cancel in `want`.
+    which passes 2e-3 when large values of opposite sign cancel in `want`.  (3) The rotated query
+    is an fp16 operand (2^-12 per element, as in the reference's MMA kernels); against rotated key
+    rows with outlier channels (elements of magnitude ~|K_c| / 16 everywhere) a score moves by
+    ~1e-3, and where two keys share a row's weight the probabilities move by that much against
+    each other: a few 1e-4 over the bound on single elements.
 
     Every call is logged with the unscaled figures: max-abs error, max-rel (max|err| / max|want|)
     and the worst excess over atol + rtol * |want| on all channels (<= 0 means the plain contract

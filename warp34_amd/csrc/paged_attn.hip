@@ -1710,7 +1710,8 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     return rc;
 }
 
-template <typename TQ, int KVF>
+// VRES: value rows stored rotated in an 8-bit format (residual operand, see rows_tile)
+template <typename TQ, int KVF, bool VRES = false>
 static int launch_rows(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
                        const warp34_attention_batch* batch, const void* q, void* out, int num_q_heads,
                        int force_single, const void* gate) {
@@ -1773,9 +1774,9 @@ static int launch_rows(const warp34_exec* ex, const warp34_kv_layer_layout* layo
             P.part_ml = P.part_acc + prows * kHeadDim;
             P.bal_table = reinterpret_cast<int32_t*>(P.part_ml + prows * 4);
             P.max_chunks = groups + 1;
-            rc = ensure_dynamic_lds(paged_attn_rows_balanced_kernel<TQ, KVF>, kv16_smem_bytes(1));
+            rc = ensure_dynamic_lds(paged_attn_rows_balanced_kernel<TQ, KVF, VRES>, kv16_smem_bytes(1));
             if (rc) return rc;
-            hipLaunchKernelGGL((paged_attn_rows_balanced_kernel<TQ, KVF>), dim3((unsigned)groups, (unsigned)kv_subs),
+            hipLaunchKernelGGL((paged_attn_rows_balanced_kernel<TQ, KVF, VRES>), dim3((unsigned)groups, (unsigned)kv_subs),
                                dim3(kKv16Waves * 64), kv16_smem_bytes(1), stream, P);
             rc = (int)hipGetLastError();
             if (rc) return rc;
@@ -1785,9 +1786,9 @@ static int launch_rows(const warp34_exec* ex, const warp34_kv_layer_layout* layo
             return (int)hipGetLastError();
         }
     }
-    rc = ensure_dynamic_lds(paged_attn_rows_kernel<TQ, 1, KVF>, kv16_smem_bytes(1));
+    rc = ensure_dynamic_lds(paged_attn_rows_kernel<TQ, 1, KVF, VRES>, kv16_smem_bytes(1));
     if (rc) return rc;
-    hipLaunchKernelGGL((paged_attn_rows_kernel<TQ, 1, KVF>), grid, dim3(kKv16Waves * 64), kv16_smem_bytes(1), stream, P);
+    hipLaunchKernelGGL((paged_attn_rows_kernel<TQ, 1, KVF, VRES>), grid, dim3(kKv16Waves * 64), kv16_smem_bytes(1), stream, P);
     rc = (int)hipGetLastError();
     if (rc) return rc;
     if (P.max_chunks > 1) {
@@ -1846,9 +1847,20 @@ static int launch_prefill_tq4(const warp34_exec* ex, const warp34_kv_layer_layou
     const dim3 grid((unsigned)tiles, (unsigned)(layout->local_kv_heads * P.q_subgroups), (unsigned)batch->num_reqs);
     P.rot_q = layout->k_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 ? 1 : 0;
     P.rot_out = layout->v_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 ? 1 : 0;
-    int rc = ensure_dynamic_lds(paged_prefill_tq4_kernel<TQ, KVF>, PfLds<KVF>::kSmem, true);
+    constexpr bool k8bit = KVF == WARP34_KV_FORMAT_FP8_E4M3 || KVF == WARP34_KV_FORMAT_Q8_0;
+    int rc;
+    if constexpr (k8bit) {
+        if (P.rot_out || P.rot_q) {  // rotated 8-bit rows: exact codes in the tiles, scales outside
+            rc = ensure_dynamic_lds(paged_prefill_tq4_kernel<TQ, KVF, true>, PfLds<KVF>::kSmem, true);
+            if (rc) return rc;
+            hipLaunchKernelGGL((paged_prefill_tq4_kernel<TQ, KVF, true>), grid, dim3(kPfWaves * 64), PfLds<KVF>::kSmem,
+                               (hipStream_t)ex->stream, P);
+            return (int)hipGetLastError();
+        }
+    }
+    rc = ensure_dynamic_lds(paged_prefill_tq4_kernel<TQ, KVF, false>, PfLds<KVF>::kSmem, true);
     if (rc) return rc;
-    hipLaunchKernelGGL((paged_prefill_tq4_kernel<TQ, KVF>), grid, dim3(kPfWaves * 64), PfLds<KVF>::kSmem,
+    hipLaunchKernelGGL((paged_prefill_tq4_kernel<TQ, KVF, false>), grid, dim3(kPfWaves * 64), PfLds<KVF>::kSmem,
                        (hipStream_t)ex->stream, P);
     return (int)hipGetLastError();
 }
@@ -1945,6 +1957,8 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
                                (long long)batch->total_tokens * num_q_heads >= 128ll * kPfRows;
         if ((force_single || many_rows) && prefill_tq4_applicable(layout, batch, num_q_heads))
             return launch_prefill_tq4<TQ, WARP34_KV_FORMAT_FP8_E4M3>(ex, layout, batch, q, out, num_q_heads, gate);
+        if (layout->v_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256)
+            return launch_rows<TQ, WARP34_KV_FORMAT_FP8_E4M3, true>(ex, layout, batch, q, out, num_q_heads, force_single, gate);
         return launch_rows<TQ, WARP34_KV_FORMAT_FP8_E4M3>(ex, layout, batch, q, out, num_q_heads, force_single, gate);
     }
     if (is_kv8(layout, WARP34_KV_FORMAT_Q8_0)) {
@@ -1953,6 +1967,8 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
                                (long long)batch->total_tokens * num_q_heads >= 128ll * kPfRows;
         if ((force_single || many_rows) && prefill_tq4_applicable(layout, batch, num_q_heads))
             return launch_prefill_tq4<TQ, WARP34_KV_FORMAT_Q8_0>(ex, layout, batch, q, out, num_q_heads, gate);
+        if (layout->v_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256)
+            return launch_rows<TQ, WARP34_KV_FORMAT_Q8_0, true>(ex, layout, batch, q, out, num_q_heads, force_single, gate);
         return launch_rows<TQ, WARP34_KV_FORMAT_Q8_0>(ex, layout, batch, q, out, num_q_heads, force_single, gate);
     }
     return (int)hipErrorNotSupported;
@@ -2060,9 +2076,11 @@ static int launch_qsa_sparse(const warp34_exec* ex, const void* q, const void* g
     } else if (form == WARP34_KV_FORMAT_FP16) {
         rc = launch_rows_form(qsa_sparse_rows_kernel<WARP34_KV_FORMAT_FP16>);
     } else if (form == WARP34_KV_FORMAT_FP8_E4M3) {
-        rc = launch_rows_form(qsa_sparse_rows_kernel<WARP34_KV_FORMAT_FP8_E4M3>);
+        rc = P.rot_out ? launch_rows_form(qsa_sparse_rows_kernel<WARP34_KV_FORMAT_FP8_E4M3, true>)
+                       : launch_rows_form(qsa_sparse_rows_kernel<WARP34_KV_FORMAT_FP8_E4M3, false>);
     } else {
-        rc = launch_rows_form(qsa_sparse_rows_kernel<WARP34_KV_FORMAT_Q8_0>);
+        rc = P.rot_out ? launch_rows_form(qsa_sparse_rows_kernel<WARP34_KV_FORMAT_Q8_0, true>)
+                       : launch_rows_form(qsa_sparse_rows_kernel<WARP34_KV_FORMAT_Q8_0, false>);
     }
     if (rc) return rc;
     if (P.n_splits > 1) {

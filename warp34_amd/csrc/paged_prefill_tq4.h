@@ -30,7 +30,7 @@ constexpr int kPfRows = 128;                                  // query rows per 
 constexpr int kPfKStride = 528;                               // bytes per dequantised K row
 constexpr int kPfKBytes = 32 * kPfKStride;                    // 16896
 constexpr int kPfVBytes = 256 * 64;                           // V^T: 256 rows x 32 halves
-constexpr int kPfScaleBytes = 4 * 32 * 4;                     // K d0, K d1, V d0, V d1 per token
+constexpr int kPfScaleBytes = 8 * 32 * 4;                     // per token: K d0, K d1, V d0, V d1 (Q8_0: K d0-d3, V d0-d3)
 constexpr int kPfDeqBytes = kPfKBytes + kPfVBytes + kPfScaleBytes;
 // LDS map per page format: [table (TQ4 only)] [2 dequantised units] [2 raw units]
 template <int KVF>
@@ -63,12 +63,23 @@ __device__ __forceinline__ f4 pf_mfma32(h8 a, h8 b, f4 c) {
     }
 }
 
-template <typename TQ, int KVF>
+// VF (8-bit rows stored rotated): the value tile holds the codes themselves (exact in fp16) and
+// the block scales go into the probabilities as a high and a low fp16 operand, as for TQ4 rows.
+// fp16(d * code) rounds partly alike across a scale block that holds few distinct codes, and the
+// inverse rotation of the finished row would gather that common part into a single channel.
+// Q8_0 key tiles hold the codes too, and the scores take the fp32 block scales (see
+// dequant_unit_q8).
+template <typename TQ, int KVF, bool VF = false>
 __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(const AttnParams P) {
     using M = PfLds<KVF>;
     constexpr bool FP8 = M::kFp8;
     constexpr bool K16 = M::k16;  // 16-bit rows, read as stored: the MFMAs run in the storage type
-    constexpr bool Q8 = M::kQ8;   // Q8_0 rows: both tiles hold fp16(d * code), no scales afterwards
+    constexpr bool Q8 = M::kQ8;   // Q8_0 rows: the key tile holds fp16(d * code), and so does the value tile unless VF
+    static_assert(!VF || FP8 || Q8, "scales in the probabilities: 8-bit rows only");
+    // VF: the tile holds code / kVfGain (a power of two: exact) and the weights p * d * kVfGain.  The
+    // block scales of 8-bit rows are small (amax / 448, amax / 127): without the gain the low-order
+    // weight operand, 2^-12 of the weight, would fall into fp16's subnormal range and lose its bits.
+    constexpr float kVfGain = FP8 ? 256.0f : 128.0f;
     constexpr bool TQ4F = !FP8 && !K16 && !Q8;
     constexpr bool IS_BF16 = KVF == WARP34_KV_FORMAT_BF16;
     static_assert(!K16 || KVF == TQ::kStorageFormat, "16-bit pages are read in the query type");
@@ -413,9 +424,10 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         float da = *reinterpret_cast<const float*>(raw + kPfRawBytes / 2 + (2 * vp) * kRowB + 256 + 4 * (vj >> 4));
         float db = *reinterpret_cast<const float*>(raw + kPfRawBytes / 2 + (2 * vp + 1) * kRowB + 256 + 4 * (vj >> 4));
         float scale = 0.f;
-        if (tid < 64) {
-            const int x = tid >> 5, r = tid & 31;  // K d0, K d1
-            scale = *reinterpret_cast<const float*>(raw + r * kRowB + 256 + 4 * x);
+        if (tid < (VF ? 128 : 64)) {
+            const int x = tid >> 5, r = tid & 31;  // K d0, K d1 (VF: then V d0, V d1)
+            scale = *reinterpret_cast<const float*>(raw + (x >> 1) * (kPfRawBytes / 2) + r * kRowB + 256 + 4 * (x & 1));
+            if (x >= 2) scale = (t0 + r >= lo_all && t0 + r <= hi_all) ? scale * kVfGain : 0.f;
         }
         // ---- phase 2: widen ----
         u4 k_lo, k_hi;
@@ -455,14 +467,17 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             const int d = 8 * vj + e;
             // (token 2p, token 2p + 1) of dim d
             *reinterpret_cast<uint32_t*>(deq + kPfKBytes + d * 64 + 16 * (bp ^ ((d >> 1) & 3)) + 8 * sl + 4 * (vp & 1)) =
-                pack_h2(da * fa[e], db * fb[e]);
+                VF ? pack_h2(fa[e] * (1.0f / kVfGain), fb[e] * (1.0f / kVfGain)) : pack_h2(da * fa[e], db * fb[e]);
         }
-        if (tid < 64) *reinterpret_cast<float*>(deq + kPfKBytes + kPfVBytes + 4 * tid) = scale;
+        if (tid < (VF ? 128 : 64)) *reinterpret_cast<float*>(deq + kPfKBytes + kPfVBytes + 4 * tid) = scale;
     };
 
     // Q8_0 rows: four blocks of {fp32 d, 64 int8}.  Both tiles receive fp16(d * code), every element
-    // rounded on its own from fp32 (what the reference's MMA kernels stage, op_paged_attn.cu:59-71);
-    // thread roles as for FP8 rows.
+    // rounded on its own from fp32 (what the reference's MMA kernels stage, op_paged_attn.cu:59-71).
+    // VF (rotated rows): both tiles receive the codes (exact in fp16); the scores take the four
+    // fp32 block scales of the key, because fp16(d * code) keys of a rotated row with outlier
+    // channels (large elements everywhere) move a score by ~2e-3, enough to shift the weights of
+    // two dominant keys against each other.  Thread roles as for FP8 rows.
     auto dequant_unit_q8 = [&](int rawbuf, int deqbuf, int t0) {
         const uint8_t* raw = smem + kPfRawBase + rawbuf * kPfRawBytes;
         uint8_t* deq = smem + kPfDeqBase + deqbuf * kPfDeqBytes;
@@ -471,6 +486,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         // ---- phase 1: raw codes and scales ----
         const uint8_t* krow = raw + kr * kRowB + 68 * (kg >> 2);
         const float kd = *reinterpret_cast<const float*>(krow);
+        float kscale = 0.f;  // VF: scale of block tid / 32 of key row tid % 32
+        if (VF && tid < 128) kscale = *reinterpret_cast<const float*>(raw + (tid & 31) * kRowB + 68 * (tid >> 5));
         uint32_t kc[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) kc[i] = *reinterpret_cast<const uint32_t*>(krow + 4 + 16 * (kg & 3) + 4 * i);
@@ -484,14 +501,24 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             va[i] = *reinterpret_cast<const uint32_t*>(va_row + 4 + 8 * (vj & 7) + 4 * i);
             vb[i] = *reinterpret_cast<const uint32_t*>(vb_row + 4 + 8 * (vj & 7) + 4 * i);
         }
-        // ---- phase 2: dequantise ----
+        float vscale = 0.f;  // VF: scale of block (tid - 128) / 32 of value row tid % 32
+        if (VF && tid >= 128 && tid < 256) {
+            const int r = tid & 31;
+            vscale = *reinterpret_cast<const float*>(raw + kPfRawBytes / 2 + r * kRowB + 68 * ((tid - 128) >> 5));
+            vscale = (t0 + r >= lo_all && t0 + r <= hi_all) ? vscale * kVfGain : 0.f;
+        }
+        // ---- phase 2: widen the key codes (exact), dequantise the values ----
         uint32_t kh[8];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            float f[4];
-            codes4_to_f32<false>(kc[i], f);
-            kh[2 * i] = pack_h2(kd * f[0], kd * f[1]);
-            kh[2 * i + 1] = pack_h2(kd * f[2], kd * f[3]);
+            if constexpr (VF) {
+                i8x4_to_h4(kc[i], kh[2 * i], kh[2 * i + 1]);
+            } else {
+                float f[4];
+                codes4_to_f32<false>(kc[i], f);
+                kh[2 * i] = pack_h2(kd * f[0], kd * f[1]);
+                kh[2 * i + 1] = pack_h2(kd * f[2], kd * f[3]);
+            }
         }
         {
             const int pa = t0 + 2 * vp;
@@ -519,8 +546,10 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         for (int e = 0; e < 8; ++e) {
             const int d = 8 * vj + e;
             *reinterpret_cast<uint32_t*>(deq + kPfKBytes + d * 64 + 16 * (bp ^ ((d >> 1) & 3)) + 8 * sl + 4 * (vp & 1)) =
-                pack_h2(da * fa[e], db * fb[e]);
+                VF ? pack_h2(fa[e] * (1.0f / kVfGain), fb[e] * (1.0f / kVfGain)) : pack_h2(da * fa[e], db * fb[e]);
         }
+        if (VF && tid < 128) *reinterpret_cast<float*>(deq + kPfKBytes + kPfVBytes + 4 * tid) = kscale;
+        if (VF && tid >= 128 && tid < 256) *reinterpret_cast<float*>(deq + kPfKBytes + kPfVBytes + 4 * tid) = vscale;
     };
 
     // 16-bit rows: nothing to dequantise.  K: thread (row r = tid / 16, segment g = tid % 16)
@@ -573,6 +602,25 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             if constexpr (!K16 && !Q8) {
                 kd0 = *reinterpret_cast<const f4*>(sc + 16 * s + 4 * b);
                 kd1 = *reinterpret_cast<const f4*>(sc + 32 + 16 * s + 4 * b);
+            }
+            if constexpr (Q8 && VF) {
+                // one partial score per 64-element scale block (two 32-wide steps), then the fp32 scales
+                f4 kd[4], s_blk[4];
+#pragma unroll
+                for (int blk = 0; blk < 4; ++blk) {
+                    kd[blk] = *reinterpret_cast<const f4*>(sc + 32 * blk + 16 * s + 4 * b);
+                    s_blk[blk] = f4{0.f, 0.f, 0.f, 0.f};
+                }
+#pragma unroll
+                for (int m = 0; m < 4; ++m)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+                        s_blk[2 * h + (m >> 1)] = pf_mfma32<false>(a[h][m], bq[h][m], s_blk[2 * h + (m >> 1)]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    score[4 * s + i] = (kd[0][i] * s_blk[0][i] + kd[1][i] * s_blk[1][i]) +
+                                       (kd[2][i] * s_blk[2][i] + kd[3][i] * s_blk[3][i]);
+                continue;
             }
             f4 s_acc[2] = {f4{0.f, 0.f, 0.f, 0.f}, f4{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
@@ -636,7 +684,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         }
         u4 pb[2];
         u4 pb_lo = {0u, 0u, 0u, 0u};
-        u4 pb_l2[2] = {u4{0u, 0u, 0u, 0u}, u4{0u, 0u, 0u, 0u}};  // TQ4: low-order operands per half
+        u4 pb_l2[2] = {u4{0u, 0u, 0u, 0u}, u4{0u, 0u, 0u, 0u}};  // TQ4, rotated FP8: low-order operands per half
+        u4 pq[Q8 && VF ? 4 : 1], pq_lo[Q8 && VF ? 4 : 1];        // rotated Q8_0: operands per 64-element block
         if constexpr (IS_BF16) {
             // bf16 keeps 8 bits of a probability: the rest goes into a second operand (two MFMAs)
             uint32_t hi[8], lo[8];
@@ -648,9 +697,29 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             pb[0] = u4{hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16), hi[4] | (hi[5] << 16), hi[6] | (hi[7] << 16)};
             pb[1] = pb[0];
             pb_lo = u4{lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16), lo[4] | (lo[5] << 16), lo[6] | (lo[7] << 16)};
-        } else if constexpr (FP8 || K16 || Q8) {  // the value tile already carries its scales
+        } else if constexpr ((FP8 || K16 || Q8) && !VF) {  // the value tile already carries its scales
             pb[0] = u4{pack_h2(p[0], p[1]), pack_h2(p[2], p[3]), pack_h2(p[4], p[5]), pack_h2(p[6], p[7])};
             pb[1] = pb[0];
+        } else if constexpr (Q8) {
+#pragma unroll
+            for (int blk = 0; blk < 4; ++blk) {
+                const f4 da = *reinterpret_cast<const f4*>(sc + 128 + 32 * blk + 4 * b);
+                const f4 db = *reinterpret_cast<const f4*>(sc + 128 + 32 * blk + 16 + 4 * b);
+                float w[8];
+#pragma unroll
+                for (int t = 0; t < 8; ++t) w[t] = p[t] * (t < 4 ? da[t] : db[t - 4]);
+                if (MASKED) {
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) w[t] = p[t] > 0.f ? w[t] : 0.f;
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    uint32_t whi, wlo;
+                    split_h2(w[2 * k], w[2 * k + 1], whi, wlo);
+                    pq[blk][k] = whi;
+                    pq_lo[blk][k] = wlo;
+                }
+            }
         } else {
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
@@ -683,6 +752,15 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
                 const int d = 128 * h + 16 * j + n;
                 a[j] = (IS_BF16 && h == 0) ? av0[j] : *reinterpret_cast<const h8*>(vb + d * 64 + 16 * (b ^ ((d >> 1) & 3)));
             }
+            if constexpr (Q8 && VF) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    o_acc[h][j] = pf_mfma32<false>(a[j], __builtin_bit_cast(h8, pq[2 * h + (j >> 2)]), o_acc[h][j]);
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    o_acc[h][j] = pf_mfma32<false>(a[j], __builtin_bit_cast(h8, pq_lo[2 * h + (j >> 2)]), o_acc[h][j]);
+                continue;
+            }
 #pragma unroll
             for (int j = 0; j < 8; ++j) o_acc[h][j] = pf_mfma32<IS_BF16>(a[j], __builtin_bit_cast(h8, pb[h]), o_acc[h][j]);
             // the low-order operands in a pass of their own: a tile's two MFMAs are then eight
@@ -691,7 +769,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
 #pragma unroll
                 for (int j = 0; j < 8; ++j) o_acc[h][j] = pf_mfma32<true>(a[j], __builtin_bit_cast(h8, pb_lo), o_acc[h][j]);
             }
-            if constexpr (TQ4F) {
+            if constexpr (TQ4F || (FP8 && VF)) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) o_acc[h][j] = pf_mfma32<false>(a[j], __builtin_bit_cast(h8, pb_l2[h]), o_acc[h][j]);
             }

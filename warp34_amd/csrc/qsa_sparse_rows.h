@@ -10,8 +10,11 @@
 
 namespace w34 {
 
-template <int KVF>
+// VRES (8-bit value rows stored rotated): a second operand with the rounding residuals of
+// fp16(d * code) and a second MFMA per P V tile, as in rows_tile.
+template <int KVF, bool VRES = false>
 __global__ __launch_bounds__(kKv16Waves * 64, 1) void qsa_sparse_rows_kernel(const QsaParams P) {
+    static_assert(!VRES || KVF == WARP34_KV_FORMAT_FP8_E4M3 || KVF == WARP34_KV_FORMAT_Q8_0, "residual operand: 8-bit rows");
     constexpr bool K8 = KVF == WARP34_KV_FORMAT_FP8_E4M3 || KVF == WARP34_KV_FORMAT_Q8_0;
     constexpr bool FP8 = KVF == WARP34_KV_FORMAT_FP8_E4M3;
     constexpr int kWaves = kKv16Waves;
@@ -208,6 +211,7 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void qsa_sparse_rows_kernel(con
         const uint8_t* v_rows = stage + 16 * kRowStride;
         f4 s_acc = f4{0.f, 0.f, 0.f, 0.f};
         u2v a_v[2][8];
+        u2v a_vr[VRES ? 2 : 1][VRES ? 8 : 1];  // residuals of a_v
         if constexpr (K8) {
             constexpr int kBlocks = FP8 ? 2 : 4;
             constexpr int kMPerBlock = 8 / kBlocks;
@@ -262,7 +266,17 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void qsa_sparse_rows_kernel(con
                     }
                 }
 #pragma unroll
-                for (int j = 0; j < 8; ++j) a_v[h][j] = u2v{pack_h2(vf[0][j], vf[1][j]), pack_h2(vf[2][j], vf[3][j])};
+                for (int j = 0; j < 8; ++j) {
+                    if constexpr (VRES) {
+                        uint32_t hi0, lo0, hi1, lo1;
+                        split_h2(vf[0][j], vf[1][j], hi0, lo0);
+                        split_h2(vf[2][j], vf[3][j], hi1, lo1);
+                        a_v[h][j] = u2v{hi0, hi1};
+                        a_vr[h][j] = u2v{lo0, lo1};
+                    } else {
+                        a_v[h][j] = u2v{pack_h2(vf[0][j], vf[1][j]), pack_h2(vf[2][j], vf[3][j])};
+                    }
+                }
             }
         } else {
             u4 ka[8];
@@ -318,6 +332,12 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void qsa_sparse_rows_kernel(con
         for (int h = 0; h < 2; ++h)
 #pragma unroll
             for (int j = 0; j < 8; ++j) o_acc[h][j] = mfma_x16<false>(a_v[h][j], pb, o_acc[h][j]);
+        if constexpr (VRES) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) o_acc[h][j] = mfma_x16<false>(a_vr[h][j], pb, o_acc[h][j]);
+        }
     };
 
     int half = ch_first + wave;
