@@ -1850,7 +1850,7 @@ static int launch_prefill_tq4(const warp34_exec* ex, const warp34_kv_layer_layou
     constexpr bool k8bit = KVF == WARP34_KV_FORMAT_FP8_E4M3 || KVF == WARP34_KV_FORMAT_Q8_0;
     int rc;
     if constexpr (k8bit) {
-        if (P.rot_out || P.rot_q) {  // rotated 8-bit rows: exact codes in the tiles, scales outside
+        if (P.rot_out) {  // rotated 8-bit value rows: codes in the value tile, block scales in the weights
             rc = ensure_dynamic_lds(paged_prefill_tq4_kernel<TQ, KVF, true>, PfLds<KVF>::kSmem, true);
             if (rc) return rc;
             hipLaunchKernelGGL((paged_prefill_tq4_kernel<TQ, KVF, true>), grid, dim3(kPfWaves * 64), PfLds<KVF>::kSmem,

@@ -67,14 +67,13 @@ __device__ __forceinline__ f4 pf_mfma32(h8 a, h8 b, f4 c) {
 // the block scales go into the probabilities as a high and a low fp16 operand, as for TQ4 rows.
 // fp16(d * code) rounds partly alike across a scale block that holds few distinct codes, and the
 // inverse rotation of the finished row would gather that common part into a single channel.
-// Q8_0 key tiles hold the codes too, and the scores take the fp32 block scales (see
-// dequant_unit_q8).
+// (Q8_0 key tiles hold the codes in either form, see dequant_unit_q8.)
 template <typename TQ, int KVF, bool VF = false>
 __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(const AttnParams P) {
     using M = PfLds<KVF>;
     constexpr bool FP8 = M::kFp8;
     constexpr bool K16 = M::k16;  // 16-bit rows, read as stored: the MFMAs run in the storage type
-    constexpr bool Q8 = M::kQ8;   // Q8_0 rows: the key tile holds fp16(d * code), and so does the value tile unless VF
+    constexpr bool Q8 = M::kQ8;   // Q8_0 rows: the key tile holds the codes, the value tile fp16(d * code) unless VF
     static_assert(!VF || FP8 || Q8, "scales in the probabilities: 8-bit rows only");
     // VF: the tile holds code / kVfGain (a power of two: exact) and the weights p * d * kVfGain.  The
     // block scales of 8-bit rows are small (amax / 448, amax / 127): without the gain the low-order
@@ -189,6 +188,11 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             if ((ok_mask >> c) & 1u) {
                 if constexpr (K16) {
                     packed = q_raw[c];  // as given: the scores are scaled after the MFMAs
+                } else if constexpr (FP8 || Q8) {
+                    // the softmax factor is applied with the fp32 key scales: an un-rotated fp16
+                    // query enters the MFMAs exactly as given
+                    packed.x = pack_h2(v[0], v[1]);
+                    packed.y = pack_h2(v[2], v[3]);
                 } else {
                     packed.x = pack_h2(v[0] * q_scale, v[1] * q_scale);
                     packed.y = pack_h2(v[2] * q_scale, v[3] * q_scale);
@@ -428,6 +432,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             const int x = tid >> 5, r = tid & 31;  // K d0, K d1 (VF: then V d0, V d1)
             scale = *reinterpret_cast<const float*>(raw + (x >> 1) * (kPfRawBytes / 2) + r * kRowB + 256 + 4 * (x & 1));
             if (x >= 2) scale = (t0 + r >= lo_all && t0 + r <= hi_all) ? scale * kVfGain : 0.f;
+            else scale *= q_scale;  // the softmax factor rides on the key scales: the query operand stays unscaled
         }
         // ---- phase 2: widen ----
         u4 k_lo, k_hi;
@@ -472,12 +477,12 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         if (tid < (VF ? 128 : 64)) *reinterpret_cast<float*>(deq + kPfKBytes + kPfVBytes + 4 * tid) = scale;
     };
 
-    // Q8_0 rows: four blocks of {fp32 d, 64 int8}.  Both tiles receive fp16(d * code), every element
-    // rounded on its own from fp32 (what the reference's MMA kernels stage, op_paged_attn.cu:59-71).
-    // VF (rotated rows): both tiles receive the codes (exact in fp16); the scores take the four
-    // fp32 block scales of the key, because fp16(d * code) keys of a rotated row with outlier
-    // channels (large elements everywhere) move a score by ~2e-3, enough to shift the weights of
-    // two dominant keys against each other.  Thread roles as for FP8 rows.
+    // Q8_0 rows: four blocks of {fp32 d, 64 int8}.  The key tile receives the codes (exact in fp16)
+    // and the scores take the four fp32 block scales: keys staged as fp16(d * code), as in the
+    // reference's MMA kernels (op_paged_attn.cu:59-71), move a score by ~2e-3 when the row has
+    // outlier channels, enough to shift the weights of two dominant keys against each other.  The
+    // value tile receives fp16(d * code), every element rounded on its own from fp32 (VF: the
+    // codes).  Thread roles as for FP8 rows.
     auto dequant_unit_q8 = [&](int rawbuf, int deqbuf, int t0) {
         const uint8_t* raw = smem + kPfRawBase + rawbuf * kPfRawBytes;
         uint8_t* deq = smem + kPfDeqBase + deqbuf * kPfDeqBytes;
@@ -485,9 +490,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         const int vp = tid & 15, vj = tid >> 4;
         // ---- phase 1: raw codes and scales ----
         const uint8_t* krow = raw + kr * kRowB + 68 * (kg >> 2);
-        const float kd = *reinterpret_cast<const float*>(krow);
-        float kscale = 0.f;  // VF: scale of block tid / 32 of key row tid % 32
-        if (VF && tid < 128) kscale = *reinterpret_cast<const float*>(raw + (tid & 31) * kRowB + 68 * (tid >> 5));
+        float kscale = 0.f;  // scale of block tid / 32 of key row tid % 32, times the softmax factor
+        if (tid < 128) kscale = *reinterpret_cast<const float*>(raw + (tid & 31) * kRowB + 68 * (tid >> 5)) * q_scale;
         uint32_t kc[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) kc[i] = *reinterpret_cast<const uint32_t*>(krow + 4 + 16 * (kg & 3) + 4 * i);
@@ -510,16 +514,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         // ---- phase 2: widen the key codes (exact), dequantise the values ----
         uint32_t kh[8];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            if constexpr (VF) {
-                i8x4_to_h4(kc[i], kh[2 * i], kh[2 * i + 1]);
-            } else {
-                float f[4];
-                codes4_to_f32<false>(kc[i], f);
-                kh[2 * i] = pack_h2(kd * f[0], kd * f[1]);
-                kh[2 * i + 1] = pack_h2(kd * f[2], kd * f[3]);
-            }
-        }
+        for (int i = 0; i < 4; ++i) i8x4_to_h4(kc[i], kh[2 * i], kh[2 * i + 1]);
         {
             const int pa = t0 + 2 * vp;
             const bool a_ok = pa >= lo_all && pa <= hi_all, b_ok = pa + 1 >= lo_all && pa + 1 <= hi_all;
@@ -548,7 +543,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             *reinterpret_cast<uint32_t*>(deq + kPfKBytes + d * 64 + 16 * (bp ^ ((d >> 1) & 3)) + 8 * sl + 4 * (vp & 1)) =
                 VF ? pack_h2(fa[e] * (1.0f / kVfGain), fb[e] * (1.0f / kVfGain)) : pack_h2(da * fa[e], db * fb[e]);
         }
-        if (VF && tid < 128) *reinterpret_cast<float*>(deq + kPfKBytes + kPfVBytes + 4 * tid) = kscale;
+        if (tid < 128) *reinterpret_cast<float*>(deq + kPfKBytes + kPfVBytes + 4 * tid) = kscale;
         if (VF && tid >= 128 && tid < 256) *reinterpret_cast<float*>(deq + kPfKBytes + kPfVBytes + 4 * tid) = vscale;
     };
 
@@ -603,7 +598,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
                 kd0 = *reinterpret_cast<const f4*>(sc + 16 * s + 4 * b);
                 kd1 = *reinterpret_cast<const f4*>(sc + 32 + 16 * s + 4 * b);
             }
-            if constexpr (Q8 && VF) {
+            if constexpr (Q8) {
                 // one partial score per 64-element scale block (two 32-wide steps), then the fp32 scales
                 f4 kd[4], s_blk[4];
 #pragma unroll
@@ -630,9 +625,6 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             if constexpr (K16) {  // rows as stored: no scales, the softmax factor comes in here
 #pragma unroll
                 for (int i = 0; i < 4; ++i) score[4 * s + i] = (s_acc[0][i] + s_acc[1][i]) * q_scale;
-            } else if constexpr (Q8) {  // the key tile already carries its scales
-#pragma unroll
-                for (int i = 0; i < 4; ++i) score[4 * s + i] = s_acc[0][i] + s_acc[1][i];
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) score[4 * s + i] = kd0[i] * s_acc[0][i] + kd1[i] * s_acc[1][i];
