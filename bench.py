@@ -43,6 +43,8 @@ WORKLOADS = {
     "fp8_prefill_8x2048_ctx16384": ("fp8", [18432] * 8, 0),
     "bf16_prefill_8x2048_ctx16384": ("bf16", [18432] * 8, 0),
     "q8_0_prefill_8x2048_ctx16384": ("q8_0", [18432] * 8, 0),
+    # quantize-on-append alone: 4 096 tokens x 2 kv heads (K and V) from bf16 into 64-token TQ4 pages
+    "tq4_append_4096": ("tq4", [4096], 0),
     # producer side: QK RMSNorm + RoPE fused with the TQ4 append of an 8 192-token chunk
     "tq4_norm_rope_append_8192": ("tq4", [8192], 0),
     # the target model's producer: Gemma RMSNorm + interleaved mRoPE + gate split fused with the TQ4 append
@@ -451,6 +453,59 @@ def run_qsa(args, torch, lib, ffi, layers, ctx_len, n_layers, n_tok, fmt, select
     }))
 
 
+def run_append(args, torch, lib, ffi, layers, n, n_layers, fmt):
+    """Quantize-on-append alone: n tokens x KV_HEADS (K and V) of bf16 rows into the pages of one
+    layer, the layers cycled.  One step = one layer's append of an n-token chunk."""
+    dev = "cuda:0"
+    k = synth_normal(torch, ffi, (n, KV_HEADS * HEAD_DIM), 21)
+    v = synth_normal(torch, ffi, (n, KV_HEADS * HEAD_DIM), 22)
+    ex = ffi.Warp34Exec(torch.cuda.current_stream().cuda_stream, 0, 0, 0)
+    per_layer = []
+    for L in layers:
+        posn = torch.arange(0, n, device=dev)
+        slots = (L.block_tables[0, (posn // BLOCK)].to(torch.int64) * BLOCK + posn % BLOCK).to(torch.int32)
+        qsl = torch.tensor([0, n], dtype=torch.int32, device=dev)
+        seq = torch.tensor([n], dtype=torch.int32, device=dev)
+        batch = ffi.Warp34AttentionBatch(qsl.data_ptr(), None, seq.data_ptr(), L.block_tables.data_ptr(),
+                                         slots.data_ptr(), None, None, 1, n, L.max_blocks, n, n, 0, 0, 0.0625, 0)
+        per_layer.append((L, slots, batch, qsl, seq))
+    vp = lambda t: C.c_void_p(t.data_ptr())
+
+    def step(i):
+        L, _, batch, _, _ = per_layer[i % n_layers]
+        rc = lib.warp34_kv_cache_write_bf16(C.byref(ex), C.byref(L.layout), C.byref(batch), vp(k), vp(v))
+        if rc:
+            raise RuntimeError("warp34_kv_cache_write_bf16 rc=%d" % rc)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(args.steps):
+        step(i)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / args.steps
+    # algorithmic bytes: one bf16 row read and one encoded row written per (token, kv head, K | V), one slot per token
+    bytes_step = n * KV_HEADS * 2 * (HEAD_DIM * 2 + ROW_BYTES[fmt]) + n * 4
+    gbs = bytes_step / (ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "quantize-on-append into %s pages: us/layer + achieved HBM GB/s" % fmt.upper(),
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 6), "us_per_layer": round(ms * 1e3, 2), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": args.workload, "tokens": n, "kv_heads": KV_HEADS, "head_dim": HEAD_DIM,
+                   "page_tokens": BLOCK, "kv_format": "tq4+wht256" if fmt == "tq4" else fmt, "kv_pools_cycled": n_layers,
+                   "bytes_per_step": bytes_step},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, (None, None))[0],
+                     "traffic_source": MEASURED_TRAFFIC.get(args.workload, (None, None))[1],
+                     "kernel": "kv_append_kernel", "avg_launch_us": round(ms * 1e3, 2)},
+    }))
+
+
 def run_producer(args, torch, lib, ffi, layers, n, n_layers, fmt):
     """QK RMSNorm + RoPE over packed bf16 [n, (16 + 2 * 2) * 256] rows with the K / V rows written
     into TQ4 pages: the fused entry point against the two-call sequence (operator in place, then
@@ -698,6 +753,8 @@ def run_workload(args, torch, lib, ffi, dev):
         kv_bytes = (shared + sum(int(c) - shared for c in ctx)) * KV_HEADS * 2 * row_bytes
     layer_bytes = 2 * pool_pages * KV_HEADS * BLOCK * row_bytes
     n_layers = args.layers or max(2, -(-(640 << 20) // layer_bytes))
+    if args.workload.startswith("tq4_append_") and not args.layers:
+        n_layers = 8  # the chunk being appended is cache-hot in real use too (its producer has just written it)
     layers = [Layer(torch, lib, ffi, fmt, ctx, pool_pages, s, shared) for s in range(n_layers)]
 
     if "_prefill_" in args.workload:
@@ -714,6 +771,9 @@ def run_workload(args, torch, lib, ffi, dev):
         return None
     if "_norm_rope_append_" in args.workload:
         run_producer(args, torch, lib, ffi, layers, int(ctx[0]), n_layers, fmt)
+        return None
+    if "_append_" in args.workload:
+        run_append(args, torch, lib, ffi, layers, int(ctx[0]), n_layers, fmt)
         return None
 
     R = len(ctx)

@@ -188,10 +188,17 @@ __global__ __launch_bounds__(256) void fused_qk_norm_rope_gate_kernel(const Fuse
                                (size_t)page * (is_v_half ? P.L.v_page_stride_bytes : P.L.k_page_stride_bytes) +
                                (size_t)kv_head * (is_v_half ? P.L.v_head_stride_bytes : P.L.k_head_stride_bytes) +
                                (size_t)off * (is_v_half ? P.L.v_token_stride_bytes : P.L.k_token_stride_bytes);
-                // element lane + 32 j of the finished row (head_dim 256, host check)
+                // elements 8 l32 .. 8 l32 + 7 of the finished row (head_dim 256, host check)
                 float v[8];
+                {
+                    const uint4 r8 = *reinterpret_cast<const uint4*>(row + 8 * l32);
+                    const uint32_t w[4] = {r8.x, r8.y, r8.z, r8.w};
 #pragma unroll
-                for (int j = 0; j < 8; ++j) v[j] = F16::to_f32(row[l32 + 32 * j]);
+                    for (int j = 0; j < 4; ++j) {
+                        v[2 * j] = F16::to_f32((uint16_t)(w[j] & 0xffffu));
+                        v[2 * j + 1] = F16::to_f32((uint16_t)(w[j] >> 16));
+                    }
+                }
                 encode_store_row(v, is_v_half ? P.L.v_format : P.L.k_format, is_v_half ? P.L.v_transform : P.L.k_transform,
                                  lane, s_enc[wave][half_id], dst);
             }

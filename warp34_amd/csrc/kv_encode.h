@@ -1,21 +1,24 @@
 // Row encoders of the paged KV formats for gfx950, shared by the append kernel and the fused
-// QK-norm + RoPE + append kernel.  A row is encoded by one half of a wave64 (32 lanes); the
-// arithmetic and its order follow the reference's 32-lane warp (op_kv_cache.cu:32-218) and are
-// bit-exact with the CPU restatement when the including file is built with -ffp-contract=off.
+// QK-norm + RoPE + append kernels.  A row is encoded by one half of a wave64 (32 lanes); the
+// arithmetic and the order of every sum follow the reference's 32-lane warp
+// (op_kv_cache.cu:32-218, tq4_kv_common.cuh:54-107) and are bit-exact with the CPU restatement
+// when the including file is built with -ffp-contract=off.
+//
+// Data layout: lane l32 holds the eight consecutive elements 8 l32 .. 8 l32 + 7 (the reference's
+// lane holds l32 + 32 j).  Index bits 0-2 are then register bits and bits 3-7 lane bits.  The
+// butterfly stages run in the reference's order (1, 2, 4, ..., 128, the scale on the last); its
+// 32-element sums (one per register there: elements 32 j .. 32 j + 31) are four-lane groups
+// here, all eight reduced by ONE pass of the same tree (xor 16, 8 across lanes; xor 4, 2, 1
+// across registers); two neighbouring codes share a lane.  Every sum adds the same operands in
+// the same order, so the bytes are those of the 32-lane form at half its instruction count.
 #pragma once
 
 #include "kv_common.h"
 
 namespace w34 {
 
-// Cross-lane moves are DPP / lane-swap VALU operations (lane_xor), not LDS permutes: the encode
-// of one row needs 168 of them.  They only move bits, so the arithmetic (and its order) is the
-// one of the 32-lane shuffle tree it replaces.
-__device__ __forceinline__ int lane_xor1_int(int x, int lane) {
-    return __float_as_int(lane_xor<1>(__int_as_float(x), lane));
-}
-
-// 32-lane xor butterfly sum, offsets 16,8,4,2,1 (tq4_kv_common.cuh:54-60).
+// 32-lane xor butterfly sum, offsets 16,8,4,2,1 (tq4_kv_common.cuh:54-60); cross-lane moves are
+// DPP / lane-swap VALU operations (lane_xor), not LDS permutes.
 __device__ __forceinline__ float half_wave_sum(float v, int lane) {
     v += lane_xor<16>(v, lane);
     v += lane_xor<8>(v, lane);
@@ -25,26 +28,30 @@ __device__ __forceinline__ float half_wave_sum(float v, int lane) {
     return v;
 }
 
+// One butterfly stage across lanes: lanes with bit H clear take x + x[lane ^ H], the others
+// x[lane ^ H] - x (tq4_kv_common.cuh:75-107).  flip = sign bit in the lanes with bit H set.
 template <int H>
-__device__ __forceinline__ float wht_lane_stage(float val, int lane) {
-    const float o = lane_xor<H>(val, lane);
-    return (lane & H) ? (o - val) : (val + o);
+__device__ __forceinline__ float wht_lane_stage(float val, uint32_t flip, int lane) {
+    if constexpr (H == 16) {
+        // after the swap r[0] holds the even-row operand and r[1] the odd-row operand, in both rows
+        const uint32_t xi = __float_as_uint(val);
+        const auto r = __builtin_amdgcn_permlane16_swap(xi, xi, false, false);
+        return __uint_as_float(r[0]) + __uint_as_float(r[1] ^ flip);
+    } else {
+        return lane_xor<H>(val, lane) + __uint_as_float(__float_as_uint(val) ^ flip);
+    }
 }
 
-// 256-point Walsh-Hadamard over 32 lanes x 8 registers (tq4_kv_common.cuh:75-107):
-// stages over index bits 0..4 cross lanes, bits 5..7 stay in registers; the last stage
-// carries the 1/16 scale.
-__device__ __forceinline__ void wht256_half_wave(float (&v)[8], int lane) {
+// sign[i] * x[i], then the 256-point Walsh-Hadamard transform with the 1/16 scale on the last
+// stage; v[j] = x[8 l32 + j] on entry and y[8 l32 + j] on return.
+__device__ __forceinline__ void sign_wht256(float (&v)[8], int lane) {
+    const int l32 = lane & 31;
+    {
+        const uint32_t sb = sign_word(l32 >> 2) >> (8 * (l32 & 3));
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        float val = v[j];
-        val = wht_lane_stage<1>(val, lane);
-        val = wht_lane_stage<2>(val, lane);
-        val = wht_lane_stage<4>(val, lane);
-        val = wht_lane_stage<8>(val, lane);
-        val = wht_lane_stage<16>(val, lane);
-        v[j] = val;
+        for (int j = 0; j < 8; ++j) v[j] = __uint_as_float(__float_as_uint(v[j]) ^ (((sb >> j) & 1u) << 31));
     }
+    // stages 1, 2, 4: registers
 #pragma unroll
     for (int j = 0; j < 8; j += 2) {
         const float a = v[j], b = v[j + 1];
@@ -63,60 +70,103 @@ __device__ __forceinline__ void wht256_half_wave(float (&v)[8], int lane) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const float a = v[i], b = v[i + 4];
-        v[i] = (a + b) * 0.0625f;
-        v[i + 4] = (a - b) * 0.0625f;
+        v[i] = a + b;
+        v[i + 4] = a - b;
     }
+    // stages 8 .. 128: lanes (each stage over all eight registers: independent instructions
+    // between a write and the cross-lane read of it)
+    const uint32_t f1 = (uint32_t)(lane & 1) << 31, f2 = (uint32_t)(lane & 2) << 30, f4 = (uint32_t)(lane & 4) << 29;
+    const uint32_t f8 = (uint32_t)(lane & 8) << 28, f16 = (uint32_t)(lane & 16) << 27;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = wht_lane_stage<1>(v[j], f1, lane);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = wht_lane_stage<2>(v[j], f2, lane);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = wht_lane_stage<4>(v[j], f4, lane);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = wht_lane_stage<8>(v[j], f8, lane);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = wht_lane_stage<16>(v[j], f16, lane) * 0.0625f;
 }
 
-// TQ4 encode of one 256-wide row held as v[j] = x[l32 + 32 j] (op_kv_cache.cu:152-218).
-// The 132 row bytes are assembled in `row` (LDS, private to this half-wave).
+// sums of the eight 32-element groups: lanes 4 g .. 4 g + 3 receive the sum of group g, added
+// in the order of the 32-lane butterfly (element e with e ^ 16, then ^ 8, ^ 4, ^ 2, ^ 1)
+__device__ __forceinline__ float group32_sums(const float (&p)[8], int lane) {
+    float t[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) t[r] = p[r] + lane_xor<2>(p[r], lane);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) t[r] = t[r] + lane_xor<1>(t[r], lane);
+    const float a0 = t[0] + t[4], a1 = t[1] + t[5], a2 = t[2] + t[6], a3 = t[3] + t[7];
+    const float b0 = a0 + a2, b1 = a1 + a3;
+    return b0 + b1;
+}
+
+// (((0 + S0) + S1) + S2) + S3 over the four groups of a 16-lane row, in every lane of the row
+__device__ __forceinline__ float row_sum_of_groups(float s, int lane) {
+    float x = 0.0f + s;  // the reference accumulates from +0: a sum of -0 terms ends as +0
+    x = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x114, 0xF, 0xF, false)) + s;  // row_shr:4
+    x = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x114, 0xF, 0xF, false)) + s;
+    x = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x114, 0xF, 0xF, false)) + s;
+    // lanes 12-15 of the row hold the total; hand it to the whole row
+    return __int_as_float(__builtin_amdgcn_ds_bpermute((lane | 12) << 2, __float_as_int(x)));
+}
+
+// TQ4 encode of one 256-wide row, v[j] = x[8 l32 + j] (op_kv_cache.cu:152-218).  The 132 row
+// bytes are assembled in `row` (LDS, private to this half-wave).  Lanes 0-15 hold the first
+// scale block, lanes 16-31 the second: one instruction stream computes both norms and scales.
 __device__ __forceinline__ void tq4_encode_row(float (&v)[8], int lane, uint8_t* row) {
     const int l32 = lane & 31;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = apply_sign(v[j], l32 + 32 * j);
-    wht256_half_wave(v, lane);
+    // tables in lanes: entry i in every lane with lane % 16 == i (fetched with ds_bpermute)
+    const int tab_b = __float_as_int(kBoundaries[(lane & 15) < 15 ? (lane & 15) : 14]);
+    const int tab_c = __float_as_int(kCentroids[lane & 15]);
+    sign_wht256(v, lane);
 
-    float s_sq0 = 0.0f, s_sq1 = 0.0f;
+    float p[8];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        s_sq0 += half_wave_sum(v[j] * v[j], lane);
-        s_sq1 += half_wave_sum(v[j + 4] * v[j + 4], lane);
-    }
-    const float rs0 = (float)(1.0 / sqrt((double)s_sq0));
-    const float rs1 = (float)(1.0 / sqrt((double)s_sq1));
-    const float inv_norm0 = (s_sq0 > 1e-20f) ? (0.7071067811865475f * rs0) : 0.0f;
-    const float inv_norm1 = (s_sq1 > 1e-20f) ? (0.7071067811865475f * rs1) : 0.0f;
+    for (int j = 0; j < 8; ++j) p[j] = v[j] * v[j];
+    const float s_sq = row_sum_of_groups(group32_sums(p, lane), lane);
+    const float rs = (float)(1.0 / sqrt((double)s_sq));
+    const float inv_norm = (s_sq > 1e-20f) ? (0.7071067811865475f * rs) : 0.0f;
 
-    float vc_dot0 = 0.0f, c_sq0 = 0.0f, vc_dot1 = 0.0f, c_sq1 = 0.0f;
+    // code = number of boundaries below the value (op_kv_cache.cu:186-189), found by binary
+    // search over the sorted boundaries: same count, thresholds fetched by index
+    int q[8];
+    float c[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-        const float raw_v = v[j];
-        const float rv = raw_v * ((j < 4) ? inv_norm0 : inv_norm1);
-        int q = 0;
+        const float rv = v[j] * inv_norm;
+        int code = (rv > kBoundaries[7]) ? 1 : 0;
 #pragma unroll
-        for (int i = 0; i < 15; ++i) q += (rv > kBoundaries[i]) ? 1 : 0;
-        // byte m of a 64-byte block holds elements 2m (low nibble) and 2m+1 (high nibble);
-        // elements l32 and l32^1 of register j are neighbours.
-        const int partner = lane_xor1_int(q, lane);
-        if ((l32 & 1) == 0) {
-            row[66 * (j >> 2) + 2 + (((j & 3) * 32 + l32) >> 1)] = (uint8_t)(q | (partner << 4));
+        for (int lvl = 1; lvl < 4; ++lvl) {
+            // the bits so far are the top bits of the code; the next threshold is the middle of what is left
+            const int idx = (code << (4 - lvl)) + (1 << (3 - lvl)) - 1;
+            const float t = __int_as_float(__builtin_amdgcn_ds_bpermute(idx << 2, tab_b));
+            code = 2 * code + ((rv > t) ? 1 : 0);
         }
-        const float c = kCentroids[q];
-        const float vc = half_wave_sum(raw_v * c, lane);
-        const float cc = half_wave_sum(c * c, lane);
-        if (j < 4) {
-            vc_dot0 += vc;
-            c_sq0 += cc;
-        } else {
-            vc_dot1 += vc;
-            c_sq1 += cc;
-        }
+        q[j] = code;
+        c[j] = __int_as_float(__builtin_amdgcn_ds_bpermute(code << 2, tab_c));
     }
-    if (l32 == 0) {
-        const float d0 = (c_sq0 > 1e-10f) ? (vc_dot0 / c_sq0) : 0.0f;
-        const float d1 = (c_sq1 > 1e-10f) ? (vc_dot1 / c_sq1) : 0.0f;
-        *reinterpret_cast<uint16_t*>(row) = F16::from_f32(d0);
-        *reinterpret_cast<uint16_t*>(row + 66) = F16::from_f32(d1);
+    // byte m of a 64-byte block holds elements 2m (low nibble) and 2m + 1 (high nibble):
+    // elements 8 l32 .. + 7 are bytes 4 (l32 % 16) .. + 3 of block l32 / 16
+    uint32_t word = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) word |= (uint32_t)(q[2 * k] | (q[2 * k + 1] << 4)) << (8 * k);
+    uint8_t* wdst = row + 66 * (l32 >> 4) + 2 + 4 * (l32 & 15);
+    *reinterpret_cast<uint16_t*>(wdst) = (uint16_t)word;
+    *reinterpret_cast<uint16_t*>(wdst + 2) = (uint16_t)(word >> 16);
+
+    float pv[8], pc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        pv[j] = v[j] * c[j];
+        pc[j] = c[j] * c[j];
+    }
+    const float vc_dot = row_sum_of_groups(group32_sums(pv, lane), lane);
+    const float c_sq = row_sum_of_groups(group32_sums(pc, lane), lane);
+    if ((l32 & 15) == 0) {
+        const float d = (c_sq > 1e-10f) ? (vc_dot / c_sq) : 0.0f;
+        *reinterpret_cast<uint16_t*>(row + 66 * (l32 >> 4)) = F16::from_f32(d);
     }
 }
 
@@ -187,80 +237,33 @@ __device__ __forceinline__ void q8_encode_row(const float (&v)[8], int lane, uin
     if ((l32 & 7) == 0) *reinterpret_cast<float*>(blk) = d;
 }
 
-// The same two rows from the rotated layout v[j] = y[l32 + 32 j] (y = WHT256(sign * x)), used when
-// an 8-bit layer asks for the WHT256 transform (op_kv_cache.cu:36-44,71-99).
-__device__ __forceinline__ float half_wave_max(float v, int lane) {
-    v = fmaxf(v, lane_xor<16>(v, lane));
-    v = fmaxf(v, lane_xor<8>(v, lane));
-    v = fmaxf(v, lane_xor<4>(v, lane));
-    v = fmaxf(v, lane_xor<2>(v, lane));
-    v = fmaxf(v, lane_xor<1>(v, lane));
-    return v;
-}
-
-__device__ __forceinline__ void fp8_encode_row_rotated(const float (&v)[8], int lane, uint8_t* row) {
-    const int l32 = lane & 31;
-#pragma unroll
-    for (int b = 0; b < 2; ++b) {
-        float amax = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) amax = fmaxf(amax, fabsf(v[4 * b + j]));
-        amax = half_wave_max(amax, lane);
-        const float d = amax * (1.0f / 448.0f);
-        const float inv_d = (d > 1e-30f) ? (1.0f / d) : 0.0f;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            row[l32 + 32 * (4 * b + j)] = (uint8_t)f32_to_e4m3(v[4 * b + j] * inv_d);
-        }
-        if (l32 == 0) *reinterpret_cast<float*>(row + 256 + 4 * b) = d;
-    }
-}
-
-__device__ __forceinline__ void q8_encode_row_rotated(const float (&v)[8], int lane, uint8_t* row) {
-    const int l32 = lane & 31;
-#pragma unroll
-    for (int sb = 0; sb < 4; ++sb) {
-        const float x0 = v[2 * sb], x1 = v[2 * sb + 1];
-        const float amax = half_wave_max(fmaxf(fabsf(x0), fabsf(x1)), lane);
-        const float d = amax / 127.0f;
-        const float inv_d = (d > 1e-12f) ? (1.0f / d) : 0.0f;
-        const float q0 = fminf(127.0f, fmaxf(-127.0f, roundf(x0 * inv_d)));
-        const float q1 = fminf(127.0f, fmaxf(-127.0f, roundf(x1 * inv_d)));
-        uint8_t* blk = row + 68 * sb;
-        blk[4 + l32] = (uint8_t)(int)q0;
-        blk[4 + 32 + l32] = (uint8_t)(int)q1;
-        if (l32 == 0) *reinterpret_cast<float*>(blk) = d;
-    }
-}
-
-// Encodes one 256-wide row held as v[j] = x[l32 + 32 j] (not yet transformed) in `format` /
+// Encodes one 256-wide row held as v[j] = x[8 l32 + j] (not yet transformed) in `format` /
 // `transform`, assembles it in the half-wave's LDS area `row` (272 bytes, 8-byte aligned) and
-// stores it at dst (nothing is stored for dst == nullptr).  16-bit formats are stored directly.  The caller guarantees what the append
-// entry points check: head_dim 256, TQ4 with WHT256, 8-bit rows 4-byte aligned.
+// stores it at dst (nothing is stored for dst == nullptr).  16-bit formats are stored directly.
+// Rotated 8-bit rows are the un-rotated encoders applied to the transformed row
+// (op_kv_cache.cu:36-44,71-99: the same scale and code arithmetic; max is order-free).  The
+// caller guarantees what the append entry points check: head_dim 256, TQ4 with WHT256, 8-bit
+// rows 4-byte aligned.
 __device__ __forceinline__ void encode_store_row(float (&v)[8], int format, int transform, int lane,
                                                  uint8_t* row, uint8_t* dst) {
     const int l32 = lane & 31;
     if (format == WARP34_KV_FORMAT_FP16 || format == WARP34_KV_FORMAT_BF16) {
-        uint16_t* d16 = reinterpret_cast<uint16_t*>(dst);
+        if (dst == nullptr) return;
+        uint16_t* d16 = reinterpret_cast<uint16_t*>(dst) + 8 * l32;
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-            d16[l32 + 32 * j] = (format == WARP34_KV_FORMAT_BF16) ? BF16::from_f32(v[j]) : F16::from_f32(v[j]);
+        for (int j = 0; j < 8; ++j) d16[j] = (format == WARP34_KV_FORMAT_BF16) ? BF16::from_f32(v[j]) : F16::from_f32(v[j]);
         return;
     }
     int n_dwords = 33;
     if (format == WARP34_KV_FORMAT_TQ4) {
         tq4_encode_row(v, lane, row);
     } else {
-        if (transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] = apply_sign(v[j], l32 + 32 * j);
-            wht256_half_wave(v, lane);
-        }
+        if (transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256) sign_wht256(v, lane);
         if (format == WARP34_KV_FORMAT_FP8_E4M3) {
-            fp8_encode_row_rotated(v, lane, row);
+            fp8_encode_row(v, lane, row);
             n_dwords = 66;
         } else {
-            q8_encode_row_rotated(v, lane, row);
+            q8_encode_row(v, lane, row);
             n_dwords = 68;
         }
     }
@@ -277,6 +280,22 @@ __device__ __forceinline__ void encode_store_row(float (&v)[8], int format, int 
         uint16_t* d16 = reinterpret_cast<uint16_t*>(dst);
         for (int i = l32; i < 2 * n_dwords; i += 32) d16[i] = r16[i];
     }
+}
+
+// v[j] = x[l32 + 32 j] (one element per lane and register, as a kernel holds a row whose pairs
+// (i, i + 128) it has just rotated) -> v[j] = x[8 l32 + j], through 1 KB of LDS private to the
+// half-wave.  Whole-wave call.
+__device__ __forceinline__ void strided_to_consecutive(float (&v)[8], int lane, float* xpose) {
+    const int l32 = lane & 31;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) xpose[l32 + 32 * j] = v[j];
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    __builtin_amdgcn_wave_barrier();
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    const float4 a = *reinterpret_cast<const float4*>(xpose + 8 * l32);
+    const float4 b = *reinterpret_cast<const float4*>(xpose + 8 * l32 + 4);
+    v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w;
+    v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
 }
 
 // ---- host-side checks shared by the entry points that write rows ----

@@ -60,16 +60,6 @@ __global__ __launch_bounds__(256) void kv_append_kernel(warp34_kv_layer_layout L
         uint8_t* row = rows[wave][is_v];
         const int n_dwords = format == WARP34_KV_FORMAT_FP8_E4M3 ? 66 : 68;
         const uint16_t* src8 = src + 8 * l32;
-        if ((is_v ? L.v_transform : L.k_transform) == WARP34_KV_TRANSFORM_RADEMACHER_WHT256) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] = apply_sign(TIn::to_f32(src[l32 + 32 * j]), l32 + 32 * j);
-            wht256_half_wave(v, lane);
-            if (format == WARP34_KV_FORMAT_FP8_E4M3) {
-                fp8_encode_row_rotated(v, lane, row);
-            } else {
-                q8_encode_row_rotated(v, lane, row);
-            }
-        } else {
         if ((reinterpret_cast<uintptr_t>(src8) & 15u) == 0) {
             const uint4 raw = *reinterpret_cast<const uint4*>(src8);
             const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
@@ -82,11 +72,12 @@ __global__ __launch_bounds__(256) void kv_append_kernel(warp34_kv_layer_layout L
 #pragma unroll
             for (int j = 0; j < 8; ++j) v[j] = TIn::to_f32(src8[j]);
         }
+        // rotated rows: the same encoders over the transformed row
+        if ((is_v ? L.v_transform : L.k_transform) == WARP34_KV_TRANSFORM_RADEMACHER_WHT256) sign_wht256(v, lane);
         if (format == WARP34_KV_FORMAT_FP8_E4M3) {
             fp8_encode_row(v, lane, row);
         } else {
             q8_encode_row(v, lane, row);
-        }
         }
         __atomic_signal_fence(__ATOMIC_SEQ_CST);
         __builtin_amdgcn_wave_barrier();
@@ -100,9 +91,21 @@ __global__ __launch_bounds__(256) void kv_append_kernel(warp34_kv_layer_layout L
     }
     if (format == WARP34_KV_FORMAT_TQ4) {
         // host side guarantees head_dim == 256 and the WHT256 transform for TQ4
+        // lane l32 takes elements 8 l32 .. 8 l32 + 7: one 16-byte load where the source allows it
         float v[8];
+        const uint16_t* src8 = src + 8 * l32;
+        if ((reinterpret_cast<uintptr_t>(src8) & 15u) == 0) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(src8);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = TIn::to_f32(src[l32 + 32 * j]);
+            for (int j = 0; j < 4; ++j) {
+                v[2 * j] = TIn::to_f32((uint16_t)(w[j] & 0xffffu));
+                v[2 * j + 1] = TIn::to_f32((uint16_t)(w[j] >> 16));
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = TIn::to_f32(src8[j]);
+        }
         // the row is assembled in LDS and leaves with one 32-bit store per lane (16-bit stores
         // when the destination is only 2-byte aligned, which is all the row format promises)
         uint8_t* row = rows[wave][is_v];

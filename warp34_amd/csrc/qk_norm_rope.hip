@@ -37,6 +37,7 @@ struct NormRopeParams {
 template <bool TABLE_F32, bool D256>
 __global__ __launch_bounds__(256) void qk_norm_rope_kernel(const NormRopeParams P) {
     __shared__ __align__(8) uint8_t rows_lds[4][2][272];
+    __shared__ __align__(16) float xpose_lds[4][2][256];  // register layout of the rotation -> the encoder's
     const int wave = (int)(threadIdx.x >> 6);
     const int lane = lane_id();
     const int half_id = lane >> 5;
@@ -151,6 +152,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(const NormRopeParams 
             float v[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) v[j] = is_v_half ? raw[j] : (j < 4 ? lo[j & 3] : hi[j & 3]);
+            strided_to_consecutive(v, lane, xpose_lds[wave][half_id]);
             encode_store_row(v, format, transform, lane, row_lds, dst);
         }
         return;
