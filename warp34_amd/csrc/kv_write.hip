@@ -17,18 +17,20 @@
 
 namespace w34 {
 
-// One wave per (token, kv head); lanes 0-31 write K, lanes 32-63 write V.
+// One wave per (token, kv head): blockIdx.x counts groups of four tokens, blockIdx.y the kv heads;
+// lanes 0-31 write K, lanes 32-63 write V.  Everything up to the row addresses is the same for
+// the whole wave and is kept in scalar registers (block_magic = floor(2^32 / block_size): the
+// page of a slot without a division).
 template <typename TIn>
 __global__ __launch_bounds__(256) void kv_append_kernel(warp34_kv_layer_layout L,
                                                         warp34_attention_batch B,
                                                         const uint16_t* __restrict__ k_in,
                                                         const uint16_t* __restrict__ v_in,
                                                         int k_row_stride, int v_row_stride,
-                                                        int check_req_mask) {
-    const int wave = (int)(threadIdx.x >> 6);
-    const int item = (int)blockIdx.x * 4 + wave;
-    const int tok = item / L.local_kv_heads;
-    const int head = item - tok * L.local_kv_heads;
+                                                        int check_req_mask, uint32_t block_magic) {
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int tok = (int)blockIdx.x * 4 + wave;
+    const int head = (int)blockIdx.y;
     if (tok >= B.total_tokens) return;
     if (B.valid_token_mask != nullptr && B.valid_token_mask[tok] == 0) return;
     if (check_req_mask) {
@@ -38,20 +40,22 @@ __global__ __launch_bounds__(256) void kv_append_kernel(warp34_kv_layer_layout L
     }
     const int32_t slot = B.write_slot_mapping[tok];
     if (slot < 0) return;
-    const int page = slot / L.block_size;
+    int page = (int)__umulhi((uint32_t)slot, block_magic);  // the quotient or one less
+    page += (slot - page * L.block_size >= L.block_size) ? 1 : 0;
     const int off = slot - page * L.block_size;
 
     const int lane = lane_id();
     const int is_v = lane >> 5;
     const int l32 = lane & 31;
     const int format = is_v ? L.v_format : L.k_format;
-    uint8_t* dst = reinterpret_cast<uint8_t*>((uintptr_t)(is_v ? L.v_base : L.k_base)) +
-                   (size_t)page * (is_v ? L.v_page_stride_bytes : L.k_page_stride_bytes) +
-                   (size_t)head * (is_v ? L.v_head_stride_bytes : L.k_head_stride_bytes) +
-                   (size_t)off * (is_v ? L.v_token_stride_bytes : L.k_token_stride_bytes);
-    const uint16_t* src = (is_v ? v_in : k_in) +
-                          (size_t)tok * (size_t)(is_v ? v_row_stride : k_row_stride) +
-                          (size_t)head * (size_t)L.head_dim;
+    const uint64_t k_dst = L.k_base + (uint64_t)page * L.k_page_stride_bytes + (uint64_t)head * L.k_head_stride_bytes +
+                           (uint64_t)off * L.k_token_stride_bytes;
+    const uint64_t v_dst = L.v_base + (uint64_t)page * L.v_page_stride_bytes + (uint64_t)head * L.v_head_stride_bytes +
+                           (uint64_t)off * L.v_token_stride_bytes;
+    const uint16_t* k_src = k_in + (size_t)tok * (size_t)k_row_stride + (size_t)head * (size_t)L.head_dim;
+    const uint16_t* v_src = v_in + (size_t)tok * (size_t)v_row_stride + (size_t)head * (size_t)L.head_dim;
+    uint8_t* dst = reinterpret_cast<uint8_t*>((uintptr_t)(is_v ? v_dst : k_dst));
+    const uint16_t* src = is_v ? v_src : k_src;
 
     __shared__ __align__(8) uint8_t rows[4][2][272];
     if (format == WARP34_KV_FORMAT_FP8_E4M3 || format == WARP34_KV_FORMAT_Q8_0) {
@@ -142,19 +146,22 @@ __global__ __launch_bounds__(256) void kv_append_kernel(warp34_kv_layer_layout L
     }
 }
 
+static inline uint32_t append_block_magic(int block_size) {
+    return block_size <= 1 ? 0xFFFFFFFFu : (uint32_t)((1ull << 32) / (uint32_t)block_size);
+}
+
 template <typename TIn>
 static int launch_append(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
                          const warp34_attention_batch* batch, const void* k_in, const void* v_in,
                          int k_row_stride, int v_row_stride) {
-    const long long items = (long long)batch->total_tokens * layout->local_kv_heads;
-    const unsigned grid = (unsigned)((items + 3) / 4);
+    const dim3 grid((unsigned)((batch->total_tokens + 3) / 4), (unsigned)layout->local_kv_heads);
     const int check_req = (batch->valid_req_mask != nullptr && batch->query_start_loc != nullptr &&
                            batch->num_reqs > 0)
                               ? 1
                               : 0;
-    hipLaunchKernelGGL((kv_append_kernel<TIn>), dim3(grid), dim3(256), 0, (hipStream_t)ex->stream,
+    hipLaunchKernelGGL((kv_append_kernel<TIn>), grid, dim3(256), 0, (hipStream_t)ex->stream,
                        *layout, *batch, (const uint16_t*)k_in, (const uint16_t*)v_in, k_row_stride,
-                       v_row_stride, check_req);
+                       v_row_stride, check_req, append_block_magic(layout->block_size));
     return (int)hipGetLastError();
 }
 
@@ -231,11 +238,10 @@ extern "C" int warp34_kv_cache_write_strided_bf16(const warp34_exec* ex,
     }
     if (!batch->total_tokens) return 0;
     // the reference's bf16 writer always resolves the owning request (op_kv_cache.cu:803-807)
-    const long long items = (long long)batch->total_tokens * layout->local_kv_heads;
-    const unsigned grid = (unsigned)((items + 3) / 4);
-    hipLaunchKernelGGL((kv_append_kernel<BF16>), dim3(grid), dim3(256), 0, (hipStream_t)ex->stream,
+    const dim3 grid((unsigned)((batch->total_tokens + 3) / 4), (unsigned)layout->local_kv_heads);
+    hipLaunchKernelGGL((kv_append_kernel<BF16>), grid, dim3(256), 0, (hipStream_t)ex->stream,
                        *layout, *batch, (const uint16_t*)k, (const uint16_t*)v, row_stride_elems,
-                       row_stride_elems, 1);
+                       row_stride_elems, 1, append_block_magic(layout->block_size));
     return (int)hipGetLastError();
 }
 
