@@ -113,6 +113,15 @@ def test_tq4_strided_source_bf16():
     assert gk.tobytes() == hpool.k.tobytes() and gv.tobytes() == hpool.v.tobytes()
 
 
+@pytest.mark.parametrize("in_dtype", [DT_BF16, DT_F16])
+@pytest.mark.parametrize("pad", [2, 4, 6])
+def test_tq4_source_rows_not_16_byte_aligned(in_dtype, pad):
+    """A source row stride of 2 * 256 + pad elements: every second row (or more) starts off the
+    16-byte boundary the vector load wants, so those rows take the element-wise loads."""
+    hpool, gk, gv = _run_append(FMT_TQ4, XF_WHT256, 32, 77, in_dtype, seed=21 + pad, stride=2 * 256 + pad)
+    assert gk.tobytes() == hpool.k.tobytes() and gv.tobytes() == hpool.v.tobytes()
+
+
 @pytest.mark.parametrize("fmt", [FMT_FP8, FMT_Q8_0])
 @pytest.mark.parametrize("xf", [XF_IDENTITY, XF_WHT256])
 @pytest.mark.parametrize("in_dtype", [DT_BF16, DT_F16])
