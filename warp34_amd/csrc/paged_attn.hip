@@ -234,7 +234,12 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
 __device__ __forceinline__ void split_h2(float a, float b, uint32_t& hi, uint32_t& lo) {
     const h2 h = __builtin_convertvector(f2{a, b}, h2);
     hi = __builtin_bit_cast(uint32_t, h);
-    lo = pack_h2(a - (float)h[0], b - (float)h[1]);
+    // lo = fp16(a - hi.x) | fp16(b - hi.y) << 16: one mixed-precision FMA per half (x * 1 - h with
+    // h read as fp16), the same value as widening, subtracting (exact) and rounding
+    uint32_t l;
+    asm("v_fma_mixlo_f16 %0, %1, 1.0, -%2 op_sel:[0,0,0] op_sel_hi:[0,0,1]" : "=v"(l) : "v"(a), "v"(hi));
+    asm("v_fma_mixhi_f16 %0, %1, 1.0, -%2 op_sel:[0,0,1] op_sel_hi:[0,0,1]" : "+v"(l) : "v"(b), "v"(hi));
+    lo = l;
 }
 __device__ __forceinline__ float half_lo_to_f32(uint32_t w) {
     return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xFFFFu));
