@@ -787,9 +787,14 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         // (it + 1) & 1, the MFMAs read buffer it & 1.  (With the cheaper dequantisers of the other
         // formats the same order in all waves measured faster.)
         const bool compute_first = TQ4F && wave >= 4;  // wave-uniform
+        // (TQ4: while a wave multiplies it is the one the SIMD serves first, so its MFMAs go out as
+        // soon as their operands are there and the other wave's dequantiser fills the gaps: -4 %.
+        // The other formats, whose waves all run the same order, measured 5 % slower with it.)
         if (compute_first && it >= 0) {
             const int t0 = (u_first + it) * kUnit;
+            __builtin_amdgcn_s_setprio(1);
             compute_unit(it & 1, t0, !(t0 >= i_lo && t0 + kUnit - 1 <= i_hi));
+            __builtin_amdgcn_s_setprio(0);
         }
         if (it + 1 >= 0 && it + 1 < n_units) {
             if constexpr (K16) {
@@ -804,7 +809,9 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         }
         if (!compute_first && it >= 0) {
             const int t0 = (u_first + it) * kUnit;
+            if constexpr (TQ4F) __builtin_amdgcn_s_setprio(1);
             compute_unit(it & 1, t0, !(t0 >= i_lo && t0 + kUnit - 1 <= i_hi));
+            if constexpr (TQ4F) __builtin_amdgcn_s_setprio(0);
         }
         __syncthreads();
     }
