@@ -1863,11 +1863,19 @@ static int launch_prefill_tq4(const warp34_exec* ex, const warp34_kv_layer_layou
             return (int)hipGetLastError();
         }
     }
-    rc = ensure_dynamic_lds(paged_prefill_tq4_kernel<TQ, KVF, false>, PfLds<KVF>::kSmem, true);
-    if (rc) return rc;
-    hipLaunchKernelGGL((paged_prefill_tq4_kernel<TQ, KVF, false>), grid, dim3(kPfWaves * 64), PfLds<KVF>::kSmem,
-                       (hipStream_t)ex->stream, P);
-    return (int)hipGetLastError();
+    if constexpr (KVF == WARP34_KV_FORMAT_TQ4) {  // twelve waves: eight multiply, four dequantise
+        rc = ensure_dynamic_lds(paged_prefill_tq4_kernel<TQ, KVF, false, true>, PfLds<KVF>::kSmem, true);
+        if (rc) return rc;
+        hipLaunchKernelGGL((paged_prefill_tq4_kernel<TQ, KVF, false, true>), grid, dim3(12 * 64), PfLds<KVF>::kSmem,
+                           (hipStream_t)ex->stream, P);
+        return (int)hipGetLastError();
+    } else {
+        rc = ensure_dynamic_lds(paged_prefill_tq4_kernel<TQ, KVF, false>, PfLds<KVF>::kSmem, true);
+        if (rc) return rc;
+        hipLaunchKernelGGL((paged_prefill_tq4_kernel<TQ, KVF, false>), grid, dim3(kPfWaves * 64), PfLds<KVF>::kSmem,
+                           (hipStream_t)ex->stream, P);
+        return (int)hipGetLastError();
+    }
 }
 
 static bool is_kv16(const warp34_kv_layer_layout* l, int format) {

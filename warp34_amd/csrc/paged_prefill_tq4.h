@@ -68,13 +68,18 @@ __device__ __forceinline__ f4 pf_mfma32(h8 a, h8 b, f4 c) {
 // fp16(d * code) rounds partly alike across a scale block that holds few distinct codes, and the
 // inverse rotation of the finished row would gather that common part into a single channel.
 // (Q8_0 key tiles hold the codes in either form, see dequant_unit_q8.)
-template <typename TQ, int KVF, bool VF = false>
-__global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(const AttnParams P) {
+// PC (TQ4 pages): twelve waves.  Waves 0-7 only multiply (16 columns each, as in the eight-wave
+// form); waves 8-11 load and dequantise the next unit, a whole 16-row run each.  Every SIMD then
+// holds two multiplying waves and one dequantising wave whose instruction streams never wait
+// for each other's results inside an iteration.
+template <typename TQ, int KVF, bool VF = false, bool PC = false>
+__global__ __launch_bounds__((PC ? 12 : kPfWaves) * 64, 1) void paged_prefill_tq4_kernel(const AttnParams P) {
     using M = PfLds<KVF>;
     constexpr bool FP8 = M::kFp8;
     constexpr bool K16 = M::k16;  // 16-bit rows, read as stored: the MFMAs run in the storage type
     constexpr bool Q8 = M::kQ8;   // Q8_0 rows: the key tile holds the codes, the value tile fp16(d * code) unless VF
     static_assert(!VF || FP8 || Q8, "scales in the probabilities: 8-bit rows only");
+    static_assert(!PC || (!M::kFp8 && !M::k16 && !M::kQ8), "separate dequantising waves: TQ4 pages only");
     // VF: the tile holds code / kVfGain (a power of two: exact) and the weights p * d * kVfGain.  The
     // block scales of 8-bit rows are small (amax / 448, amax / 127): without the gain the low-order
     // weight operand, 2^-12 of the weight, would fall into fp16's subnormal range and lose its bits.
@@ -93,6 +98,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15;
     const int b = lane >> 4;
+    const bool producer = PC && wave >= kPfWaves;  // wave-uniform
     const warp34_kv_layer_layout& L = P.L;
     const warp34_attention_batch& B = P.B;
 
@@ -115,7 +121,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     if (tile_tokens > B.total_tokens - tok0) tile_tokens = B.total_tokens - tok0;
 
     // ---- the pair table (64 lane replicas, as in the decode kernel) ----
-    if constexpr (TQ4F) {
+    if (TQ4F && tid < kPfWaves * 64) {
         const int e = tid >> 1;
         const uint32_t v = pack_h2(kLutGain * centroid_of_code(e & 15), kLutGain * centroid_of_code(e >> 4));
         u4 vv = {v, v, v, v};
@@ -161,7 +167,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     const float q_scale = B.sm_scale * kLog2e * (TQ4F ? kLutInvGain : 1.0f);
     const bool rot_q = !K16 && (TQ4F || P.rot_q != 0);
     const bool rot_out = !K16 && (TQ4F || P.rot_out != 0);
-    {
+    if (!producer) {
         uint2 q_raw[16];
 #pragma unroll
         for (int c = 0; c < 16; ++c) {
@@ -209,7 +215,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     for (int h = 0; h < 2; ++h)
 #pragma unroll
         for (int m = 0; m < 4; ++m)
-            bq[h][m] = *reinterpret_cast<const h8*>(qbuf + n * kQStride + 128 * h + 32 * m + 8 * b);
+            bq[h][m] = producer ? h8{} : *reinterpret_cast<const h8*>(qbuf + n * kQStride + 128 * h + 32 * m + 8 * b);
 
     // ---- loader ----
     // A unit is four runs of 16 rows: K rows 0-15, K rows 16-31, V rows 0-15, V rows 16-31.
@@ -222,21 +228,21 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
     const uint8_t* v_base = reinterpret_cast<const uint8_t*>((uintptr_t)L.v_base) +
                             (size_t)kv_head * L.v_head_stride_bytes;
     const int32_t* req_blocks = B.block_tables + (size_t)req * B.max_blocks_per_req;
-    const int ld_run = wave >> 1;
+    const int ld_run = PC ? (wave - kPfWaves) & 3 : wave >> 1;  // PC: one run per dequantising wave
     const bool ld_is_v = ld_run >= 2;
     // Q8_0: a run is 4352 B = 272 pieces; each wave of the pair loads 136 (two per lane and an eight-lane tail)
-    const bool ld_tail = !K16 && (FP8 || Q8 || (wave & 1) == 0);  // wave-uniform
+    const bool ld_tail = !K16 && (PC || FP8 || Q8 || (wave & 1) == 0);  // wave-uniform
     constexpr int kTailLanes = Q8 ? 8 : 4;
     const uint8_t* ld_base = ld_is_v ? v_base : k_base;
     const uint64_t ld_page_stride = ld_is_v ? L.v_page_stride_bytes : L.k_page_stride_bytes;
     const uint64_t ld_tok_stride = ld_is_v ? L.v_token_stride_bytes : L.k_token_stride_bytes;
     // 16-bit rows: a run is 8192 B = 512 pieces; each wave of the pair loads 256 (four per lane), no tail
-    const uint32_t ld_lane_off = (uint32_t)((wave & 1) * (K16 ? 4096 : FP8 ? 2112 : Q8 ? 2176 : 1024) + 16 * lane);
+    const uint32_t ld_lane_off = (uint32_t)((PC ? 0 : (wave & 1) * (K16 ? 4096 : FP8 ? 2112 : Q8 ? 2176 : 1024)) + 16 * lane);
     const uint32_t ld_tail_off = (uint32_t)((FP8 ? (wave & 1) * 2112 : Q8 ? (wave & 1) * 2176 : 0) + 2048 +
                                             16 * (lane & (kTailLanes - 1)));
     const uint32_t ld_commit0 = (uint32_t)(ld_run * kRunB) + ld_lane_off;
     const uint32_t ld_commit1 = (uint32_t)(ld_run * kRunB) + ld_tail_off;
-    u4 pf[K16 ? 4 : (FP8 || Q8) ? 3 : 2];
+    u4 pf[K16 ? 4 : (FP8 || Q8 || PC) ? 3 : 2];
     // page id of unit k (relative to u_first) for this wave's run; -1 = nothing to fetch.
     // Only groups that overlap the visible key range are fetched: block-table entries beyond
     // the request's pages are unspecified.
@@ -261,7 +267,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             for (int i = 1; i < 4; ++i) pf[i] = *(global_cu4*)(src + ld_lane_off + 1024 * i);
         } else {
             if (ld_tail) pf[1] = *(global_cu4*)(src + ld_tail_off);
-            if constexpr (FP8 || Q8) pf[2] = *(global_cu4*)(src + ld_lane_off + 1024);
+            if constexpr (FP8 || Q8 || PC) pf[2] = *(global_cu4*)(src + ld_lane_off + 1024);
         }
     };
     auto commit_loads = [&](int buf) {
@@ -272,7 +278,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             for (int i = 1; i < 4; ++i) *reinterpret_cast<u4*>(raw + ld_commit0 + 1024 * i) = pf[i];
         } else {
             if (ld_tail && lane < kTailLanes) *reinterpret_cast<u4*>(raw + ld_commit1) = pf[1];
-            if constexpr (FP8 || Q8) *reinterpret_cast<u4*>(raw + ld_commit0 + 1024) = pf[2];
+            if constexpr (FP8 || Q8 || PC) *reinterpret_cast<u4*>(raw + ld_commit0 + 1024) = pf[2];
         }
     };
 
@@ -303,10 +309,14 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
             shift = 0;
         }
     };
-    uint32_t k_src[2][2], k_shift[2], k_dst[2][2];
+    // (PC: 256 dequantising threads take twice the items)
+    constexpr int kDqThreads = PC ? 256 : 512;
+    constexpr int kKItems = 1024 / kDqThreads, kVItems = 512 / kDqThreads;
+    const int dq_tid = PC ? (tid - kPfWaves * 64) & 255 : tid;
+    uint32_t k_src[kKItems][2], k_shift[kKItems], k_dst[kKItems][2];
 #pragma unroll
-    for (int it = 0; it < 2; ++it) {
-        const int idx = tid + 512 * it;
+    for (int it = 0; it < kKItems; ++it) {
+        const int idx = dq_tid + kDqThreads * it;
         const int r = idx >> 5, j = idx & 31;
         uint32_t src[2];
         item_src(j, src, k_shift[it]);
@@ -318,18 +328,19 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         k_dst[it][1] = (uint32_t)(r * kPfKStride + 2 * d_hi);
     }
     const int nibsel = (lane >> 4) & 1;
-    uint32_t v_src[2], v_shift, v_dst[4];
-    {
-        const int p = tid & 15, j = tid >> 4;
+    uint32_t v_src[kVItems][2], v_shift[kVItems], v_dst[kVItems][4];
+#pragma unroll
+    for (int vi = 0; vi < kVItems; ++vi) {
+        const int p = dq_tid & 15, j = (dq_tid >> 4) + (kDqThreads / 16) * vi;  // (j keeps the parity of lane >> 4)
         uint32_t src[2];
-        item_src(j, src, v_shift);
-        v_src[0] = (uint32_t)(kPfRawBytes / 2 + (2 * p) * kTq4RowBytes) + src[0];
-        v_src[1] = (uint32_t)(kPfRawBytes / 2 + (2 * p) * kTq4RowBytes) + src[1];
+        item_src(j, src, v_shift[vi]);
+        v_src[vi][0] = (uint32_t)(kPfRawBytes / 2 + (2 * p) * kTq4RowBytes) + src[0];
+        v_src[vi][1] = (uint32_t)(kPfRawBytes / 2 + (2 * p) * kTq4RowBytes) + src[1];
         const int bp = (p >> 1) & 3, s = p >> 3;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const int d = j == 0 ? (q < 2 ? 2 * q : 120 + 2 * q) : (j < 16 ? 8 * j - 4 : 8 * j) + 2 * q;
-            v_dst[q] = (uint32_t)(kPfKBytes + d * 64 + 16 * (bp ^ ((d >> 1) & 3)) + 8 * s + 4 * (p & 1) + 64 * nibsel);
+            v_dst[vi][q] = (uint32_t)(kPfKBytes + d * 64 + 16 * (bp ^ ((d >> 1) & 3)) + 8 * s + 4 * (p & 1) + 64 * nibsel);
         }
     }
     // ---- per-wave attention state ----
@@ -347,61 +358,70 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
         const uint32_t raw = (uint32_t)(kPfRawBase + rawbuf * kPfRawBytes);
         const uint32_t deq = (uint32_t)(kPfDeqBase + deqbuf * kPfDeqBytes);
         // ---- phase 1: raw dwords ----
-        uint32_t kw0[2], kw1[2];
+        uint32_t kw0[kKItems], kw1[kKItems];
 #pragma unroll
-        for (int it = 0; it < 2; ++it) {
+        for (int it = 0; it < kKItems; ++it) {
             kw0[it] = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + k_src[it][0]));
             kw1[it] = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + k_src[it][1]));
         }
-        const uint32_t a0 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[0]));
-        const uint32_t a1 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[1]));
-        const uint32_t b0 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[0] + kTq4RowBytes));
-        const uint32_t b1 = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[1] + kTq4RowBytes));
-        // scales: thread x * 32 + r (x = 0: K d0, 1: K d1, 2: V d0, 3: V d1) of waves 0 and 1
+        uint32_t a0[kVItems], a1[kVItems], b0[kVItems], b1[kVItems];
+#pragma unroll
+        for (int vi = 0; vi < kVItems; ++vi) {
+            a0[vi] = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[vi][0]));
+            a1[vi] = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[vi][1]));
+            b0[vi] = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[vi][0] + kTq4RowBytes));
+            b1[vi] = *reinterpret_cast<lds_cu32*>((uintptr_t)(raw + v_src[vi][1] + kTq4RowBytes));
+        }
+        // scales: thread x * 32 + r (x = 0: K d0, 1: K d1, 2: V d0, 3: V d1) of the first two dequantising waves
         uint16_t scale_bits = 0;
-        if (tid < 128) {
-            const int x = tid >> 5, r = tid & 31;
+        if (dq_tid < 128) {
+            const int x = dq_tid >> 5, r = dq_tid & 31;
             scale_bits = *reinterpret_cast<const uint16_t*>(smem + raw + (x >> 1) * (kPfRawBytes / 2) +
                                                             r * kTq4RowBytes + (x & 1) * 66);
         }
         // ---- phase 2: table reads ----
-        uint2 k_lo[2], k_hi[2];
+        uint2 k_lo[kKItems], k_hi[kKItems];
 #pragma unroll
-        for (int it = 0; it < 2; ++it) {
+        for (int it = 0; it < kKItems; ++it) {
             const uint32_t word = __builtin_amdgcn_alignbit(kw1[it], kw0[it], k_shift[it]);
             k_lo[it].x = lut_read(word, lut_lane, 0x0c0c0400u);
             k_lo[it].y = lut_read(word, lut_lane, 0x0c0c0500u);
             k_hi[it].x = lut_read(word, lut_lane, 0x0c0c0600u);
             k_hi[it].y = lut_read(word, lut_lane, 0x0c0c0700u);
         }
-        const uint32_t wa = __builtin_amdgcn_alignbit(a1, a0, v_shift);
-        const uint32_t wb = __builtin_amdgcn_alignbit(b1, b0, v_shift);
-        // byte q of ev / od = (even / odd element of token 2p) | (same of token 2p+1) << 4
-        const uint32_t ev = (wa & 0x0F0F0F0Fu) | ((wb << 4) & 0xF0F0F0F0u);
-        const uint32_t od = ((wa >> 4) & 0x0F0F0F0Fu) | (wb & 0xF0F0F0F0u);
-        const uint32_t first = nibsel ? od : ev;   // elements of parity nibsel, stored at v_dst
-        const uint32_t second = nibsel ? ev : od;  // the other parity, one V^T row (64 B) away
-        uint32_t vx0[4], vx1[4];
+        uint32_t vx0[kVItems][4], vx1[kVItems][4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const uint32_t sel = 0x0c0c0400u + ((uint32_t)q << 8);
-            vx0[q] = lut_read(first, lut_lane, sel);
-            vx1[q] = lut_read(second, lut_lane, sel);
+        for (int vi = 0; vi < kVItems; ++vi) {
+            const uint32_t wa = __builtin_amdgcn_alignbit(a1[vi], a0[vi], v_shift[vi]);
+            const uint32_t wb = __builtin_amdgcn_alignbit(b1[vi], b0[vi], v_shift[vi]);
+            // byte q of ev / od = (even / odd element of token 2p) | (same of token 2p+1) << 4
+            const uint32_t ev = (wa & 0x0F0F0F0Fu) | ((wb << 4) & 0xF0F0F0F0u);
+            const uint32_t od = ((wa >> 4) & 0x0F0F0F0Fu) | (wb & 0xF0F0F0F0u);
+            const uint32_t first = nibsel ? od : ev;   // elements of parity nibsel, stored at v_dst
+            const uint32_t second = nibsel ? ev : od;  // the other parity, one V^T row (64 B) away
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t sel = 0x0c0c0400u + ((uint32_t)q << 8);
+                vx0[vi][q] = lut_read(first, lut_lane, sel);
+                vx1[vi][q] = lut_read(second, lut_lane, sel);
+            }
         }
         // ---- phase 3: writes ----
 #pragma unroll
-        for (int it = 0; it < 2; ++it) {
+        for (int it = 0; it < kKItems; ++it) {
             *reinterpret_cast<uint2*>(smem + deq + k_dst[it][0]) = k_lo[it];
             *reinterpret_cast<uint2*>(smem + deq + k_dst[it][1]) = k_hi[it];
         }
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const uint32_t addr = deq + v_dst[q];
-            *reinterpret_cast<uint32_t*>(smem + addr) = vx0[q];
-            *reinterpret_cast<uint32_t*>(smem + (addr ^ 64u)) = vx1[q];
-        }
-        if (tid < 128) {
-            *reinterpret_cast<float*>(smem + deq + kPfKBytes + kPfVBytes + 4 * tid) =
+        for (int vi = 0; vi < kVItems; ++vi)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t addr = deq + v_dst[vi][q];
+                *reinterpret_cast<uint32_t*>(smem + addr) = vx0[vi][q];
+                *reinterpret_cast<uint32_t*>(smem + (addr ^ 64u)) = vx1[vi][q];
+            }
+        if (dq_tid < 128) {
+            *reinterpret_cast<float*>(smem + deq + kPfKBytes + kPfVBytes + 4 * dq_tid) =
                 (float)__builtin_bit_cast(_Float16, scale_bits);
         }
     };
@@ -770,50 +790,79 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void paged_prefill_tq4_kernel(con
 
     // ---- pipeline ----
     __syncthreads();  // table complete; query staging (aliases the dequant buffers) consumed
-    const int32_t pg_first = __builtin_amdgcn_readfirstlane(load_page(0));
-    int32_t pg_next = load_page(1);
-    if (n_units > 0) issue_loads(0, pg_first);
-    for (int it = -2; it < n_units; ++it) {
-        // commit unit it + 2 (loaded during the previous iteration), then start unit it + 3
-        if (it + 2 < n_units) commit_loads((it + 2) & 1);
-        // The page id of unit it + 4 is requested BEFORE the key loads of unit it + 3: a
-        // write to its register after them would have to wait for all of them to return.
-        const int32_t pg_s = __builtin_amdgcn_readfirstlane(pg_next);
-        pg_next = load_page(it + 4);
-        if (it + 3 < n_units) issue_loads(it + 3, pg_s);
-        // TQ4 pages: the two waves of a SIMD (w and w + 4) take the two halves of an iteration in
-        // opposite order, so that one dequantises (table reads and VALU) while the other
-        // multiplies.  Both orders are valid between two barriers: the dequantiser writes buffer
-        // (it + 1) & 1, the MFMAs read buffer it & 1.  (With the cheaper dequantisers of the other
-        // formats the same order in all waves measured faster.)
-        const bool compute_first = TQ4F && wave >= 4;  // wave-uniform
-        // (TQ4: while a wave multiplies it is the one the SIMD serves first, so its MFMAs go out as
-        // soon as their operands are there and the other wave's dequantiser fills the gaps: -4 %.
-        // The other formats, whose waves all run the same order, measured 5 % slower with it.)
-        if (compute_first && it >= 0) {
-            const int t0 = (u_first + it) * kUnit;
-            __builtin_amdgcn_s_setprio(1);
-            compute_unit(it & 1, t0, !(t0 >= i_lo && t0 + kUnit - 1 <= i_hi));
-            __builtin_amdgcn_s_setprio(0);
-        }
-        if (it + 1 >= 0 && it + 1 < n_units) {
-            if constexpr (K16) {
-                dequant_unit_16((it + 1) & 1, (it + 1) & 1, (u_first + it + 1) * kUnit);
-            } else if constexpr (Q8) {
-                dequant_unit_q8((it + 1) & 1, (it + 1) & 1, (u_first + it + 1) * kUnit);
-            } else if constexpr (FP8) {
-                dequant_unit_fp8((it + 1) & 1, (it + 1) & 1, (u_first + it + 1) * kUnit);
-            } else {
-                dequant_unit((it + 1) & 1, (it + 1) & 1);
+    if constexpr (PC) {
+        // Same schedule, the roles in different waves: between two barriers the dequantising
+        // waves commit unit it + 2, request unit it + 3 and dequantise unit it + 1 into buffer
+        // (it + 1) & 1, the multiplying waves work on unit it in buffer it & 1.
+        if (producer) {
+            const int32_t pg_first = __builtin_amdgcn_readfirstlane(load_page(0));
+            int32_t pg_next = load_page(1);
+            if (n_units > 0) issue_loads(0, pg_first);
+            for (int it = -2; it < n_units; ++it) {
+                if (it + 2 < n_units) commit_loads((it + 2) & 1);
+                const int32_t pg_s = __builtin_amdgcn_readfirstlane(pg_next);
+                pg_next = load_page(it + 4);
+                if (it + 3 < n_units) issue_loads(it + 3, pg_s);
+                if (it + 1 >= 0 && it + 1 < n_units) dequant_unit((it + 1) & 1, (it + 1) & 1);
+                __syncthreads();
             }
+            return;  // the epilogue has no workgroup barrier
         }
-        if (!compute_first && it >= 0) {
-            const int t0 = (u_first + it) * kUnit;
-            if constexpr (TQ4F) __builtin_amdgcn_s_setprio(1);
-            compute_unit(it & 1, t0, !(t0 >= i_lo && t0 + kUnit - 1 <= i_hi));
-            if constexpr (TQ4F) __builtin_amdgcn_s_setprio(0);
+        __builtin_amdgcn_s_setprio(1);  // (measured: none 8.20 ms, the multiplying waves 8.04, the dequantising waves 8.65)
+        for (int it = -2; it < n_units; ++it) {
+            if (it >= 0) {
+                const int t0 = (u_first + it) * kUnit;
+                compute_unit(it & 1, t0, !(t0 >= i_lo && t0 + kUnit - 1 <= i_hi));
+            }
+            __syncthreads();
         }
-        __syncthreads();
+        __builtin_amdgcn_s_setprio(0);
+    } else {
+        const int32_t pg_first = __builtin_amdgcn_readfirstlane(load_page(0));
+        int32_t pg_next = load_page(1);
+        if (n_units > 0) issue_loads(0, pg_first);
+        for (int it = -2; it < n_units; ++it) {
+            // commit unit it + 2 (loaded during the previous iteration), then start unit it + 3
+            if (it + 2 < n_units) commit_loads((it + 2) & 1);
+            // The page id of unit it + 4 is requested BEFORE the key loads of unit it + 3: a
+            // write to its register after them would have to wait for all of them to return.
+            const int32_t pg_s = __builtin_amdgcn_readfirstlane(pg_next);
+            pg_next = load_page(it + 4);
+            if (it + 3 < n_units) issue_loads(it + 3, pg_s);
+            // TQ4 pages: the two waves of a SIMD (w and w + 4) take the two halves of an iteration in
+            // opposite order, so that one dequantises (table reads and VALU) while the other
+            // multiplies.  Both orders are valid between two barriers: the dequantiser writes buffer
+            // (it + 1) & 1, the MFMAs read buffer it & 1.  (With the cheaper dequantisers of the other
+            // formats the same order in all waves measured faster.)
+            const bool compute_first = TQ4F && wave >= 4;  // wave-uniform
+            // (TQ4: while a wave multiplies it is the one the SIMD serves first, so its MFMAs go out as
+            // soon as their operands are there and the other wave's dequantiser fills the gaps: -4 %.
+            // The other formats, whose waves all run the same order, measured 5 % slower with it.)
+            if (compute_first && it >= 0) {
+                const int t0 = (u_first + it) * kUnit;
+                __builtin_amdgcn_s_setprio(1);
+                compute_unit(it & 1, t0, !(t0 >= i_lo && t0 + kUnit - 1 <= i_hi));
+                __builtin_amdgcn_s_setprio(0);
+            }
+            if (it + 1 >= 0 && it + 1 < n_units) {
+                if constexpr (K16) {
+                    dequant_unit_16((it + 1) & 1, (it + 1) & 1, (u_first + it + 1) * kUnit);
+                } else if constexpr (Q8) {
+                    dequant_unit_q8((it + 1) & 1, (it + 1) & 1, (u_first + it + 1) * kUnit);
+                } else if constexpr (FP8) {
+                    dequant_unit_fp8((it + 1) & 1, (it + 1) & 1, (u_first + it + 1) * kUnit);
+                } else {
+                    dequant_unit((it + 1) & 1, (it + 1) & 1);
+                }
+            }
+            if (!compute_first && it >= 0) {
+                const int t0 = (u_first + it) * kUnit;
+                if constexpr (TQ4F) __builtin_amdgcn_s_setprio(1);
+                compute_unit(it & 1, t0, !(t0 >= i_lo && t0 + kUnit - 1 <= i_hi));
+                if constexpr (TQ4F) __builtin_amdgcn_s_setprio(0);
+            }
+            __syncthreads();
+        }
     }
 
     // ---- epilogue: normalise, transpose through LDS, rotate back, store ----
