@@ -784,7 +784,8 @@ def run_workload(args, torch, lib, ffi, dev):
     qsl = (torch.arange(0, R + 1, dtype=torch.int32, device=dev) * ql).to(torch.int32)
     seq = torch.tensor(ctx, dtype=torch.int32, device=dev)
     ctxb = (seq - ql).to(torch.int32)
-    scratch_bytes = 32 << 20
+    # at least 32 MB, and what the library asks for this batch shape
+    scratch_bytes = max(32 << 20, int(lib.warp34_paged_attention_scratch_bytes(R * ql, Q_HEADS, int(ctx.max()))))
     scratch = torch.zeros(scratch_bytes, dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
     ex = ffi.Warp34Exec(stream, scratch.data_ptr(), scratch_bytes, 0)

@@ -105,6 +105,13 @@ struct AttnParams {
     // chunk geometry of a tile whose keys are exactly [0, max_seq_len): worked out on the host, so a
     // request that is as long as the host's bound needs no division on the device
     int spec_units, spec_upc, spec_chunks;
+    // Partial records: part_stride slots per output row.  Slots [0, max_chunks) belong to the
+    // split-K chunks of the decode kernels; a shared-prefix pass (tile kernel over the keys every
+    // request of the batch has in common) owns slots [pf_slot_base, pf_slot_base + pf_split), and
+    // the decode kernel then starts at key *key_floor.
+    int part_stride;
+    int pf_split, pf_slot_base;
+    const int32_t* key_floor;
 };
 
 // A finished output row leaves the kernels here: lane l holds channels 4 l .. 4 l + 3.  With a gate
@@ -453,8 +460,11 @@ __device__ __forceinline__ void wait_lds_reads() { asm volatile("s_waitcnt lgkmc
 // LDS: [pair table 64 KB][kTq4Waves staging areas of 8448 B][query operand table 9216 B][(m, l) tables].
 // A staging area holds one 32-token unit as it lies in the pages, written by LDS-direct loads:
 // K rows 0-31, then V rows 0-31, 132 bytes each (four runs of 16 rows = 2112 bytes).
-template <typename TQ, bool BAL>
+// SP: the keys below *P.key_floor belong to a shared-prefix pass (see AttnParams); a separate
+// instantiation, so that the plain form carries no trace of it.
+template <typename TQ, bool BAL, bool SP = false>
 __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, const BalItem& item, bool build_table) {
+    static_assert(!(SP && BAL), "shared-prefix pass: split-K form only");
     constexpr int kWaves = kTq4Waves;
     uint8_t* stage_all = smem + kLutBytes;
 
@@ -611,6 +621,9 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
     int i_lo = 0, i_hi = 0x7fffffff;   // intersection of the visible ranges
     uint32_t ok_mask = 0u;             // bit c: column c is live (wave-uniform)
     const bool simple = B.valid_token_mask == nullptr && B.sliding_window <= 0;
+    // keys below the floor were handled by the shared-prefix pass (a multiple of the unit size)
+    int key_floor = 0;
+    if constexpr (SP) key_floor = __builtin_amdgcn_readfirstlane(*P.key_floor);
     auto column_info = [&](bool accumulate) {
         const int t = fast_div(ncol, P.q_group);
         const int tok = tok0 + t;
@@ -618,8 +631,8 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         const int q_off = tok - rq_start;
         int mx = (B.mask_mode == WARP34_ATTN_MASK_NONCAUSAL_WINDOW) ? seq_after - 1 : ctx_before + q_off;
         if (mx >= seq_after) mx = seq_after - 1;
-        int mn = 0;
-        if (B.sliding_window > 0) mn = max(0, ctx_before + q_off - B.sliding_window + 1);
+        int mn = key_floor;
+        if (B.sliding_window > 0) mn = max(key_floor, ctx_before + q_off - B.sliding_window + 1);
         col_ok = ok;
         col_lo = ok ? mn : 0;
         col_hi = ok ? mx : -1;
@@ -641,9 +654,9 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         int hi_last = window ? seq_after - 1 : ctx_before + q_off0 + tile_tokens - 1;
         if (hi_first >= seq_after) hi_first = seq_after - 1;
         if (hi_last >= seq_after) hi_last = seq_after - 1;
-        u_lo = 0;
-        u_hi = hi_last >= 0 ? hi_last : -1;
-        i_lo = 0;
+        u_lo = key_floor;
+        u_hi = hi_last >= key_floor ? hi_last : -1;
+        i_lo = key_floor;
         i_hi = hi_first;
     } else {
         column_info(true);
@@ -1187,7 +1200,7 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
             if (BAL ? item.n_chunks > 1 : P.max_chunks > 1) {
                 // un-normalised, rotated, still carrying the table gain; the merge kernel finishes
                 const size_t prow = BAL ? bal_partial_row(item.slot, (int)gridDim.y, kv_sub, col)
-                                        : row * P.max_chunks + chunk;
+                                        : row * (SP ? P.part_stride : P.max_chunks) + chunk;
                 float* dst = P.part_acc + prow * kHeadDim;
                 *reinterpret_cast<f4*>(dst + 4 * lane) = f4{v[0], v[1], v[2], v[3]};
                 if (lane == 0) {
@@ -1208,13 +1221,13 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
     }
 }
 
-template <typename TQ, int NT>
+template <typename TQ, int NT, bool SP = false>
 __global__ __launch_bounds__(kTq4Waves * 64, 1) void paged_attn_tq4_kernel(const AttnParams P) {
     static_assert(NT == 1, "one 16-column tile per workgroup");
     extern __shared__ __align__(16) uint8_t smem[];
     // lut_read() addresses the table absolutely: the dynamic block starts at LDS address 0 because
     // the kernel has no static LDS (checked on the host before the first launch)
-    tq4_tile<TQ, false>(P, smem, BalItem{}, true);
+    tq4_tile<TQ, false, SP>(P, smem, BalItem{}, true);
 }
 
 // Balanced decode: grid = (groups, kv head x q subgroup).  Every wave computes the plan (the
@@ -1409,7 +1422,7 @@ __global__ __launch_bounds__(1024) void balanced_merge_kernel(const AttnParams P
 // Everything the row needs (validity, chunk records, accumulators) is requested in ONE memory
 // round trip: records and accumulators of all max_chunks slots are loaded speculatively and
 // the slots beyond the row's chunk count are discarded with selects.
-template <typename TQ>
+template <typename TQ, bool SP = false>
 __global__ __launch_bounds__(1024) void split_merge_kernel(const float* part_acc_in, const float* part_ml_in,
                                                            int max_chunks_in, const AttnParams P,
                                                            float out_scale, int rotate) {
@@ -1462,10 +1475,17 @@ __global__ __launch_bounds__(1024) void split_merge_kernel(const float* part_acc
     if (!s_valid) return;  // masked row: output untouched (uniform for the block)
     int n_chunks = (int)s_rec[0][2];
     if (n_chunks > P.max_chunks) n_chunks = P.max_chunks;
+    // slots of the row: its split-K chunks, then (SP, behind a gap) those of the shared-prefix pass
+    auto live_slot = [&](int s) {
+        if constexpr (SP) return s < n_chunks || (s >= P.pf_slot_base && s < P.pf_slot_base + P.pf_split);
+        return s < n_chunks;
+    };
+    const int n_slots = SP ? max_chunks_in : n_chunks;
 
     // global maximum of m over chunks with l > 0 (every thread scans the LDS copy)
     float m_tot = kNegBig;
-    for (int s = lane; s < n_chunks; s += 64) {
+    for (int s = lane; s < n_slots; s += 64) {
+        if (!live_slot(s)) continue;
         const f4 r = s_rec[s];
         if (r[1] > 0.f) m_tot = fmaxf(m_tot, r[0]);
     }
@@ -1481,7 +1501,7 @@ __global__ __launch_bounds__(1024) void split_merge_kernel(const float* part_acc
 #pragma unroll
     for (int k = 0; k < kMergeMaxPerGroup; ++k) {
         const int s = grp + k * kMergeGroups;
-        if (s < n_chunks) {
+        if (s < n_slots && live_slot(s)) {
             const f4 r = s_rec[s];
             if (r[1] > 0.f) {
                 const float w = __builtin_amdgcn_exp2f(r[0] - m_tot);
@@ -1620,6 +1640,89 @@ static void fill_spec_geometry(AttnParams& P, int max_seq_len) {
     if (P.spec_chunks < 1) P.spec_chunks = 1;
 }
 
+// ---- shared-prefix pass (verify batches whose requests share their leading pages) ----
+// The host cannot see the block tables, so a one-workgroup kernel finds the common leading run:
+// the pages that every request's block table holds at the same index and that lie below every
+// request's first query position (every query of the batch sees all of their keys).  It leaves
+// the length in tokens (a multiple of the unit; 0 below kSpMinTokens) and the descriptor of one
+// pseudo request -- all query tokens of the batch over exactly those keys -- in the header.
+struct SpHeader {
+    int32_t floor;   // keys [0, floor) are the shared prefix
+    int32_t qsl[2];  // query_start_loc of the pseudo request: {0, total_tokens}
+    int32_t seq;     // its seq_lens_after (= floor)
+    int32_t ctx;     // its context_lens_before (= floor: every key visible to every token)
+    int32_t pad[3];
+};
+constexpr int kSpMinTokens = 4096;
+
+__global__ __launch_bounds__(1024) void shared_prefix_probe_kernel(const warp34_attention_batch B, int block_size,
+                                                                   SpHeader* hdr) {
+    __shared__ int s_first_diff, s_min_ctx;
+    const int tid = (int)threadIdx.x;
+    if (tid == 0) {
+        s_first_diff = B.max_blocks_per_req;
+        s_min_ctx = 0x7fffffff;
+    }
+    __syncthreads();
+    for (int r = tid; r < B.num_reqs; r += 1024) {
+        const int q_len = B.query_start_loc[r + 1] - B.query_start_loc[r];
+        const int ctx = B.context_lens_before != nullptr ? B.context_lens_before[r] : B.seq_lens_after[r] - q_len;
+        atomicMin(&s_min_ctx, ctx < 0 ? 0 : ctx);
+    }
+    __syncthreads();
+    int max_pages = s_min_ctx / block_size;  // pages that lie entirely below every first query position
+    if (max_pages > B.max_blocks_per_req) max_pages = B.max_blocks_per_req;
+    // (request, page) pairs, sixteen per thread and round trip: the loads of a batch are independent
+    const long long pairs = (long long)(B.num_reqs - 1) * max_pages;
+    int first_diff = 0x7fffffff;
+    for (long long base = tid; base < pairs; base += 16 * 1024) {
+        int32_t mine[16], ref[16];
+        int page[16];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            const long long i = base + 1024ll * k;
+            const bool in = i < pairs;
+            const int r = in ? 1 + (int)(i / max_pages) : 1;
+            page[k] = in ? (int)(i - (long long)(r - 1) * max_pages) : 0x7fffffff;
+            const int p = in ? page[k] : 0;
+            mine[k] = B.block_tables[(size_t)r * B.max_blocks_per_req + p];
+            ref[k] = B.block_tables[p];
+        }
+#pragma unroll
+        for (int k = 0; k < 16; ++k)
+            if (mine[k] != ref[k] && page[k] < first_diff) first_diff = page[k];
+    }
+    if (first_diff != 0x7fffffff) atomicMin(&s_first_diff, first_diff);
+    __syncthreads();
+    if (tid == 0) {
+        const int pages = s_first_diff < max_pages ? s_first_diff : max_pages;
+        int floor = (pages * block_size) & ~(kUnit - 1);
+        if (floor < kSpMinTokens) floor = 0;
+        hdr->floor = floor;
+        hdr->qsl[0] = 0;
+        hdr->qsl[1] = B.total_tokens;
+        hdr->seq = floor;
+        hdr->ctx = floor;
+    }
+}
+
+// Batches that may take the pass: several requests, a few query tokens each (a verify step),
+// long contexts, plain causal masking.  (Decode batches keep the balanced shares; the pass costs
+// two small launches and wide partial records when nothing is shared.)
+static bool shared_prefix_applicable(const warp34_attention_batch* b, int q_group, int force_single) {
+    return !force_single && b->num_reqs >= 4 && b->max_q_len >= 2 && b->max_q_len <= kPfRows / q_group &&
+           b->total_tokens >= 16 && b->max_seq_len >= 8 * kSpMinTokens && b->sliding_window <= 0 &&
+           b->mask_mode == WARP34_ATTN_MASK_CAUSAL && b->valid_token_mask == nullptr && b->valid_req_mask == nullptr &&
+           b->context_lens_before != nullptr && (q_group & (q_group - 1)) == 0;
+}
+// parts of the prefix per tile: a function of the batch and of gqa only, never of the number of
+// local kv heads (a rank with one kv head must produce the bits of a rank with two)
+static int shared_prefix_parts(int total_tokens, int q_group, int q_subgroups) {
+    const int tiles = (total_tokens + kPfRows / q_group - 1) / (kPfRows / q_group) * q_subgroups;
+    int parts = (kTargetWorkgroupsPerHead + tiles - 1) / tiles;  // about one workgroup per CU at two kv heads
+    return parts < 1 ? 1 : (parts > 32 ? 32 : parts);
+}
+
 template <typename TQ>
 static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
                       const warp34_attention_batch* batch, const void* q, void* out, int num_q_heads,
@@ -1666,6 +1769,7 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     // tile's count is limited by its own units first) and keeps the partial records, and what
     // the merge kernel loads ahead of knowing the count, as small as the bound allows.
     P.max_chunks = grid_x;
+    P.part_stride = grid_x;
     fill_spec_geometry(P, batch->max_seq_len);
     if (P.max_chunks > 1) {
         uint8_t* ws = reinterpret_cast<uint8_t*>((uintptr_t)ex->scratch_ptr);
@@ -1680,6 +1784,51 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     const dim3 grid((unsigned)grid_x, (unsigned)kv_subs, (unsigned)grid_z);
     hipStream_t stream = (hipStream_t)ex->stream;
     int rc;
+    // Verify batches: the keys every request has in common go through the tile kernel once, for
+    // all query rows of the batch (its dequantisation is shared by 128 rows instead of 16); the
+    // decode kernel takes the private rest, the merge kernel both sets of partial records.
+    if (P.max_chunks > 1 && shared_prefix_applicable(batch, q_group, force_single)) {
+        const int parts = shared_prefix_parts(batch->total_tokens, q_group, P.q_subgroups);
+        const int stride = P.max_chunks + parts;
+        const size_t need = partial_bytes(rows, stride) + sizeof(SpHeader);
+        if (stride <= kMergeGroups * kMergeMaxPerGroup && need <= ex->scratch_size) {
+            P.part_stride = stride;
+            P.pf_split = parts;
+            P.pf_slot_base = P.max_chunks;
+            P.part_ml = P.part_acc + (size_t)rows * stride * kHeadDim;
+            SpHeader* hdr = reinterpret_cast<SpHeader*>(P.part_ml + (size_t)rows * stride * 4);
+            P.key_floor = &hdr->floor;
+            hipLaunchKernelGGL(shared_prefix_probe_kernel, dim3(1), dim3(1024), 0, stream, *batch, layout->block_size, hdr);
+            rc = (int)hipGetLastError();
+            if (rc) return rc;
+            AttnParams T = P;  // the pseudo request of the header, 128-row tiles
+            T.B.num_reqs = 1;
+            T.B.query_start_loc = hdr->qsl;
+            T.B.seq_lens_after = &hdr->seq;
+            T.B.context_lens_before = &hdr->ctx;
+            T.B.max_q_len = batch->total_tokens;
+            T.tok_tile = kPfRows / q_group;
+            T.key_floor = nullptr;
+            const int pf_tiles = (batch->total_tokens + T.tok_tile - 1) / T.tok_tile;
+            using PfL = PfLds<WARP34_KV_FORMAT_TQ4>;
+            rc = ensure_dynamic_lds(paged_prefill_tq4_kernel<TQ, WARP34_KV_FORMAT_TQ4, false, true, true>, PfL::kSmem, true);
+            if (rc) return rc;
+            hipLaunchKernelGGL((paged_prefill_tq4_kernel<TQ, WARP34_KV_FORMAT_TQ4, false, true, true>),
+                               dim3((unsigned)(pf_tiles * parts), (unsigned)kv_subs, 1u), dim3(12 * 64), PfL::kSmem,
+                               stream, T);
+            rc = (int)hipGetLastError();
+            if (rc) return rc;
+            rc = ensure_dynamic_lds(paged_attn_tq4_kernel<TQ, 1, true>, smem_bytes_for(1), true);
+            if (rc) return rc;
+            hipLaunchKernelGGL((paged_attn_tq4_kernel<TQ, 1, true>), grid, dim3(waves_for(1) * 64), smem_bytes_for(1),
+                               stream, P);
+            rc = (int)hipGetLastError();
+            if (rc) return rc;
+            hipLaunchKernelGGL((split_merge_kernel<TQ, true>), dim3((unsigned)rows), dim3(1024), 0, stream,
+                               (const float*)P.part_acc, (const float*)P.part_ml, stride, P, kLutInvGain, 1);
+            return (int)hipGetLastError();
+        }
+    }
     // Decode batches of several requests: equal shares of the batch's units per workgroup
     // instead of per-request chunks (the requests' lengths are unknown to the host and differ).
     if (balanced_decode_applicable(ex, batch, P.tiles_by_request, force_single)) {
@@ -1757,6 +1906,7 @@ static int launch_rows(const warp34_exec* ex, const warp34_kv_layer_layout* layo
     // tile's count is limited by its own units first) and keeps the partial records, and what
     // the merge kernel loads ahead of knowing the count, as small as the bound allows.
     P.max_chunks = grid_x;
+    P.part_stride = grid_x;
     fill_spec_geometry(P, batch->max_seq_len);
     if (P.max_chunks > 1) {
         uint8_t* ws = reinterpret_cast<uint8_t*>((uintptr_t)ex->scratch_ptr);
@@ -2194,6 +2344,14 @@ static size_t scratch_bytes_for(int local_kv_heads, int total_tokens, int num_re
         if (bound < want) want = bound;
     }
     size_t bytes = want >= 2 ? partial_bytes((long long)total_tokens * num_q_heads, (int)want) : 0;
+    // verify batches over long contexts may take the shared-prefix pass: its partial slots sit
+    // behind the split-K ones, and a header behind the records
+    if (want >= 2 && total_tokens >= 16 && (num_reqs < 0 || num_reqs >= 4) && max_seq_len >= 8 * kSpMinTokens &&
+        (max_q_len <= 0 || (max_q_len >= 2 && max_q_len <= kPfRows / q_group)) && (q_group & (q_group - 1)) == 0) {
+        const int parts = shared_prefix_parts(total_tokens, q_group, q_subgroups);
+        if ((int)want + parts <= kMergeGroups * kMergeMaxPerGroup)
+            bytes = partial_bytes((long long)total_tokens * num_q_heads, (int)want + parts) + sizeof(SpHeader);
+    }
     // balanced decode: (shares + requests) partial slots of 16 columns per (kv head, q subgroup)
     // and the per-token table
     // (only batches in which no request has more than one tile take it; max_q_len <= 0: not known)

@@ -72,7 +72,10 @@ __device__ __forceinline__ f4 pf_mfma32(h8 a, h8 b, f4 c) {
 // form); waves 8-11 load and dequantise the next unit, a whole 16-row run each.  Every SIMD then
 // holds two multiplying waves and one dequantising wave whose instruction streams never wait
 // for each other's results inside an iteration.
-template <typename TQ, int KVF, bool VF = false, bool PC = false>
+// SPLIT (with PC): blockIdx.x = tile * P.pf_split + part; a workgroup takes one of P.pf_split equal
+// parts of the tile's units and leaves un-normalised partial records (slot P.pf_slot_base + part
+// of every row, the decode kernels' format) for the merge kernel.
+template <typename TQ, int KVF, bool VF = false, bool PC = false, bool SPLIT = false>
 __global__ __launch_bounds__((PC ? 12 : kPfWaves) * 64, 1) void paged_prefill_tq4_kernel(const AttnParams P) {
     using M = PfLds<KVF>;
     constexpr bool FP8 = M::kFp8;
@@ -80,6 +83,7 @@ __global__ __launch_bounds__((PC ? 12 : kPfWaves) * 64, 1) void paged_prefill_tq
     constexpr bool Q8 = M::kQ8;   // Q8_0 rows: the key tile holds the codes, the value tile fp16(d * code) unless VF
     static_assert(!VF || FP8 || Q8, "scales in the probabilities: 8-bit rows only");
     static_assert(!PC || (!M::kFp8 && !M::k16 && !M::kQ8), "separate dequantising waves: TQ4 pages only");
+    static_assert(!SPLIT || PC, "split form: TQ4 pages");
     // VF: the tile holds code / kVfGain (a power of two: exact) and the weights p * d * kVfGain.  The
     // block scales of 8-bit rows are small (amax / 448, amax / 127): without the gain the low-order
     // weight operand, 2^-12 of the weight, would fall into fp16's subnormal range and lose its bits.
@@ -114,7 +118,9 @@ __global__ __launch_bounds__((PC ? 12 : kPfWaves) * 64, 1) void paged_prefill_tq
     const int ctx_before = B.context_lens_before != nullptr ? B.context_lens_before[req]
                                                             : seq_after - (rq_end - rq_start);
     const int tile_tok = P.tok_tile;  // 128 / q_group
-    const int tok0 = rq_start + (int)blockIdx.x * tile_tok;
+    const int tile_x = SPLIT ? (int)blockIdx.x / P.pf_split : (int)blockIdx.x;
+    const int part_x = SPLIT ? (int)blockIdx.x - tile_x * P.pf_split : 0;
+    const int tok0 = rq_start + tile_x * tile_tok;
     if (tok0 >= rq_end || tok0 >= B.total_tokens) return;
     int tile_tokens = rq_end - tok0;
     if (tile_tokens > tile_tok) tile_tokens = tile_tok;
@@ -141,8 +147,16 @@ __global__ __launch_bounds__((PC ? 12 : kPfWaves) * 64, 1) void paged_prefill_tq
     };
     const int lo_all = range_lo(q_off0);
     const int hi_all = range_hi(q_off0 + tile_tokens - 1);
-    const int u_first = lo_all >> 5;
-    const int n_units = hi_all >= lo_all ? (hi_all >> 5) - u_first + 1 : 0;
+    int u_first = lo_all >> 5;
+    int n_units = hi_all >= lo_all ? (hi_all >> 5) - u_first + 1 : 0;
+    if constexpr (SPLIT) {  // this workgroup's part of the units
+        const int per_part = (n_units + P.pf_split - 1) / P.pf_split;
+        const int first = part_x * per_part;
+        int n = n_units - first;
+        n = n < 0 ? 0 : (n > per_part ? per_part : n);
+        u_first += first;
+        n_units = n;
+    }
 
     const int my_col = 16 * wave + n;
     const int my_t = fast_div(my_col, P.q_group);
@@ -868,7 +882,7 @@ __global__ __launch_bounds__((PC ? 12 : kPfWaves) * 64, 1) void paged_prefill_tq
     // ---- epilogue: normalise, transpose through LDS, rotate back, store ----
     l_run = sum_over_rows(l_run);
     float* reg = reinterpret_cast<float*>(smem) + wave * 16 * 260;
-    const float inv = l_run > 0.f ? (TQ4F ? kLutInvGain : 1.0f) / l_run : 0.f;
+    const float inv = SPLIT ? 1.0f : (l_run > 0.f ? (TQ4F ? kLutInvGain : 1.0f) / l_run : 0.f);
 #pragma unroll
     for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -884,6 +898,16 @@ __global__ __launch_bounds__((PC ? 12 : kPfWaves) * 64, 1) void paged_prefill_tq
         const int a = col - t * P.q_group;
         const f4 x = *reinterpret_cast<const f4*>(reg + c * 260 + 4 * lane);
         float o[4] = {x[0], x[1], x[2], x[3]};
+        if constexpr (SPLIT) {
+            // un-normalised, rotated, still carrying the table gain: the merge kernel finishes
+            const size_t row = (size_t)(tok0 + t) * P.num_q_heads + (size_t)(q_head_base + a);
+            const size_t prow = row * P.part_stride + (size_t)(P.pf_slot_base + part_x);
+            *reinterpret_cast<f4*>(P.part_acc + prow * kHeadDim + 4 * lane) = x;
+            const float m_c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(m_run), c));
+            const float l_c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(l_run), c));
+            if (lane == 0) *reinterpret_cast<f4*>(P.part_ml + prow * 4) = f4{m_c, l_c, (float)P.pf_split, 0.f};
+            continue;
+        }
         if (rot_out) {  // values stored rotated: rotate the finished row back
             wht256_wave(o, lane);
 #pragma unroll
