@@ -72,7 +72,8 @@ MEASURED_TRAFFIC = {
     "fp8_decode_b32_ctx1k_64k": (1_190_750_000, "profiles/paged_attn_rows_fp8_decode_b32_ctx1k_64k.txt"),
     "fp8_decode_b1_ctx131072": (140_920_000, "profiles/paged_attn_rows_fp8_decode_b1_ctx131072.txt"),
     "q8_0_decode_b1_ctx131072": (145_100_000, "profiles/paged_attn_rows_q8_0_decode_b1_ctx131072.txt"),
-    "tq4_verify_16x4_ctx262144_shared200k": (720_130_000, "profiles/paged_attn_tq4_verify_16x4_ctx262144_shared200k.txt"),
+    # (the four kernels of the shared-prefix path together: probe 0.3 + tile 144.8 + decode 535.1 + merge 39.1 MB)
+    "tq4_verify_16x4_ctx262144_shared200k": (719_260_000, "profiles/paged_attn_tq4_verify_16x4_ctx262144_shared200k.txt"),
     "tq4_prefill_8x2048_ctx16384": (890_170_000, "profiles/paged_prefill_tq4_8x2048_ctx16384.txt"),
     "tq4_qsa_sparse_16x513_ctx131072": (23_400_000, "profiles/qsa_sparse_tq4_16x513_ctx131072.txt"),
     "tq4_norm_rope_append_8192": (183_280_000, "profiles/qk_norm_rope_tq4_append_8192.txt"),
@@ -857,7 +858,10 @@ def run_workload(args, torch, lib, ffi, dev):
             "frac": round(gbs / HBM_PEAK_GBS, 4),
             "traffic": MEASURED_TRAFFIC.get(args.workload, (None, None))[0],
             "traffic_source": MEASURED_TRAFFIC.get(args.workload, (None, None))[1],
-            "kernel": "paged_attn_%s_kernel (+ merge kernel, both inside the timed launch)"
+            "kernel": ("shared_prefix_probe_kernel + paged_prefill_tq4_kernel (shared pages, 32 parts) + "
+                       "paged_attn_tq4_kernel (private rest) + split_merge_kernel, all inside the timed launch")
+                      if args.workload in SHARED_PREFIX else
+                      "paged_attn_%s_kernel (+ merge kernel, both inside the timed launch)"
                       % (("tq4" if fmt == "tq4" else "rows") + ("_balanced" if R > 1 and ql == 1 else "")),
             "avg_launch_us": round(ms_per_step * 1e3, 3),
             "host_wall_us_per_step": round(t_wall / args.steps * 1e6, 2),

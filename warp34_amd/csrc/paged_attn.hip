@@ -1672,25 +1672,27 @@ __global__ __launch_bounds__(1024) void shared_prefix_probe_kernel(const warp34_
     __syncthreads();
     int max_pages = s_min_ctx / block_size;  // pages that lie entirely below every first query position
     if (max_pages > B.max_blocks_per_req) max_pages = B.max_blocks_per_req;
-    // (request, page) pairs, sixteen per thread and round trip: the loads of a batch are independent
-    const long long pairs = (long long)(B.num_reqs - 1) * max_pages;
+    // one request per wave (r = 1 + wave, + 16, ...), sixteen pages per lane and round trip: the
+    // loads of a batch are independent of each other
+    const int wave = tid >> 6, lane = tid & 63;
     int first_diff = 0x7fffffff;
-    for (long long base = tid; base < pairs; base += 16 * 1024) {
-        int32_t mine[16], ref[16];
-        int page[16];
+    for (int r = 1 + wave; r < B.num_reqs; r += 16) {
+        const int32_t* row = B.block_tables + (size_t)r * B.max_blocks_per_req;
+        for (int base = lane; base < max_pages; base += 16 * 64) {
+            int32_t mine[16], ref[16];
 #pragma unroll
-        for (int k = 0; k < 16; ++k) {
-            const long long i = base + 1024ll * k;
-            const bool in = i < pairs;
-            const int r = in ? 1 + (int)(i / max_pages) : 1;
-            page[k] = in ? (int)(i - (long long)(r - 1) * max_pages) : 0x7fffffff;
-            const int p = in ? page[k] : 0;
-            mine[k] = B.block_tables[(size_t)r * B.max_blocks_per_req + p];
-            ref[k] = B.block_tables[p];
+            for (int k = 0; k < 16; ++k) {
+                const int p = base + 64 * k;
+                const int pc = p < max_pages ? p : 0;
+                mine[k] = row[pc];
+                ref[k] = B.block_tables[pc];
+            }
+#pragma unroll
+            for (int k = 0; k < 16; ++k) {
+                const int p = base + 64 * k;
+                if (p < max_pages && mine[k] != ref[k] && p < first_diff) first_diff = p;
+            }
         }
-#pragma unroll
-        for (int k = 0; k < 16; ++k)
-            if (mine[k] != ref[k] && page[k] < first_diff) first_diff = page[k];
     }
     if (first_diff != 0x7fffffff) atomicMin(&s_first_diff, first_diff);
     __syncthreads();
