@@ -27,7 +27,7 @@ namespace w34 {
 
 constexpr int kPfWaves = 8;
 constexpr int kPfRows = 128;                                  // query rows per workgroup
-constexpr int kPfKStride = 528;                               // bytes per dequantised K row
+constexpr int kPfKStride = 544;                               // bytes per dequantised K row (measured: 128-bit reads of 16 rows at this stride do not conflict; 528, 560, 576 do)
 constexpr int kPfKBytes = 32 * kPfKStride;                    // 16896
 constexpr int kPfVBytes = 256 * 64;                           // V^T: 256 rows x 32 halves
 constexpr int kPfScaleBytes = 8 * 32 * 4;                     // per token: K d0, K d1, V d0, V d1 (Q8_0: K d0-d3, V d0-d3)
