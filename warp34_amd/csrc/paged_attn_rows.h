@@ -30,10 +30,11 @@ constexpr int kKv16Waves = 8;
 constexpr int kKv16RowStride = 528;                      // bytes, 512 + 16 pad
 constexpr int kKv8RowStride = 272;                       // bytes: Q8_0 rows as stored, FP8 rows + 8 pad
 constexpr int kKv16Stage = 2 * 16 * kKv16RowStride;      // K half + V half: 16896 B per wave
+constexpr int kKv16ColStride = 264;                      // dwords per column of a merge region (see kMergeColStride)
 // byte offset of the (m, l) exchange table: behind both the staging areas and the merge regions
 __host__ __device__ constexpr int kv16_ml_offset(int nt) {
     const int loop_bytes = kKv16Waves * kKv16Stage;
-    const int region_bytes = kKv16Waves * (nt * 16 * 260) * 4;
+    const int region_bytes = kKv16Waves * (nt * 16 * kKv16ColStride) * 4;
     return loop_bytes > region_bytes ? loop_bytes : region_bytes;
 }
 __host__ __device__ constexpr int kv16_smem_bytes(int nt) {
@@ -657,7 +658,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
     for (int nt = 0; nt < NT; ++nt) l_run[nt] = sum_over_rows(l_run[nt]);
 
     // ---- merge of the waves' states (same scheme and region layout as the TQ4 kernel) ----
-    constexpr int kColStride = 260;
+    constexpr int kColStride = kKv16ColStride;
     constexpr int kRegion = NT * 16 * kColStride;
     float* xbuf = reinterpret_cast<float*>(smem);
     float* mlbuf = reinterpret_cast<float*>(smem + kv16_ml_offset(NT));

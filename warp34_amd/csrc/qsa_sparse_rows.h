@@ -368,7 +368,7 @@ __global__ __launch_bounds__(kKv16Waves * 64, 1) void qsa_sparse_rows_kernel(con
 
     // ---- merge of the waves' states (scheme and region layout of the dense kernels) ----
     l_run = sum_over_rows(l_run);
-    constexpr int kColStride = 260;
+    constexpr int kColStride = kKv16ColStride;
     constexpr int kRegion = 16 * kColStride;
     float* xbuf = reinterpret_cast<float*>(smem);
     float* mlbuf = reinterpret_cast<float*>(smem + kv16_ml_offset(1));
