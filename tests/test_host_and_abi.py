@@ -92,3 +92,14 @@ def test_error_string_needs_no_gpu():
     lib = ffi.load()
     s = lib.warp34_cuda_error_string(1)
     assert s and b"invalid" in s.lower()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The benchmark measures one GPU; asked for more it says so and exits without touching a GPU."""
+    import sys
+
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in (r.stdout + r.stderr)
+    assert not any(ln.startswith("{") for ln in r.stdout.splitlines())
