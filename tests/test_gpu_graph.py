@@ -288,3 +288,82 @@ def test_bucketed_decode_graph_serves_any_live_count():
         assert hk.tobytes() == ref_pool.k.tobytes() and hv.tobytes() == ref_pool.v.tobytes(), "replay %d: pool bytes" % it
         ref = oracle.paged_attention(ref_pool, wb, q_in.cpu().numpy().view(np.uint16)[:n], DT_BF16, q_heads, n_threads=4)
         G.assert_close(got[:n], DT_BF16, ref, what="bucket replay %d (%d live) vs oracle" % (it, n))
+
+
+def test_shared_prefix_verify_step_replays_with_new_tables_and_lengths():
+    """A verify step over requests that share their leading pages, captured once.  What is shared
+    is found on the device from the block tables and lengths the step reads (the host never looks
+    at them), so the one graph serves tables that share 32 768 keys, tables that share nothing,
+    a request that ends inside the common pages and a request too short for the pass; every replay
+    gives the bytes of the eager call on the same device state and matches the oracle."""
+    import torch
+
+    import gpu_harness as G
+    from test_gpu_full_size import BS, BigPool
+    from warp34_amd import ffi
+
+    lib = G.lib()
+    q_heads, q_len = 16, 4
+    ctx0 = [40000, 40037, 41111, 39000]
+    R = len(ctx0)
+    pool = BigPool(ctx0, sum((c + BS - 1) // BS for c in ctx0) + 8, seed=941, shared_prefix=32768)
+    L = pool.dev.layout()
+    bound = 49152  # graph bucket: an upper bound on every sequence length
+
+    swapped = pool.bt.copy()
+    swapped[2, [0, 1]] = swapped[2, [1, 0]]  # request 2 holds the same pages, the first two in the other order
+    states = [
+        (pool.bt, ctx0),                          # 32 768 keys in common
+        (swapped, ctx0),                          # no common leading page
+        (pool.bt, [40000, 20010, 41111, 39000]),  # request 1 ends inside the common pages
+        (pool.bt, [40000, 40037, 3000, 39000]),   # request 2 is shorter than the smallest shared run the pass takes
+    ]
+
+    qsl = G.to_dev(np.arange(R + 1, dtype=np.int32) * q_len)
+    seq = G.to_dev(np.array(ctx0, dtype=np.int32))
+    ctxb = G.to_dev(np.array(ctx0, dtype=np.int32) - q_len)
+    btd = G.to_dev(pool.bt)
+    q_in = torch.zeros((R * q_len, q_heads, 256), dtype=torch.int16, device=G.DEV)
+    out = torch.zeros_like(q_in)
+    scratch = torch.zeros(96 << 20, dtype=torch.uint8, device=G.DEV)
+
+    def step_call():
+        ex = ffi.Warp34Exec(torch.cuda.current_stream().cuda_stream, scratch.data_ptr(), scratch.numel(), 0)
+        b = ffi.Warp34AttentionBatch(qsl.data_ptr(), ctxb.data_ptr(), seq.data_ptr(), btd.data_ptr(), None, None, None,
+                                     R, R * q_len, pool.bt.shape[1], q_len, bound, 0, 0, 0.0625, 0)
+        rc = lib.warp34_paged_attention_bf16(C.byref(ex), C.byref(L), C.byref(b), C.c_void_p(q_in.data_ptr()),
+                                             C.c_void_p(out.data_ptr()), q_heads)
+        assert rc == 0
+
+    def set_state(i):
+        bt, ctx = states[i]
+        btd.copy_(G.to_dev(bt))
+        seq.copy_(G.to_dev(np.array(ctx, dtype=np.int32)))
+        ctxb.copy_(G.to_dev(np.array(ctx, dtype=np.int32) - q_len))
+        q_in.copy_(G.to_dev(oracle.fill_normal(R * q_len * q_heads * 256, 950 + i, DT_BF16).reshape(R * q_len, q_heads, 256)))
+
+    set_state(0)
+    step_call()  # eager warm-up: configures the kernels' dynamic LDS once
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        step_call()
+
+    results = []
+    for i in [0, 1, 2, 3, 0]:
+        set_state(i)
+        out.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        got = out.cpu().numpy().view(np.uint16).copy()
+        out.zero_()
+        step_call()
+        torch.cuda.synchronize()
+        assert got.tobytes() == out.cpu().numpy().view(np.uint16).tobytes(), "state %d: replay differs from the eager call" % i
+        bt, ctx = states[i]
+        hb = oracle.HostBatch(np.arange(R + 1) * q_len, ctx, bt, context_lens_before=[c - q_len for c in ctx])
+        want = oracle.paged_attention(pool.host, hb, q_in.cpu().numpy().view(np.uint16), DT_BF16, q_heads,
+                                      n_threads=oracle.hw_threads())
+        G.assert_close(got, DT_BF16, want, what="shared-prefix graph, state %d" % i, scale=pool.scale_for(hb))
+        results.append(got)
+    assert results[0].tobytes() == results[4].tobytes(), "the first state replayed again gives other bytes"
