@@ -87,3 +87,32 @@ def test_one_kv_head_layouts_give_the_same_bytes():
         rc, part, _ = pool.G.dev_attention(pool.dev, hb, q_h, DT_BF16, 8, scratch_bytes=BIG, layout=lay)
         assert rc == 0
         assert part.tobytes() == np.ascontiguousarray(full[:, head * 8:(head + 1) * 8]).tobytes()
+
+
+def test_gated_entry_through_the_pass():
+    """The gate of warp34_paged_attention_gated_f16 is applied where the merged rows are stored, so through
+    the pass too it equals attention followed by warp34_apply_attn_output_gate_f16, byte for byte
+    (model/forward.rs:1192-1211 makes the two calls)."""
+    from oracle import DT_F16
+    from test_gpu_full_size import BS, BigPool
+    from test_gpu_output_gate import _run as gate_op
+
+    ctx, q_len = [40000, 40037, 41111, 39000], 4
+    R = len(ctx)
+    pool = BigPool(ctx, sum((c + BS - 1) // BS for c in ctx) + 8, seed=951, shared_prefix=32768)
+    n = R * q_len
+    q = oracle.fill_normal(n * Q_HEADS * D, 952, DT_F16).reshape(n, Q_HEADS, D)
+    hb = oracle.HostBatch(np.arange(R + 1) * q_len, pool.ctx, pool.bt, context_lens_before=[c - q_len for c in pool.ctx])
+    gate = oracle.f32_to_f16_bits(3.0 * oracle.f16_bits_to_f32(oracle.fill_normal(n * Q_HEADS * D, 953, DT_F16)))
+    gate = gate.reshape(n, Q_HEADS * D)
+    rc, plain, _ = pool.G.dev_attention(pool.dev, hb, q, DT_F16, Q_HEADS, scratch_bytes=BIG)
+    assert rc == 0
+    rc, small, _ = pool.G.dev_attention(pool.dev, hb, q, DT_F16, Q_HEADS, scratch_bytes=SMALL)
+    assert rc == 0 and plain.tobytes() != small.tobytes()  # the pass is taken
+    rc, want = gate_op(plain.reshape(n, Q_HEADS * D), gate)
+    assert rc == 0
+    rc, got, _ = pool.G.dev_attention(pool.dev, hb, q, DT_F16, Q_HEADS, scratch_bytes=BIG, gate=gate)
+    assert rc == 0
+    assert got.reshape(n, Q_HEADS * D).tobytes() == want.tobytes()
+    ref = oracle.paged_attention(pool.host, hb, q, DT_F16, Q_HEADS, n_threads=oracle.hw_threads())
+    pool.G.assert_close(plain, DT_F16, ref, what="shared prefix, fp16 queries", scale=pool.scale_for(hb))
