@@ -97,7 +97,7 @@ __device__ __forceinline__ f4 mfma_x16(u2v a, u2v b, f4 c) {
 // of a rotated row with large entries holds few distinct codes, so part of the fp16 rounding of
 // d * code is common to the block, and the inverse rotation of the finished row would gather
 // that common part into a single channel.
-template <typename TQ, int NT, int KVF, bool BAL, bool VRES = false>
+template <typename TQ, int NT, int KVF, bool BAL, bool VRES = false, bool STREAM = BAL>
 __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, const BalItem& item) {
     static_assert(!VRES || KVF == WARP34_KV_FORMAT_FP8_E4M3 || KVF == WARP34_KV_FORMAT_Q8_0, "residual operand: 8-bit rows");
     constexpr bool K8 = KVF == WARP34_KV_FORMAT_FP8_E4M3 || KVF == WARP34_KV_FORMAT_Q8_0;
@@ -357,12 +357,22 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
         const bool live = pos <= u_hi && pos + 15 >= u_lo && pg >= 0;
         const uint8_t* kp = k_base + (live ? (size_t)pg * L.k_page_stride_bytes + (size_t)in_page * L.k_token_stride_bytes : 0);
         const uint8_t* vp = v_base + (live ? (size_t)pg * L.v_page_stride_bytes + (size_t)in_page * L.v_token_stride_bytes : 0);
+        // STREAM: every key is read by exactly one workgroup (decode steps: no request has more
+        // than one tile), and the loads carry the non-temporal hint, which is worth 8 to 13 % on a
+        // plain streaming read of HBM and 3 to 8 % here.  Tiles that share a request's keys
+        // (verify, prefill through this kernel) keep ordinary loads: with the hint their batches
+        // measure 7 to 22 % slower, the lines are gone when the next tile asks for them.
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
             // pieces beyond the run (last, partial round of the 8-bit formats) re-read piece 0
             const int c = (kPieces % 64 == 0 || lane + 64 * i < kPieces) ? lane + 64 * i : 0;
-            pf[i] = *(global_cu4*)(kp + 16 * c);
-            pf[kLoads + i] = *(global_cu4*)(vp + 16 * c);
+            if constexpr (STREAM) {
+                pf[i] = __builtin_nontemporal_load((global_cu4*)(kp + 16 * c));
+                pf[kLoads + i] = __builtin_nontemporal_load((global_cu4*)(vp + 16 * c));
+            } else {
+                pf[i] = *(global_cu4*)(kp + 16 * c);
+                pf[kLoads + i] = *(global_cu4*)(vp + 16 * c);
+            }
         }
     };
     // rows outside [u_lo, u_hi] are stored as zeros: unwritten pool memory may hold NaN
@@ -752,7 +762,13 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
 template <typename TQ, int NT, int KVF, bool VRES>
 __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_rows_kernel(const AttnParams P) {
     extern __shared__ __align__(16) uint8_t smem[];
-    rows_tile<TQ, NT, KVF, false, VRES>(P, smem, BalItem{});
+    // (one body per kind of load: a branch around the loads themselves keeps the compiler from
+    // scheduling them freely and loses what the hint gains)
+    if (P.tiles_by_request != 0 && P.q_subgroups == 1) {  // uniform for the grid
+        rows_tile<TQ, NT, KVF, false, VRES, true>(P, smem, BalItem{});
+    } else {
+        rows_tile<TQ, NT, KVF, false, VRES, false>(P, smem, BalItem{});
+    }
 }
 
 template <typename TQ, int KVF, bool VRES>
