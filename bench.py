@@ -65,13 +65,13 @@ WORKLOADS = {
 # be read from inside this process, so workloads without such a profile report null.
 MEASURED_TRAFFIC = {
     # workload: (HBM bytes per launch of the dominant kernel, the profile that holds the counter readings)
-    "tq4_decode_b1_ctx131072": (71_810_000, "profiles/paged_attn_tq4_decode_b1_ctx131072.txt"),
-    "tq4_decode_b8_ctx131072": (557_580_000, "profiles/paged_attn_tq4_decode_b8_ctx131072.txt"),
-    "tq4_decode_b32_ctx1k_64k": (585_410_000, "profiles/paged_attn_tq4_decode_b32_ctx1k_64k.txt"),
-    "bf16_decode_b1_ctx32768": (69_540_000, "profiles/paged_attn_rows_bf16_decode_b1_ctx32768.txt"),
-    "fp8_decode_b32_ctx1k_64k": (1_191_950_000, "profiles/paged_attn_rows_fp8_decode_b32_ctx1k_64k.txt"),
-    "fp8_decode_b1_ctx131072": (140_920_000, "profiles/paged_attn_rows_fp8_decode_b1_ctx131072.txt"),
-    "q8_0_decode_b1_ctx131072": (145_110_000, "profiles/paged_attn_rows_q8_0_decode_b1_ctx131072.txt"),
+    "tq4_decode_b1_ctx131072": (71_830_000, "profiles/paged_attn_tq4_decode_b1_ctx131072.txt"),
+    "tq4_decode_b8_ctx131072": (557_550_000, "profiles/paged_attn_tq4_decode_b8_ctx131072.txt"),
+    "tq4_decode_b32_ctx1k_64k": (584_750_000, "profiles/paged_attn_tq4_decode_b32_ctx1k_64k.txt"),
+    "bf16_decode_b1_ctx32768": (69_550_000, "profiles/paged_attn_rows_bf16_decode_b1_ctx32768.txt"),
+    "fp8_decode_b32_ctx1k_64k": (1_193_900_000, "profiles/paged_attn_rows_fp8_decode_b32_ctx1k_64k.txt"),
+    "fp8_decode_b1_ctx131072": (142_270_000, "profiles/paged_attn_rows_fp8_decode_b1_ctx131072.txt"),
+    "q8_0_decode_b1_ctx131072": (145_270_000, "profiles/paged_attn_rows_q8_0_decode_b1_ctx131072.txt"),
     # (the four kernels of the shared-prefix path together: probe 0.27 + tile 144.82 + decode 534.24 + merge 39.06 MB)
     "tq4_verify_16x4_ctx262144_shared200k": (718_390_000, "profiles/paged_attn_tq4_verify_16x4_ctx262144_shared200k.txt"),
     "tq4_prefill_8x2048_ctx16384": (1_126_470_000, "profiles/paged_prefill_tq4_8x2048_ctx16384.txt"),
