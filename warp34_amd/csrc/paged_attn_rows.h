@@ -3,9 +3,9 @@
 // gfx950.  Same work decomposition, chunk geometry, wave merge and split-K partial format as
 // the TQ4 kernel in paged_attn.hip (which includes this file); only the per-unit body differs:
 //   * a 32-token unit is processed as two 16-token halves; the wave copies the 16 K rows and
-//     16 V rows of a half into its private LDS area.  16-bit rows (512 B) get a 528-byte row
-//     stride (132 dwords: the 8 lanes of a 128-bit read pass land on 32 distinct banks),
-//     8-bit rows (264 B / 272 B, codes and their fp32 block scales) a 272-byte one;
+//     16 V rows of a half into its private LDS area.  16-bit rows (512 B) get a row stride of
+//     544 bytes (keys) or 576 bytes (values), the strides at which their 128-bit operand reads
+//     are conflict-free; 8-bit rows (264 B / 272 B, codes and their fp32 block scales) 272 bytes;
 //   * S^T = K Q^T: A operand = 16 K rows read from LDS, B operand = the query rows, loaded
 //     once in MFMA layout.  8-bit codes are widened to fp16 in registers (exact) and the fp32
 //     block scales are applied to per-block partial scores, so K is never rounded;
@@ -27,9 +27,14 @@ typedef short s4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
 
 constexpr int kKv16Waves = 8;
-constexpr int kKv16RowStride = 528;                      // bytes, 512 + 16 pad
+// LDS row strides of 16-bit rows (512 B).  The key operand reads are 128 bits at (row n, piece b)
+// for 16 rows x 4 pieces per instruction, the value reads 128 bits at (row 4 b + i, piece n): a
+// probe of those two patterns measures the rate of a contiguous read at 544 / 608 / 672 bytes for
+// the first and at 576 bytes for the second, 40 % less at 528.
+constexpr int kKv16RowStride = 544;                      // key rows
+constexpr int kKv16VRowStride = 576;                     // value rows
 constexpr int kKv8RowStride = 272;                       // bytes: Q8_0 rows as stored, FP8 rows + 8 pad
-constexpr int kKv16Stage = 2 * 16 * kKv16RowStride;      // K half + V half: 16896 B per wave
+constexpr int kKv16Stage = 16 * (kKv16RowStride + kKv16VRowStride);  // K half + V half: 17920 B per wave
 constexpr int kKv16ColStride = 264;                      // dwords per column of a merge region (see kMergeColStride)
 // byte offset of the (m, l) exchange table: behind both the staging areas and the merge regions
 __host__ __device__ constexpr int kv16_ml_offset(int nt) {
@@ -106,7 +111,8 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
     constexpr bool IS_BF16 = !K8 && TQ::kStorageFormat == WARP34_KV_FORMAT_BF16;
     constexpr bool Q_BF16 = TQ::kStorageFormat == WARP34_KV_FORMAT_BF16;
     constexpr int kWaves = kKv16Waves;
-    constexpr int kRowStride = K8 ? kKv8RowStride : kKv16RowStride;  // LDS row stride
+    constexpr int kRowStride = K8 ? kKv8RowStride : kKv16RowStride;    // LDS row stride of the key rows
+    constexpr int kVRowStride = K8 ? kKv8RowStride : kKv16VRowStride;  // ... of the value rows
     constexpr int kRowBytes = K8 ? (FP8 ? 264 : 272) : 512;          // row in memory
 
     const int tid = (int)threadIdx.x;
@@ -400,7 +406,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
                         v8 = u2v{0u, 0u};
                     }
                     *reinterpret_cast<u2v*>(k_rows + row * kRowStride + 8 * col) = k8;
-                    *reinterpret_cast<u2v*>(v_rows + row * kRowStride + 8 * col) = v8;
+                    *reinterpret_cast<u2v*>(v_rows + row * kVRowStride + 8 * col) = v8;
                 }
             } else {
                 constexpr int kPiecesPerRow = kRowBytes / 16;  // 32 or 17
@@ -414,7 +420,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
                     }
                 }
                 *reinterpret_cast<u4*>(k_rows + row * kRowStride + 16 * col) = kv;
-                *reinterpret_cast<u4*>(v_rows + row * kRowStride + 16 * col) = vv;
+                *reinterpret_cast<u4*>(v_rows + row * kVRowStride + 16 * col) = vv;
             }
         }
     };
@@ -489,7 +495,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
                 float vf[4][8];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const uint8_t* vrow = v_rows + (4 * b + i) * kRowStride;
+                    const uint8_t* vrow = v_rows + (4 * b + i) * kVRowStride;
                     const int blk = 2 * h + (n >> 3);  // Q8_0 block of element 128 h + 8 n
                     const int off = FP8 ? 128 * h + 8 * n : 68 * blk + 4 + 8 * (n & 7);
                     const uint32_t* src = reinterpret_cast<const uint32_t*>(vrow + off);
@@ -533,7 +539,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
                 u4 vr[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    vr[i] = *reinterpret_cast<const u4*>(v_rows + (4 * b + i) * kRowStride + 256 * h + 16 * n);
+                    vr[i] = *reinterpret_cast<const u4*>(v_rows + (4 * b + i) * kVRowStride + 256 * h + 16 * n);
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     // 16-bit element j of the four token slices -> (t0,t1), (t2,t3)
