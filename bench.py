@@ -34,6 +34,7 @@ WORKLOADS = {
     "tq4_decode_b8_ctx131072": ("tq4", [131072] * 8, 0),
     "tq4_decode_b32_ctx1k_64k": ("tq4", None, 2 << 20),
     "bf16_decode_b1_ctx32768": ("bf16", [32768], 0),
+    "bf16_decode_b16_ctx32768": ("bf16", [32768] * 16, 0),
     # the un-rotated 8-bit rows the default TQ4 policy keeps for its last four layers
     "fp8_decode_b1_ctx131072": ("fp8", [131072], 0),
     "q8_0_decode_b1_ctx131072": ("q8_0", [131072], 0),
