@@ -115,6 +115,10 @@ struct AttnParams {
     int part_stride;
     int pf_split, pf_slot_base;
     const int32_t* key_floor;
+    // TQ4 decode kernels: a 32-token unit never straddles two pages (the page size is a multiple of
+    // 32) and both page strides fit 32 bits, so a unit's four runs follow from ONE block-table entry
+    // and two 32 x 32-bit products
+    int unit_in_page;
 };
 
 // A finished output row leaves the kernels here: lane l holds channels 4 l .. 4 l + 3.  With a gate
@@ -250,6 +254,23 @@ __device__ __forceinline__ void split_h2(float a, float b, uint32_t& hi, uint32_
     asm("v_fma_mixlo_f16 %0, %1, 1.0, -%2 op_sel:[0,0,0] op_sel_hi:[0,0,1]" : "=v"(l) : "v"(a), "v"(hi));
     asm("v_fma_mixhi_f16 %0, %1, 1.0, -%2 op_sel:[0,0,1] op_sel_hi:[0,0,1]" : "+v"(l) : "v"(b), "v"(hi));
     lo = l;
+}
+// a * (fp16 half of w) as one mixed-precision FMA that reads the half in place (v_fma_mix_f32 with
+// a zero addend; written as an fma so that the compiler forms it and places the wait states that
+// separate it from the instruction that produced a).  A product of -0 comes out as +0.
+__device__ __forceinline__ float mul_by_half_lo(float a, uint32_t w) {
+    return __builtin_fmaf(a, (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xFFFFu)), 0.0f);
+}
+__device__ __forceinline__ float mul_by_half_hi(float a, uint32_t w) {
+    return __builtin_fmaf(a, (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16)), 0.0f);
+}
+// maximum of three finite values in one instruction (fmaxf would first quiet each operand); the
+// operands must come from ordinary vector instructions: the compiler places no wait states in
+// front of an assembly statement that reads the result of an MFMA
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
 }
 __device__ __forceinline__ float half_lo_to_f32(uint32_t w) {
     return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xFFFFu));
@@ -730,6 +751,29 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
     const uint8_t* nk[2];  // run bases of the unit that is loaded next (wave-uniform)
     const uint8_t* nv[2];
     auto locate_unit = [&](int unit) {
+        if (P.unit_in_page) {  // uniform for the launch
+            const int pos = unit * kUnit;
+            const int page_slot = div_block(pos, P);
+            const int in_page = pos - page_slot * L.block_size;
+            int rel = page_slot - slot_base;
+            if (rel >= 64) {  // wave-uniform, at most once per 64 slots
+                slot_base = page_slot;
+                load_page_vec();
+                rel = 0;
+            }
+            const int32_t pg = __builtin_amdgcn_readlane(page_vec, rel);
+            // (the unit overlaps the visible key range, so its page holds a visible key and its
+            // block-table entry is a real page; rows of the unit outside the range are masked)
+            const bool live = pg >= 0;
+            const uint64_t tok_off = (uint64_t)((uint32_t)in_page * (uint32_t)kTq4RowBytes);
+            const uint64_t koff = live ? (uint64_t)(uint32_t)pg * (uint32_t)L.k_page_stride_bytes + tok_off : 0;
+            const uint64_t voff = live ? (uint64_t)(uint32_t)pg * (uint32_t)L.v_page_stride_bytes + tok_off : 0;
+            nk[0] = k_base + koff;
+            nk[1] = nk[0] + kRunBytes;
+            nv[0] = v_base + voff;
+            nv[1] = nv[0] + kRunBytes;
+            return;
+        }
 #pragma unroll
         for (int gidx = 0; gidx < 2; ++gidx) {
             const int pos = unit * kUnit + 16 * gidx;
@@ -891,6 +935,7 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
     const uint8_t* ka_lo = stage + unit_token(0, n >> 2, n & 3) * kTq4RowBytes;  // A row of sub-tile 0; sub-tile 1: + 8 rows
     const uint8_t* kt_lo = stage + unit_token(0, b, 0) * kTq4RowBytes;           // token of output row 4b; + 8 s + i rows
     const uint8_t* vt_lo = kt_lo + 2 * kRunBytes;
+    const uint32_t vt_lo_addr = stage_addr + (uint32_t)(2 * kRunBytes + unit_token(0, b, 0) * kTq4RowBytes);  // its LDS address
     const uint8_t* kt_n = kt_lo + (n & 3) * kTq4RowBytes;  // the token whose K scales this lane fetches (+ 8 s rows)
     const uint8_t* vt_n = vt_lo + (8 * ((n >> 2) & 1) + (n & 3)) * kTq4RowBytes;  // ... and V scales: token n & 7
 
@@ -999,7 +1044,15 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
                 const uint32_t* row32 = reinterpret_cast<const uint32_t*>(vt_lo + (8 * (t >> 2) + (t & 3)) * kTq4RowBytes);
-                vw[0][t] = n == 0 ? c0[t] : row32[n];  // (lane n = 0 reads dword 0 and drops it)
+                // (lane n = 0 reads dword 0 and drops it; the read is volatile so that it stays one
+                // unconditional instruction instead of a branch around the lanes with n = 0, and goes
+                // through an LDS-typed address: a volatile read through a generic pointer would be a
+                // FLAT load, which completes out of order with the LDS-direct loads and would break
+                // the hand-placed vmcnt waits)
+                typedef __attribute__((address_space(3))) const volatile uint32_t lds_vol_u32;
+                const uint32_t first_half = *reinterpret_cast<lds_vol_u32*>(
+                    (uintptr_t)(vt_lo_addr + (uint32_t)((8 * (t >> 2) + (t & 3)) * kTq4RowBytes + 4 * n)));
+                vw[0][t] = n == 0 ? c0[t] : first_half;
                 vw[1][t] = row32[17 + n];
             }
         }
@@ -1009,7 +1062,7 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         // ---- online softmax (log2 domain), per lane = per query column --------------------
         float p[8];
         {
-            float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+            float mx = fmaxf(max3(sc[0], sc[1], sc[2]), max3(sc[3], sc[4], max3(sc[5], sc[6], sc[7])));
             mx = max_over_rows(mx);
             const float m_new = fmaxf(m_run, mx);
             const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
@@ -1037,19 +1090,19 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         // ---- O^T += V^T P^T ------------------------------------------------------------------
         // weights of each half: probability times the half-row scale of the value row, as a high
         // and a low fp16 operand (split_h2)
+        if (MASKED) {
+            // masked tokens have p == 0; their scale pair is zeroed so that a garbage scale (rows
+            // beyond the sequence end) cannot inject NaN into the weights
+#pragma unroll
+            for (int t = 0; t < 8; ++t) vsc[t] = p[t] > 0.f ? vsc[t] : 0u;
+        }
         u4 ph[2], pl[2];
         uint32_t lo[2][4], hi[2][4];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             float w[8];
 #pragma unroll
-            for (int t = 0; t < 8; ++t) w[t] = p[t] * (h == 0 ? half_lo_to_f32(vsc[t]) : half_hi_to_f32(vsc[t]));
-            if (MASKED) {
-                // masked tokens have p == 0; select instead of multiply so that a garbage scale
-                // (rows beyond the sequence end) cannot inject NaN
-#pragma unroll
-                for (int t = 0; t < 8; ++t) w[t] = p[t] > 0.f ? w[t] : 0.f;
-            }
+            for (int t = 0; t < 8; ++t) w[t] = h == 0 ? mul_by_half_lo(p[t], vsc[t]) : mul_by_half_hi(p[t], vsc[t]);
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 uint32_t whi, wlo;
@@ -1772,6 +1825,10 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     P.tok_tile = (16 * nt) / q_group;
     if (P.tok_tile < 1) P.tok_tile = 1;
     P.min_upc = kMinUnitsPerChunk;
+    P.unit_in_page = (layout->block_size % kUnit == 0 && layout->k_page_stride_bytes <= 0xFFFFFFFFull &&
+                      layout->v_page_stride_bytes <= 0xFFFFFFFFull)
+                         ? 1
+                         : 0;
     P.max_chunks = force_single ? 1 : choose_max_chunks(ex, batch->total_tokens, num_q_heads, P.tok_tile,
                                                         P.q_subgroups);
     P.part_acc = nullptr;
