@@ -741,9 +741,18 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
     const int32_t* req_blocks = B.block_tables + (size_t)req * B.max_blocks_per_req;
     int slot_base = div_block(cu_first * kUnit, P);
     int page_vec;
+    // (Loaded and waited for in one assembly statement: were the load the compiler's, it would place
+    // a vmcnt(0) in front of every readlane of page_vec -- once per unit -- and that wait, which
+    // cannot tell the compiler's loads from the LDS-direct ones, would make every unit wait for all
+    // the K / V data in flight.  The reload happens once per 64 block-table slots.)
     auto load_page_vec = [&]() {
         const int slot = slot_base + lane;
-        page_vec = slot < B.max_blocks_per_req ? req_blocks[slot] : -1;
+        int32_t ids = -1;
+        if (slot < B.max_blocks_per_req) {
+            const int32_t* src = req_blocks + slot;
+            asm volatile("global_load_dword %0, %1, off\n\ts_waitcnt vmcnt(0)" : "=v"(ids) : "v"(src) : "memory");
+        }
+        page_vec = ids;
     };
     // Runs that do not overlap the visible key range, or whose block-table entry is missing,
     // are read from page 0 of the slab instead: every row they deliver is masked, and any
