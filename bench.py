@@ -64,7 +64,7 @@ WORKLOADS = {
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by
 # a plain copy of known size (the scale is stated in each profile); counters cannot
 # be read from inside this process, so workloads without such a profile report null.
-MEASURED_TRAFFIC = {
+PROFILED_TRAFFIC = {
     # workload: (HBM bytes per launch of the dominant kernel, the profile that holds the counter readings)
     "tq4_decode_b1_ctx131072": (71_830_000, "profiles/paged_attn_tq4_decode_b1_ctx131072.txt"),
     "tq4_decode_b8_ctx131072": (557_550_000, "profiles/paged_attn_tq4_decode_b8_ctx131072.txt"),
@@ -244,6 +244,20 @@ def cpu_baseline(torch, sample, threads, min_seconds=1.5):
     t0 = time.perf_counter()
     oracle.kv_cache_write(small, wb, kk, kk, oracle.DT_BF16)
     t_append = time.perf_counter() - t0
+    # the same append on all threads: every thread appends its own 4 096 rows into its own pages
+    # (the oracle's append is a plain C loop over rows; ctypes releases the interpreter lock)
+    from concurrent.futures import ThreadPoolExecutor
+
+    pools = [oracle.HostPool(rows // (2 * KV_HEADS) // BLOCK, KV_HEADS, HEAD_DIM, BLOCK, ofmt, xf) for _ in range(threads)]
+    with ThreadPoolExecutor(threads) as ex:
+        list(ex.map(lambda pl: oracle.kv_cache_write(pl, wb, kk, kk, oracle.DT_BF16), pools))  # warm-up
+        t0 = time.perf_counter()
+        list(ex.map(lambda pl: oracle.kv_cache_write(pl, wb, kk, kk, oracle.DT_BF16), pools))
+        t_append_all = time.perf_counter() - t0
+    # decode on one thread: one run (16 x the time of the all-threads run)
+    t0 = time.perf_counter()
+    oracle.paged_attention(pool, hb, qb, oracle.DT_BF16, Q_HEADS, n_threads=1)
+    t_one = time.perf_counter() - t0
     reps, t_total, want = 0, 0.0, None
     while t_total < min_seconds:
         t0 = time.perf_counter()
@@ -258,10 +272,19 @@ def cpu_baseline(torch, sample, threads, min_seconds=1.5):
         "value": round(kv_bytes / dt / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
         "sample": "CPU oracle (oracle/tq4_oracle.c) over the same workload: layer 0's pages as written by the append "
                   "kernel, %d of %d requests (%d context tokens), %d query token(s) each, %d pthreads on %s "
-                  "(%d hardware threads): %.1f ms/layer, mean of %d runs; append of %d rows single-thread: %.0f rows/s"
-                  % (keep, len(ctx), tot, ql, threads, cpu_model(), os.cpu_count() or 0, dt * 1e3, reps, rows,
-                     rows / t_append),
+                  "(%d hardware threads): %.1f ms/layer, mean of %d runs; the same on 1 thread: %.1f ms/layer; append of "
+                  "%d rows: %.0f rows/s on 1 thread, %.0f rows/s on %d threads"
+                  % (keep, len(ctx), tot, ql, threads, cpu_model(), os.cpu_count() or 0, dt * 1e3, reps, t_one * 1e3, rows,
+                     rows / t_append, threads * rows / t_append_all, threads),
         "us_per_layer": round(dt * 1e6, 1),
+        # the four legs: decode and append, one thread and all threads (`value` is decode on all threads)
+        "legs": {
+            "decode_all_threads": {"threads": threads, "GBps": round(kv_bytes / dt / 1e9, 4), "us_per_layer": round(dt * 1e6, 1)},
+            "decode_1_thread": {"threads": 1, "GBps": round(kv_bytes / t_one / 1e9, 4), "us_per_layer": round(t_one * 1e6, 1)},
+            "append_1_thread": {"threads": 1, "rows_per_s": round(rows / t_append), "rows": rows},
+            "append_all_threads": {"threads": threads, "rows_per_s": round(threads * rows / t_append_all),
+                                   "rows": threads * rows},
+        },
         "gpu_vs_oracle": {"max_abs_err": float(err.max()), "max_rel": float(err.max() / max(np.abs(want).max(), 1e-30)),
                           "worst_excess_over_2e-3_plus_1e-2_want": float((err - (2e-3 + 1e-2 * np.abs(want))).max())},
     }
@@ -339,8 +362,8 @@ def run_prefill(args, torch, lib, ffi, layers, ctx, n_layers, pool_pages, fmt):
                    "pool_pages": pool_pages,
                    "attention_flops_per_step": flops, "rows_appended_per_step": N * KV_HEADS * 2},
         "roofline": {"bound": "mfma", "achieved": round(tf_attn, 1), "peak": peak, "unit": "TFLOP/s",
-                     "frac": round(tf_attn / peak, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, (None, None))[0],
-                     "traffic_source": MEASURED_TRAFFIC.get(args.workload, (None, None))[1],
+                     "frac": round(tf_attn / peak, 4), "traffic": PROFILED_TRAFFIC.get(args.workload, (None, None))[0],
+                     "traffic_source": PROFILED_TRAFFIC.get(args.workload, (None, None))[1],
                      "kernel": "paged_prefill_tq4_kernel (attention-only launches)",
                      "avg_launch_us": round(ms_attn * 1e3, 1)},
     }))
@@ -382,8 +405,8 @@ def run_gate(args, torch, lib, ffi):
         "dtype": "f32 arithmetic on f16 rows", "data": "synthetic",
         "config": {"workload": args.workload, "tokens": n, "total_dim": dim, "bytes_per_step": nbytes},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, (None, None))[0],
-                     "traffic_source": MEASURED_TRAFFIC.get(args.workload, (None, None))[1], "kernel": "attn_output_gate_kernel<true>",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": PROFILED_TRAFFIC.get(args.workload, (None, None))[0],
+                     "traffic_source": PROFILED_TRAFFIC.get(args.workload, (None, None))[1], "kernel": "attn_output_gate_kernel<true>",
                      "avg_launch_us": round(ms * 1e3, 2)},
     }))
 
@@ -448,8 +471,8 @@ def run_qsa(args, torch, lib, ffi, layers, ctx_len, n_layers, n_tok, fmt, select
                    "head_dim": HEAD_DIM, "page_tokens": BLOCK, "kv_format": "tq4+wht256" if fmt == "tq4" else fmt,
                    "kv_pools_cycled": n_layers, "bytes_per_step": nbytes},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, (None, None))[0],
-                     "traffic_source": MEASURED_TRAFFIC.get(args.workload, (None, None))[1],
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": PROFILED_TRAFFIC.get(args.workload, (None, None))[0],
+                     "traffic_source": PROFILED_TRAFFIC.get(args.workload, (None, None))[1],
                      "kernel": ("qsa_sparse_tq4_kernel" if fmt == "tq4" else "qsa_sparse_rows_kernel") +
                                " + qsa_sparse_merge_kernel (whole call)",
                      "avg_launch_us": round(ms * 1e3, 2)},
@@ -503,8 +526,8 @@ def run_append(args, torch, lib, ffi, layers, n, n_layers, fmt):
                    "page_tokens": BLOCK, "kv_format": "tq4+wht256" if fmt == "tq4" else fmt, "kv_pools_cycled": n_layers,
                    "bytes_per_step": bytes_step},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, (None, None))[0],
-                     "traffic_source": MEASURED_TRAFFIC.get(args.workload, (None, None))[1],
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": PROFILED_TRAFFIC.get(args.workload, (None, None))[0],
+                     "traffic_source": PROFILED_TRAFFIC.get(args.workload, (None, None))[1],
                      "kernel": "kv_append_kernel", "avg_launch_us": round(ms * 1e3, 2)},
     }))
 
@@ -586,8 +609,8 @@ def run_producer(args, torch, lib, ffi, layers, n, n_layers, fmt):
                    "head_dim": HEAD_DIM, "page_tokens": BLOCK, "kv_format": "tq4+wht256" if fmt == "tq4" else fmt,
                    "kv_pools_cycled": n_layers, "bytes_per_step": bytes_step},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, (None, None))[0],
-                     "traffic_source": MEASURED_TRAFFIC.get(args.workload, (None, None))[1],
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": PROFILED_TRAFFIC.get(args.workload, (None, None))[0],
+                     "traffic_source": PROFILED_TRAFFIC.get(args.workload, (None, None))[1],
                      "kernel": "qk_norm_rope_kernel<true, true> (fused cache write)",
                      "avg_launch_us": round(ms_fused * 1e3, 2)},
     }))
@@ -672,8 +695,8 @@ def run_fused_qk_gate(args, torch, lib, ffi, layers, n, n_layers, fmt):
                    "kv_format": "tq4+wht256" if fmt == "tq4" else fmt, "kv_pools_cycled": n_layers,
                    "bytes_per_step": bytes_step},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, (None, None))[0],
-                     "traffic_source": MEASURED_TRAFFIC.get(args.workload, (None, None))[1],
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": PROFILED_TRAFFIC.get(args.workload, (None, None))[0],
+                     "traffic_source": PROFILED_TRAFFIC.get(args.workload, (None, None))[1],
                      "kernel": "fused_qk_norm_rope_gate_kernel (cache write fused)",
                      "avg_launch_us": round(ms_fused * 1e3, 2)},
     }))
@@ -857,8 +880,11 @@ def run_workload(args, torch, lib, ffi, dev):
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(gbs / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC.get(args.workload, (None, None))[0],
-            "traffic_source": MEASURED_TRAFFIC.get(args.workload, (None, None))[1],
+            # HBM bytes per launch as the named profile measured them (rocprofv3 counters cannot be read
+            # inside this process): a figure of that profile's run, not of this one; null with --ctx
+            "traffic": None if args.ctx else PROFILED_TRAFFIC.get(args.workload, (None, None))[0],
+            "traffic_source": None if args.ctx else PROFILED_TRAFFIC.get(args.workload, (None, None))[1],
+            "traffic_measured_in_this_run": False,
             "kernel": ("shared_prefix_probe_kernel + paged_prefill_tq4_kernel (shared pages, 32 parts) + "
                        "paged_attn_tq4_kernel (private rest) + split_merge_kernel, all inside the timed launch")
                       if args.workload in SHARED_PREFIX else

@@ -177,9 +177,10 @@ int warp34_paged_attention_bf16(const warp34_exec* ex, const warp34_kv_layer_lay
                                 const warp34_attention_batch* batch,
                                 const void* q_in, void* attn_out, int num_q_heads); /* warp34_cuda.h:366-367 */
 
-/* Test-only kernel selector (op_paged_attn.cu:1451-1519): 0 = split-K decode/verify kernel
- * run as a single pass, 1 / 2 = the multi-row MFMA tile kernel.  All selections compute
- * the same function. */
+/* Test-only kernel selector (op_paged_attn.cu:1451-1519): use_64q == 0 runs the decode / verify
+ * kernel as a single pass (no split, scratch untouched), any other value the 128-row MFMA tile
+ * kernel (when the layout admits it: a power-of-two number of q heads per kv head; otherwise as 0).
+ * Both compute the same function, with different summation orders. */
 int warp34_paged_attention_f16_force_kernel_for_test(
     const warp34_exec* ex, const warp34_kv_layer_layout* layout,
     const warp34_attention_batch* batch,
@@ -314,10 +315,12 @@ size_t warp34_paged_attention_scratch_bytes_for_layout(const warp34_kv_layer_lay
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
  * reference.  The split-K partials go to a WARP34_STATIC_SCRATCH_BYTES array inside the library,
  * one copy per device, held until the process ends; ex->scratch_ptr / scratch_size are ignored and
- * nothing is allocated or freed.  A batch that would want more scratch than that
- * (warp34_paged_attention_scratch_bytes_for_layout) is refused with hipErrorOutOfMemory (2) and
- * nothing is launched.  Results equal warp34_paged_attention_bf16 with an 8 MiB scratch bit for
- * bit.  All calls on one device share the array: calls that overlap in time on one device (two
+ * nothing is allocated or freed.  Results equal warp34_paged_attention_bf16 with an 8 MiB scratch
+ * bit for bit: like that call, a batch whose full split wants more than the array holds
+ * (warp34_paged_attention_scratch_bytes_for_layout) runs with fewer chunks, or without the
+ * shared-prefix pass.  Limit: a batch of more than 4032 query rows (total_tokens x num_q_heads;
+ * two 1040-byte records per row no longer fit) is refused with hipErrorOutOfMemory (2) and nothing
+ * is launched.  All calls on one device share the array: calls that overlap in time on one device (two
  * streams) race on it and must be ordered by the caller.  The first call on a device looks up the
  * array's address; make it outside stream capture. */
 #define WARP34_STATIC_SCRATCH_BYTES (8u << 20)

@@ -1,7 +1,9 @@
 """GPU parity: paged GQA decode / verify attention through the C ABI vs the CPU oracle.
 
-Tolerance: |got - want| <= 2e-3 * scale + 1e-2 |want| against the fp64-accumulating oracle,
-scale = magnitude of the V channel being averaged (1 on unit-scale data, see gpu_harness.assert_close).
+Tolerance (gpu_harness.assert_close): |got - want| <= 2e-3 + 1e-2 |want| against the fp64-accumulating
+oracle on every channel of unit-scale data; only on the x20 outlier channels of the benchmark inputs
+(three per head) is the absolute part taken relative to the channel's magnitude, 2e-3 * max|V|.  Every
+call logs its worst excess over the plain bound on ALL channels (pytest's terminal summary).
 Invariants follow the reference's GPU tests: page-permutation 0-ULP
 (tests/backbone_and_collectives.rs:455-572), split vs single pass < 2e-3 and graph-bucket
 bound independence (tests/tq4_vision_and_moe.rs:1355-1663), masked rows untouched
@@ -164,10 +166,16 @@ def test_force_kernel_selector_agrees():
     hb = oracle.HostBatch(aq, [260], bt, context_lens_before=ctx)
     want = oracle.paged_attention(pool, hb, q, DT_F16, 8)
     dpool = _dev_pool(pool)
+    outs = {}
     for sel in (0, 1, 2):
         rc, got, _ = G.dev_attention(dpool, hb, q, DT_F16, 8, force_kernel=sel)
         assert rc == 0
         G.assert_close(got, DT_F16, want, what="selector %d" % sel)
+        outs[sel] = got.tobytes()
+    # 0 = the decode / verify kernel as one pass, anything else = the 128-row tile kernel: two
+    # kernels that add the same products in different orders, so the bytes differ
+    assert outs[1] == outs[2]
+    assert outs[0] != outs[1]
 
 
 # ---- 16-bit pages (FP16 pages with the f16 entry point, BF16 pages with the bf16 one) ----
@@ -336,7 +344,7 @@ def _prefill_case(dtype, block_size, seq_lens, q_lens, seed, q_heads=16, force=N
 def test_prefill_tile_kernel_forced_small(block_size):
     """Ragged tiles: chunk lengths that are not multiples of the 16-token tile, one request with
     no prefix, one whose chunk starts in the middle of a page."""
-    _prefill_case(DT_F16, block_size, [300, 77, 45], [150, 77, 3], 201, force=0)
+    _prefill_case(DT_F16, block_size, [300, 77, 45], [150, 77, 3], 201, force=2)
     _prefill_case(DT_F16, block_size, [33, 700], [1, 37], 202, q_heads=8, force=1)
 
 
@@ -348,7 +356,7 @@ def test_prefill_tile_kernel_auto_dispatch(dtype):
 
 @pytest.mark.parametrize("mask_mode,window", [(0, 100), (1, 0), (1, 64)])
 def test_prefill_tile_kernel_windows(mask_mode, window):
-    _prefill_case(DT_F16, 16, [400, 130], [90, 130], 221, force=0, mask_mode=mask_mode, window=window)
+    _prefill_case(DT_F16, 16, [400, 130], [90, 130], 221, force=1, mask_mode=mask_mode, window=window)
 
 
 @pytest.mark.parametrize("dtype", [DT_BF16, DT_F16])
@@ -466,7 +474,7 @@ def test_prefill_tile_kernel_masks_and_page_permutation():
         hb = oracle.HostBatch(aq, seq_lens, bt, context_lens_before=ctx, valid_token_mask=tmask, valid_req_mask=rmask)
         want = oracle.paged_attention(pool, hb, q, DT_F16, 8)
         dpool = _dev_pool(pool)
-        rc, got, _ = G.dev_attention(dpool, hb, q, DT_F16, 8, force_kernel=0, sentinel=0x5500)
+        rc, got, _ = G.dev_attention(dpool, hb, q, DT_F16, 8, force_kernel=1, sentinel=0x5500)
         assert rc == 0
         dead = np.zeros(sum(q_lens), dtype=bool)
         dead[[0, 17, 41, 153]] = True

@@ -6,7 +6,9 @@ The pools are too large to build with the CPU oracle in test time, so each test
      the appended rows against the oracle's encoder, byte for byte, at this size;
   2. downloads the pool and lets the oracle attend over those very bytes;
   3. compares the library's attention output with it under the usual tolerance
-     (|err| <= 2e-3 * scale + 1e-2 |want|, scale = magnitude of the V channel, see gpu_harness).
+     (|err| <= 2e-3 + 1e-2 |want| on every plain channel; on the three x20 outlier channels per
+     head the absolute part is 2e-3 * max|V| of the channel, see gpu_harness.assert_close, which
+     also logs the worst excess over the plain bound on all channels).
 Where the oracle would take minutes (prefill: 16 384 query tokens) it is run on a sample of the
 query tokens through its own token mask; the library computes every token.
 """
@@ -183,6 +185,19 @@ def test_chunked_prefill_8x2048_on_16k_prefix():
     ob = oracle.HostBatch(np.arange(R + 1) * chunk, pool.ctx, pool.bt, context_lens_before=[prefix] * R,
                           valid_token_mask=mask)
     _attend_and_compare(pool, hb, q, rows=rows, oracle_batch=ob)
+
+
+def test_tq4_decode_131072_tokens_headline_shape():
+    """The headline shape itself: ONE sequence of 131 072 tokens over TQ4 pages, one query token --
+    split over the whole chip (128 chunks per kv head, 2.2 MB of partial records) and, without
+    scratch, as a single pass."""
+    n = 131072
+    pool = BigPool([n], n // BS + 8, seed=451)
+    pool.check_sampled_rows_bit_exact()
+    q = oracle.fill_normal(Q_HEADS * D, 452, DT_BF16).reshape(1, Q_HEADS, D)
+    hb = oracle.HostBatch([0, 1], pool.ctx, pool.bt, context_lens_before=[n - 1])
+    _attend_and_compare(pool, hb, q, scratch=4 << 20)
+    _attend_and_compare(pool, hb, q, scratch=0)
 
 
 def test_fp8_decode_131072_tokens():

@@ -2,7 +2,8 @@
 (split-K partials in a device array inside the library).  Called through the C ABI with an exec
 that carries no scratch, and compared byte for byte with warp34_paged_attention_bf16 given an
 8 MiB scratch, on two calls in a row, the second with a smaller input (the array keeps the first
-call's contents); then a batch whose scratch need exceeds the array is refused."""
+call's contents); batches whose full split wants more than the array run as they do with an 8 MiB
+scratch; a batch with more query rows than the entry point's limit is refused."""
 import ctypes as C
 
 import numpy as np
@@ -51,20 +52,27 @@ def test_static_scratch_entry_point_matches_on_two_calls_in_a_row():
     _both(FMT_BF16, 64, [5000], [1], 9104)               # row-format kernel
 
 
+def test_static_scratch_entry_point_degrades_like_an_8mib_scratch():
+    """Shapes whose full split wants more than the array (a verify batch that may take the
+    shared-prefix pass: 38 slots per row; a decode batch of 200 requests: 328 shares) run as
+    warp34_paged_attention_bf16 runs them with 8 MiB, byte for byte."""
+    _both(FMT_TQ4, 64, [33000, 33100, 34000, 32900], [4, 4, 4, 4], 9106)
+    _both(FMT_TQ4, 16, [40] * 200, [1] * 200, 9107)
+
+
 def test_static_scratch_entry_point_refuses_what_does_not_fit():
     import torch
 
     import gpu_harness as G
 
-    n_req = 200  # balanced shares: (128 + 200) x 2 x 16 partial rows of 1040 B > 8 MiB
+    n_req = 260  # 260 x 16 = 4160 query rows: two records per row no longer fit in 8 MiB
     seq_lens = [40] * n_req
     pool, bt, k, v, q, aq, ctx = make_case(FMT_TQ4, 16, seq_lens, [1] * n_req, 9105, DT_BF16, q_heads=16)
     hb = oracle.HostBatch(aq, seq_lens, bt, context_lens_before=ctx)
     dpool = G.DevPool(pool)
     dpool.upload()
     L = dpool.layout()
-    need = G.lib().warp34_paged_attention_scratch_bytes_for_layout(C.byref(L), n_req, n_req, 16, 40)
-    assert need > STATIC_BYTES
+    assert n_req * 16 * 2 * 1040 > STATIC_BYTES
     db = G.DevBatch(hb)
     B = db.struct()
     ex, _ = G.make_exec(0)

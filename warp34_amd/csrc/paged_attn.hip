@@ -2170,7 +2170,11 @@ static int common_checks(const warp34_exec* ex, const warp34_kv_layer_layout* la
 template <typename TQ>
 static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
                            const warp34_attention_batch* batch, const void* q, void* out, int num_q_heads,
-                           int force_single, const void* gate = nullptr) {
+                           int force, const void* gate = nullptr) {
+    // force (the test selector): 0 = the dispatch below, 1 = the decode / verify kernel as a single
+    // pass, 2 = the 128-row tile kernel (where the batch shape admits it, else as 1)
+    const int force_single = force != 0 ? 1 : 0;
+    const bool force_tile = force == 2;
     if (layout->local_kv_heads <= 0 || num_q_heads % layout->local_kv_heads != 0 || batch->num_reqs <= 0 ||
         !batch->query_start_loc || !batch->seq_lens_after || !batch->block_tables ||
         batch->max_blocks_per_req <= 0 || batch->sliding_window < 0 ||
@@ -2180,10 +2184,10 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
     if (is_tq4_wht(layout)) {
         if (!tq4_geometry_ok(layout, q) || (((uintptr_t)out) & 7u) != 0) return (int)hipErrorNotSupported;
         // Many query rows per request and enough tiles to fill the chip: the tile kernel shares
-        // every dequantised key block between 128 query rows.  The test selector forces it.
+        // every dequantised key block between 128 query rows.
         const bool many_rows = batch->max_q_len >= 32 &&
                                (long long)batch->total_tokens * num_q_heads >= 128ll * kPfRows;
-        if ((force_single || many_rows) && prefill_tq4_applicable(layout, batch, num_q_heads))
+        if ((force_tile || (!force && many_rows)) && prefill_tq4_applicable(layout, batch, num_q_heads))
             return launch_prefill_tq4<TQ, WARP34_KV_FORMAT_TQ4>(ex, layout, batch, q, out, num_q_heads, gate);
         return launch_tq4<TQ>(ex, layout, batch, q, out, num_q_heads, force_single, gate);
     }
@@ -2191,11 +2195,10 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
     // point, BF16 pages with the bf16 one, as in the reference)
     if (is_kv16(layout, TQ::kStorageFormat)) {
         if (!kv16_geometry_ok(layout, q, out)) return (int)hipErrorNotSupported;
-        // many query rows per request: the tile kernel (rows copied as stored).  The test selector
-        // keeps its meaning of "one pass of the row kernel" for these pages.
+        // many query rows per request: the tile kernel (rows copied as stored)
         const bool many_rows = batch->max_q_len >= 32 &&
                                (long long)batch->total_tokens * num_q_heads >= 128ll * kPfRows;
-        if (!force_single && many_rows && prefill_tq4_applicable(layout, batch, num_q_heads))
+        if ((force_tile || (!force && many_rows)) && prefill_tq4_applicable(layout, batch, num_q_heads))
             return launch_prefill_tq4<TQ, TQ::kStorageFormat>(ex, layout, batch, q, out, num_q_heads, gate);
         return launch_rows<TQ, TQ::kStorageFormat>(ex, layout, batch, q, out, num_q_heads, force_single, gate);
     }
@@ -2205,7 +2208,7 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
         // many query rows per request: the tile kernel (FP8 rows have the shape of TQ4 rows)
         const bool many_rows = batch->max_q_len >= 32 &&
                                (long long)batch->total_tokens * num_q_heads >= 128ll * kPfRows;
-        if ((force_single || many_rows) && prefill_tq4_applicable(layout, batch, num_q_heads))
+        if ((force_tile || (!force && many_rows)) && prefill_tq4_applicable(layout, batch, num_q_heads))
             return launch_prefill_tq4<TQ, WARP34_KV_FORMAT_FP8_E4M3>(ex, layout, batch, q, out, num_q_heads, gate);
         if (layout->v_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256)
             return launch_rows<TQ, WARP34_KV_FORMAT_FP8_E4M3, true>(ex, layout, batch, q, out, num_q_heads, force_single, gate);
@@ -2215,7 +2218,7 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
         if (!kv8_geometry_ok(layout, q, out, 272)) return (int)hipErrorNotSupported;
         const bool many_rows = batch->max_q_len >= 32 &&
                                (long long)batch->total_tokens * num_q_heads >= 128ll * kPfRows;
-        if ((force_single || many_rows) && prefill_tq4_applicable(layout, batch, num_q_heads))
+        if ((force_tile || (!force && many_rows)) && prefill_tq4_applicable(layout, batch, num_q_heads))
             return launch_prefill_tq4<TQ, WARP34_KV_FORMAT_Q8_0>(ex, layout, batch, q, out, num_q_heads, gate);
         if (layout->v_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256)
             return launch_rows<TQ, WARP34_KV_FORMAT_Q8_0, true>(ex, layout, batch, q, out, num_q_heads, force_single, gate);
@@ -2396,8 +2399,9 @@ extern "C" int warp34_paged_attention_f16_force_kernel_for_test(
     const int rc = common_checks(ex, layout, batch, q_in, attn_out, num_q_heads);
     if (rc) return rc;
     if (batch->total_tokens <= 0 || num_q_heads <= 0) return 0;
-    (void)use_64q;
-    return attention_entry<F16>(ex, layout, batch, q_in, attn_out, num_q_heads, 1);
+    // the reference's selector picks the 16-row kernel (0) or one of its 64 / 128-row prefill kernels;
+    // here: the decode / verify kernel as a single pass, or the 128-row tile kernel
+    return attention_entry<F16>(ex, layout, batch, q_in, attn_out, num_q_heads, use_64q == 0 ? 1 : 2);
 }
 
 // Scratch that lets a batch split fully, computed the way the launchers compute it.
@@ -2524,10 +2528,11 @@ extern "C" int warp34_paged_attention_bf16_static_scratch(const warp34_exec* ex,
     if (rc) return rc;
     if (num_q_heads <= 0 || batch->total_tokens < 0) return (int)hipErrorInvalidValue;
     if (!batch->total_tokens) return 0;
-    // a batch that would want more scratch than the array holds is refused, not run with fewer chunks
-    const size_t need = scratch_bytes_for(layout->local_kv_heads, batch->total_tokens, batch->num_reqs, num_q_heads,
-                                          batch->max_seq_len, batch->max_q_len);
-    if (need > kStaticScratchBytes) return (int)hipErrorOutOfMemory;
+    // The array serves every batch the way an 8 MiB ex->scratch would: the launchers take fewer
+    // chunks, or leave a pass out, when the records of the full split do not fit.  Refused are only
+    // batches too large for the array to be of any use: not even two records per query row fit.
+    const long long rows = (long long)batch->total_tokens * num_q_heads;
+    if (partial_bytes(rows, 2) > kStaticScratchBytes) return (int)hipErrorOutOfMemory;
     uintptr_t addr = 0;
     const int arc = static_scratch_address(&addr);
     if (arc) return arc;
