@@ -1184,46 +1184,69 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
     wait_vm<0>();  // nothing of this wave may still be on its way into LDS when the areas are reused
 
     // ---- packed tile: column n += its mirror column n + 8 (the low-order share of the weights) ----
+    // Both lanes of a pair end up with sums, and both take part in the stores below: lane n < 8 keeps
+    // the value tiles with even j in the even slots, its mirror lane those with odd j.
     if (pack) {
+        const bool upper = (n & 8) != 0;
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
+            for (int i = 0; i < 4; ++i)
 #pragma unroll
-                for (int k = 0; k < 4; ++k) o_acc[h][j][k] += row_ror8(o_acc[h][j][k]);
+                for (int k = 0; k < 4; ++k) {
+                    const float even = o_acc[h][2 * i][k], odd = o_acc[h][2 * i + 1][k];
+                    const float keep = upper ? odd : even;   // this lane's tile of the pair
+                    const float give = upper ? even : odd;   // what the mirror lane keeps
+                    o_acc[h][2 * i][k] = keep + row_ror8(give);
+                }
     }
 
     // ---- combine the per-lane partial sums of l over the four k-block lanes of a column ------
     l_run = sum_over_rows(l_run);
 
     // ---- merge the waves' states through LDS ---------------------------------------------------
-    // Every wave publishes (m, l); then, for each half of the 16 columns that has a live column,
-    // the waves store their O of those columns, rescaled by 2^(m - m_tot), in their own region, and
-    // waves 0-7 each add the regions of one column up in wave order.  (Two passes because ten
-    // regions of sixteen columns do not fit the LDS; a decode tile has live columns in one half only.)
+    // Every wave publishes (m, l) and its O, as it stands, in its own region -- its own staging area,
+    // which nobody else touches, so the stores need not wait for the other waves -- and after ONE
+    // barrier wave c adds up column c of the eight regions, each weighted by 2^(m_w - m_tot), in wave
+    // order.  A region holds eight columns: a tile with live columns in both halves (more than
+    // eight columns, never a decode step) takes a second pass.
     // Region layout: column stride kMergeColStride dwords; inside a column the four values a lane
     // holds for one MFMA result (rows 4b..4b+3 of (h, j)) are contiguous at ((h*8 + j)*4 + b)*4,
-    // so a lane stores them with one 128-bit write.
+    // so a lane stores them with one 128-bit write and the adding wave reads one 128-bit piece per
+    // lane and region.  The sums reach the element order of the head dimension (lane l: elements
+    // 4 l .. 4 l + 3) through a 1 KB transposition buffer per wave in the idle query operand table.
     constexpr int kColStride = kMergeColStride;
     constexpr int kRegion = 8 * kColStride;
-    float* xbuf = reinterpret_cast<float*>(stage_all);  // the staging areas are idle now; the table stays
-    // [kWaves][16][2], then (m_tot, l_tot)[16]: in an area of its own, a wave publishes its state
-    // while others are still in their loops
+    static_assert(kRegion * 4 == kStageTq4, "a wave's merge region is its own staging area");
+    static_assert(kWaves * 1024 <= kQopBytes, "transposition buffers");
+    float* xbuf = reinterpret_cast<float*>(stage_all);
+    float* tbuf = reinterpret_cast<float*>(qop) + wave * 256;
+    // [kWaves][16][2]: in an area of its own, a wave publishes its state while others are still in their loops
     float* mlbuf = reinterpret_cast<float*>(smem + ml_offset_for(1));
     static_assert(kWaves * kRegion == merge_floats_for(1), "merge layout");
     if (b == 0) {
         mlbuf[(wave * 16 + n) * 2 + 0] = m_run;
         mlbuf[(wave * 16 + n) * 2 + 1] = l_run;
     }
-    __syncthreads();  // every wave is done with the table and with its staging area
-    float m_tot = kNegBig, l_tot = 0.f;
+    auto store_region = [&](int half) {
+        float* c = xbuf + wave * kRegion + (n & 7) * kColStride;
+        if (pack) {  // (half 0) all 64 lanes store: eight tiles each, see above
+            if (col_ok) {
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) m_tot = fmaxf(m_tot, mlbuf[(w * 16 + n) * 2]);
+                for (int h = 0; h < 2; ++h)
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w)
-        l_tot += mlbuf[(w * 16 + n) * 2 + 1] * __builtin_amdgcn_exp2f(mlbuf[(w * 16 + n) * 2] - m_tot);
-    const float wgt = __builtin_amdgcn_exp2f(m_run - m_tot);
-    float* mltot = mlbuf + kWaves * 16 * 2;
+                    for (int i = 0; i < 4; ++i)
+                        *reinterpret_cast<f4*>(c + ((h * 8 + 2 * i + (n >> 3)) * 4 + b) * 4) = o_acc[h][2 * i];
+            }
+        } else if ((n >> 3) == half && col_ok) {  // dead columns are never read back
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) *reinterpret_cast<f4*>(c + ((h * 8 + j) * 4 + b) * 4) = o_acc[h][j];
+        }
+    };
+    const bool live0 = (ok_mask & 0xFFu) != 0u, live1 = (ok_mask >> 8) != 0u;  // the same in every wave
+    store_region(live0 ? 0 : 1);
 
     int merge_slot[4];  // region slot of element 4*lane + k (inverse of tq4_pv_elem)
 #pragma unroll
@@ -1241,37 +1264,44 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
         }
         merge_slot[k] = ((h * 8 + j) * 4 + (r >> 2)) * 4 + (r & 3);
     }
+    __syncthreads();  // every wave is done with the table, and the regions of the first pass are there
 #pragma unroll 1
     for (int half = 0; half < 2; ++half) {
-        if (((ok_mask >> (8 * half)) & 0xFFu) == 0u) continue;  // the same in every wave
-        if (half == 1 && (ok_mask & 0xFFu) != 0u) __syncthreads();  // the first pass has read the regions
-        if ((n >> 3) == half && col_ok) {  // dead columns are never read back
-            float* c = xbuf + wave * kRegion + (n & 7) * kColStride;
-#pragma unroll
-            for (int h = 0; h < 2; ++h)
-#pragma unroll
-                for (int j = 0; j < 8; ++j) *reinterpret_cast<f4*>(c + ((h * 8 + j) * 4 + b) * 4) = o_acc[h][j] * wgt;
-            if (wave == 0 && b == 0) {
-                mltot[n * 2 + 0] = m_tot;
-                mltot[n * 2 + 1] = l_tot;
-            }
+        if (!(half ? live1 : live0)) continue;
+        if (half == 1 && live0) {
+            __syncthreads();  // the first pass has read the regions
+            store_region(1);
+            __syncthreads();
         }
-        __syncthreads();
         const int col = 8 * half + wave;
         if (wave < 8 && ((ok_mask >> col) & 1u)) {
+            // state of the column in the eight waves (the same addresses in every lane)
+            float mw[kWaves], lw[kWaves];
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) {
+                const f2 r = *reinterpret_cast<const f2*>(mlbuf + (w * 16 + col) * 2);
+                mw[w] = r[0];
+                lw[w] = r[1];
+            }
+            float m_col = kNegBig, l_col = 0.f;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) m_col = fmaxf(m_col, mw[w]);
+            f4 tot = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) {
+                const float wgt = __builtin_amdgcn_exp2f(mw[w] - m_col);
+                l_col += lw[w] * wgt;
+                tot += *reinterpret_cast<const f4*>(xbuf + w * kRegion + wave * kColStride + 4 * lane) * wgt;
+            }
+            *reinterpret_cast<f4*>(tbuf + 4 * lane) = tot;
+            // element e = 4*lane + k is value (h, j, row r) with e = tq4_pv_elem(h, j, r); the reads
+            // follow the write of the same wave in LDS order
+            float v[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) v[k] = tbuf[merge_slot[k]];
             const int t = fast_div(col, P.q_group);
             const int a = col - t * P.q_group;
             const size_t row = (size_t)(tok0 + t) * P.num_q_heads + (size_t)(q_head_base + a);
-            float v[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int w = 0; w < kWaves; ++w) {
-                // element e = 4*lane + k is value (h, j, row r) with e = tq4_pv_elem(h, j, r)
-                const float* c = xbuf + w * kRegion + wave * kColStride;
-#pragma unroll
-                for (int k = 0; k < 4; ++k) v[k] += c[merge_slot[k]];
-            }
-            const float m_col = mltot[col * 2 + 0];
-            const float l_col = mltot[col * 2 + 1];
             if (BAL ? item.n_chunks > 1 : P.max_chunks > 1) {
                 // un-normalised, rotated, still carrying the table gain; the merge kernel finishes
                 const size_t prow = BAL ? bal_partial_row(item.slot, (int)gridDim.y, kv_sub, col)
