@@ -676,7 +676,6 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
     // ---- merge of the waves' states (same scheme and region layout as the TQ4 kernel) ----
     constexpr int kColStride = kKv16ColStride;
     constexpr int kRegion = NT * 16 * kColStride;
-    float* xbuf = reinterpret_cast<float*>(smem);
     float* mlbuf = reinterpret_cast<float*>(smem + kv16_ml_offset(NT));
     static_assert(kv16_ml_offset(NT) >= kWaves * kRegion * 4 && kv16_ml_offset(NT) >= kWaves * kKv16Stage,
                   "(m, l) table must not alias live LDS");
@@ -687,40 +686,6 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
             mlbuf[(wave * NT * 16 + nt * 16 + n) * 2 + 1] = l_run[nt];
         }
     }
-    __syncthreads();
-    float m_tot[NT], l_tot[NT];
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        float mt = kNegBig;
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) mt = fmaxf(mt, mlbuf[(w * NT * 16 + nt * 16 + n) * 2]);
-        float lt = 0.f;
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w)
-            lt += mlbuf[(w * NT * 16 + nt * 16 + n) * 2 + 1] *
-                  __builtin_amdgcn_exp2f(mlbuf[(w * NT * 16 + nt * 16 + n) * 2] - mt);
-        m_tot[nt] = mt;
-        l_tot[nt] = lt;
-        const float wgt = __builtin_amdgcn_exp2f(m_run[nt] - mt);
-        float* c = xbuf + wave * kRegion + (nt * 16 + n) * kColStride;
-        if (col_ok[nt]) {
-#pragma unroll
-            for (int h = 0; h < 2; ++h)
-#pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    *reinterpret_cast<f4*>(c + ((h * 8 + j) * 4 + b) * 4) = o_acc[nt][h][j] * wgt;
-        }
-    }
-    float* mltot = mlbuf + kWaves * NT * 16 * 2;
-    if (wave == 0 && b == 0) {
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            mltot[(nt * 16 + n) * 2 + 0] = m_tot[nt];
-            mltot[(nt * 16 + n) * 2 + 1] = l_tot[nt];
-        }
-    }
-    __syncthreads();
-
     // element e = 128 h + 8 r + j sits in slot ((h*8 + j)*4 + (r >> 2))*4 + (r & 3)
     int merge_slot[4];
 #pragma unroll
@@ -729,20 +694,11 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
         const int h = e >> 7, r = (e >> 3) & 15, j = e & 7;
         merge_slot[k] = ((h * 8 + j) * 4 + (r >> 2)) * 4 + (r & 3);
     }
-    for (int col = wave; col < 16 * NT; col += kWaves) {
+    // finishes column `col` from its sums v (element order of the head dimension) and its state
+    auto finish_column = [&](int col, float (&v)[4], float m_col, float l_col) {
         const int t = fast_div(col, P.q_group);
         const int a = col - t * P.q_group;
-        if (!((ok_mask[col >> 4] >> (col & 15)) & 1u)) continue;
         const size_t row = (size_t)(tok0 + t) * P.num_q_heads + (size_t)(q_head_base + a);
-        float v[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) {
-            const float* c = xbuf + w * kRegion + col * kColStride;
-#pragma unroll
-            for (int k = 0; k < 4; ++k) v[k] += c[merge_slot[k]];
-        }
-        const float m_col = mltot[col * 2 + 0];
-        const float l_col = mltot[col * 2 + 1];
         if (BAL ? item.n_chunks > 1 : P.max_chunks > 1) {
             const size_t prow = BAL ? bal_partial_row(item.slot, (int)gridDim.y, kv_sub, col)
                                     : row * P.max_chunks + chunk;
@@ -761,6 +717,49 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
                 for (int k = 0; k < 4; ++k) v[k] = apply_sign(v[k], 4 * lane + k);
             }
             store_out_row<TQ>(P, row, lane, v);
+        }
+    };
+    {
+        static_assert(NT == 1, "the merge below is the one-tile form");
+        // One 16-column tile: a wave's region fits its own staging area, which nobody else touches.
+        // The wave stores its O as it stands, before the barrier; the adding wave weights the eight
+        // regions by 2^(m_w - m_tot), reads one 128-bit piece per lane and region, and brings the
+        // sums into element order through the 1 KB its staging area has left behind the region.
+        static_assert(kRegion * 4 + 1024 <= kKv16Stage, "region and transposition buffer inside the staging area");
+        float* region = reinterpret_cast<float*>(stage);
+        float* tbuf = region + kRegion;
+        if (col_ok[0]) {
+            float* c = region + n * kColStride;
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) *reinterpret_cast<f4*>(c + ((h * 8 + j) * 4 + b) * 4) = o_acc[0][h][j];
+        }
+        __syncthreads();
+        for (int col = wave; col < 16; col += kWaves) {
+            if (!((ok_mask[0] >> col) & 1u)) continue;
+            float mw[kWaves], lw[kWaves];
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) {
+                const f2 r = *reinterpret_cast<const f2*>(mlbuf + (w * 16 + col) * 2);
+                mw[w] = r[0];
+                lw[w] = r[1];
+            }
+            float m_col = kNegBig, l_col = 0.f;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) m_col = fmaxf(m_col, mw[w]);
+            f4 tot = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) {
+                const float wgt = __builtin_amdgcn_exp2f(mw[w] - m_col);
+                l_col += lw[w] * wgt;
+                tot += *reinterpret_cast<const f4*>(smem + w * kKv16Stage + (col * kColStride + 4 * lane) * 4) * wgt;
+            }
+            *reinterpret_cast<f4*>(tbuf + 4 * lane) = tot;
+            float v[4];  // the reads follow the write of the same wave in LDS order
+#pragma unroll
+            for (int k = 0; k < 4; ++k) v[k] = tbuf[merge_slot[k]];
+            finish_column(col, v, m_col, l_col);
         }
     }
 }
