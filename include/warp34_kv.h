@@ -167,8 +167,9 @@ int warp34_kv_cache_write_strided_bf16(const warp34_exec* ex, const warp34_kv_la
  * Output = softmax(sm_scale * q.K^T) V in fp32 accumulation; an empty key range gives zeros.
  * _f16 accepts FP16, TQ4+WHT256, Q8_0 and FP8_E4M3 layouts (the 8-bit ones plain or with
  * WHT256; K and V in the same format); _bf16 accepts BF16 (reference) and, additionally,
- * the TQ4 and 8-bit layouts.  head_dim must be 256, block_size a multiple of 16, and the
- * token stride the row size (512 / 132 / 272 / 264 bytes) with 16-byte aligned slabs.
+ * the TQ4 and 8-bit layouts.  head_dim must be 256 -- or, for the 16-bit layouts, 128
+ * (op_kv_cache.cu:873,1227) --, block_size a multiple of 16, and the token stride the row size
+ * (2 * head_dim / 132 / 272 / 264 bytes) with 16-byte aligned slabs.
  * ------------------------------------------------------------------------------------ */
 int warp34_paged_attention_f16(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
                                const warp34_attention_batch* batch,

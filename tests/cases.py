@@ -6,14 +6,14 @@ from oracle import FMT_TQ4, XF_IDENTITY, XF_WHT256
 
 
 def make_case(fmt, block_size, seq_lens, q_lens, seed, dtype, kv_heads=2, q_heads=8, perm_seed=5,
-              extra_pages=3, xf=None):
+              extra_pages=3, xf=None, head_dim=256):
     """Append seq_len tokens per request through the oracle's write, return everything."""
     if xf is None:
         xf = XF_WHT256 if fmt == FMT_TQ4 else XF_IDENTITY
     pages_per = [(s + block_size - 1) // block_size for s in seq_lens]
     num_pages = sum(pages_per) + extra_pages
     perm = oracle.permutation(num_pages, perm_seed)
-    pool = oracle.HostPool(num_pages, kv_heads, 256, block_size, fmt, xf)
+    pool = oracle.HostPool(num_pages, kv_heads, head_dim, block_size, fmt, xf)
     mb = max(pages_per)
     bt = np.zeros((len(seq_lens), mb), dtype=np.int32)
     at = 0
@@ -24,8 +24,8 @@ def make_case(fmt, block_size, seq_lens, q_lens, seed, dtype, kv_heads=2, q_head
         slots.append(oracle.slot_mapping(bt[r], 0, s, block_size))
         qsl.append(qsl[-1] + s)
     total = qsl[-1]
-    k = oracle.fill_kv_rows(total, kv_heads, 256, seed, dtype, 3)
-    v = oracle.fill_kv_rows(total, kv_heads, 256, seed + 1, dtype, 3)
+    k = oracle.fill_kv_rows(total, kv_heads, head_dim, seed, dtype, 3)
+    v = oracle.fill_kv_rows(total, kv_heads, head_dim, seed + 1, dtype, 3)
     wb = oracle.HostBatch(qsl, seq_lens, bt, context_lens_before=[0] * len(seq_lens),
                           write_slot_mapping=np.concatenate(slots))
     oracle.kv_cache_write(pool, wb, k, v, dtype)
@@ -33,7 +33,7 @@ def make_case(fmt, block_size, seq_lens, q_lens, seed, dtype, kv_heads=2, q_head
     aq = [0]
     for ql in q_lens:
         aq.append(aq[-1] + ql)
-    q = oracle.fill_normal(aq[-1] * q_heads * 256, seed + 2, dtype).reshape(aq[-1], q_heads, 256)
+    q = oracle.fill_normal(aq[-1] * q_heads * head_dim, seed + 2, dtype).reshape(aq[-1], q_heads, head_dim)
     ctx = [s - ql for s, ql in zip(seq_lens, q_lens)]
     return pool, bt, k, v, q, aq, ctx
 

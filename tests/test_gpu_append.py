@@ -17,7 +17,7 @@ pytestmark = pytest.mark.gpu
 
 
 def _run_append(fmt, xf, block_size, n_tokens, in_dtype, seed, kv_heads=2, tmask=None, rmask=None,
-                neg_slots=(), stride=None):
+                neg_slots=(), stride=None, head_dim=256):
     import gpu_harness as G
 
     n_pages = (n_tokens + block_size - 1) // block_size
@@ -26,16 +26,16 @@ def _run_append(fmt, xf, block_size, n_tokens, in_dtype, seed, kv_heads=2, tmask
     slots = oracle.slot_mapping(bt[0], 0, n_tokens, block_size)
     for i in neg_slots:
         slots[i] = -1
-    k = oracle.fill_kv_rows(n_tokens, kv_heads, 256, seed, in_dtype, 3)
-    v = oracle.fill_kv_rows(n_tokens, kv_heads, 256, seed + 1, in_dtype, 3)
+    k = oracle.fill_kv_rows(n_tokens, kv_heads, head_dim, seed, in_dtype, 3)
+    v = oracle.fill_kv_rows(n_tokens, kv_heads, head_dim, seed + 1, in_dtype, 3)
     if stride is not None:
-        pad = stride - kv_heads * 256
+        pad = stride - kv_heads * head_dim
         filler = oracle.fill_normal(n_tokens * pad, seed + 2, in_dtype).reshape(n_tokens, pad)
         k_src = np.concatenate([k.reshape(n_tokens, -1), filler], axis=1)
         v_src = np.concatenate([v.reshape(n_tokens, -1), filler[:, ::-1]], axis=1)
     else:
         k_src, v_src = k, v
-    hpool = oracle.HostPool(n_pages + 2, kv_heads, 256, block_size, fmt, xf)
+    hpool = oracle.HostPool(n_pages + 2, kv_heads, head_dim, block_size, fmt, xf)
     hb = oracle.HostBatch([0, n_tokens], [n_tokens], bt, context_lens_before=[0], write_slot_mapping=slots,
                           valid_token_mask=tmask, valid_req_mask=rmask)
     oracle.kv_cache_write(hpool, hb, k_src, v_src, in_dtype, stride, stride)
@@ -105,6 +105,15 @@ def test_append_masks_and_negative_slots_write_nothing():
 @pytest.mark.parametrize("fmt,in_dtype", [(FMT_FP16, DT_F16), (FMT_BF16, DT_BF16), (FMT_BF16, DT_F16)])
 def test_16bit_formats_and_strided_source(fmt, in_dtype):
     hpool, gk, gv = _run_append(fmt, XF_IDENTITY, 16, 50, in_dtype, seed=7, stride=2 * 256 + 64)
+    assert gk.tobytes() == hpool.k.tobytes() and gv.tobytes() == hpool.v.tobytes()
+
+
+@pytest.mark.parametrize("fmt,in_dtype", [(FMT_FP16, DT_F16), (FMT_BF16, DT_BF16), (FMT_BF16, DT_F16)])
+def test_16bit_formats_at_head_dim_128(fmt, in_dtype):
+    """The 16-bit row formats exist at every head dimension up to 256 (ops/op_kv_cache.cu:860-865)."""
+    hpool, gk, gv = _run_append(fmt, XF_IDENTITY, 16, 50, in_dtype, seed=8, head_dim=128)
+    assert gk.tobytes() == hpool.k.tobytes() and gv.tobytes() == hpool.v.tobytes()
+    hpool, gk, gv = _run_append(fmt, XF_IDENTITY, 64, 130, in_dtype, seed=9, stride=2 * 128 + 24, head_dim=128)
     assert gk.tobytes() == hpool.k.tobytes() and gv.tobytes() == hpool.v.tobytes()
 
 

@@ -30,11 +30,11 @@ def _dev_pool(pool):
 
 
 def _check(fmt, dtype, block_size, seq_lens, q_lens, seed, scratch=SCRATCH, q_heads=8, kv_heads=2,
-           mask_mode=0, window=0, ctx_null=False, xf=None, **kw):
+           mask_mode=0, window=0, ctx_null=False, xf=None, head_dim=256, **kw):
     import gpu_harness as G
 
     pool, bt, k, v, q, aq, ctx = make_case(fmt, block_size, seq_lens, q_lens, seed, dtype, kv_heads=kv_heads,
-                                           q_heads=q_heads, xf=xf)
+                                           q_heads=q_heads, xf=xf, head_dim=head_dim)
     hb = oracle.HostBatch(aq, seq_lens, bt, context_lens_before=None if ctx_null else ctx, mask_mode=mask_mode,
                           sliding_window=window)
     want = oracle.paged_attention(pool, hb, q, dtype, q_heads, n_threads=4)
@@ -211,6 +211,55 @@ def test_kv16_verify_multi_token_causal(fmt, dtype, q_lens):
 @pytest.mark.parametrize("mask_mode,window", [(0, 40), (1, 0), (1, 100), (0, 5)])
 def test_kv16_windows(mask_mode, window):
     _check(FMT_BF16, DT_BF16, 16, [333, 90], [3, 2], 151, mask_mode=mask_mode, window=window, ctx_null=True)
+
+
+# ---- head dimension 128 (16-bit pages only, ops/op_kv_cache.cu:873,1227) ----
+
+@pytest.mark.parametrize("fmt,dtype", KV16)
+@pytest.mark.parametrize("block_size", [16, 64])
+def test_kv16_head_dim_128_decode(fmt, dtype, block_size):
+    _check(fmt, dtype, block_size, [70, 33, 129, 1, 32], [1, 1, 1, 1, 1], 181, head_dim=128)
+
+
+@pytest.mark.parametrize("fmt,dtype", KV16)
+@pytest.mark.parametrize("scratch", [0, SCRATCH])
+def test_kv16_head_dim_128_decode_gqa8_long(fmt, dtype, scratch):
+    """Split-K (partial records keep their 256-float stride) and the single pass."""
+    _check(fmt, dtype, 64, [5000], [1], 182, scratch=scratch, q_heads=16, head_dim=128)
+    _check(fmt, dtype, 16, [20000, 777], [1, 1], 183, scratch=scratch, q_heads=16, head_dim=128)
+
+
+@pytest.mark.parametrize("fmt,dtype", KV16)
+@pytest.mark.parametrize("q_lens", [[4, 4], [2, 3], [16], [200]])
+def test_kv16_head_dim_128_verify_and_prefill(fmt, dtype, q_lens):
+    """Several query tokens per request, up to a prefill chunk: every shape runs the decode / verify kernel."""
+    seq = [300 + 7 * i for i in range(len(q_lens))]
+    _check(fmt, dtype, 64, seq, q_lens, 184, q_heads=16, head_dim=128)
+    _check(fmt, dtype, 16, seq, q_lens, 185, q_heads=8, scratch=0, head_dim=128)
+
+
+@pytest.mark.parametrize("mask_mode,window", [(0, 40), (1, 0), (1, 100), (0, 5)])
+def test_kv16_head_dim_128_windows(mask_mode, window):
+    _check(FMT_BF16, DT_BF16, 16, [333, 90], [3, 2], 186, mask_mode=mask_mode, window=window, ctx_null=True, head_dim=128)
+
+
+def test_kv16_head_dim_128_gqa_shapes():
+    """One and four q heads per kv head, and more than sixteen (two q subgroups)."""
+    _check(FMT_BF16, DT_BF16, 16, [90, 41], [1, 2], 187, q_heads=2, kv_heads=2, head_dim=128)
+    _check(FMT_BF16, DT_BF16, 16, [90, 41], [1, 2], 188, q_heads=4, kv_heads=1, head_dim=128)
+    _check(FMT_FP16, DT_F16, 32, [150], [3], 189, q_heads=32, kv_heads=1, head_dim=128)
+
+
+def test_kv16_head_dim_128_8bit_and_tq4_pages_are_refused():
+    """Only 16-bit rows exist at head dimension 128: the other formats answer "not supported"."""
+    import gpu_harness as G
+
+    pool, bt, k, v, q, aq, ctx = make_case(FMT_BF16, 16, [40], [1], 190, DT_BF16, head_dim=128)
+    hb = oracle.HostBatch(aq, [40], bt, context_lens_before=ctx)
+    dpool = _dev_pool(pool)
+    for fmt in (FMT_TQ4, FMT_FP8, FMT_Q8_0):
+        rc, got, _ = G.dev_attention(dpool, hb, q, DT_BF16, 8, layout=dpool.layout(fmt))
+        assert rc == 801 and (got == 0x5500).all()
 
 
 def test_kv16_unwritten_pool_bytes_do_not_leak():

@@ -25,7 +25,7 @@ def gather_rows(pool, which, table, kv_head, n):
     """Independent gather + dequant (numpy) of logical rows 0..n-1 -> fp64 [n, 256] in the
     ORIGINAL (un-rotated) domain."""
     slab = pool.k if which == "k" else pool.v
-    out = np.empty((n, 256))
+    out = np.empty((n, pool.head_dim))
     c = oracle.centroids().astype(np.float64)
     s = oracle.signs().astype(np.float64)
     for pos in range(n):
@@ -47,7 +47,7 @@ def gather_rows(pool, which, table, kv_head, n):
 
 def brute(qf, K, V, lo, hi, scale):
     if hi < lo:
-        return np.zeros(256)
+        return np.zeros(V.shape[1])
     sc = (K[lo:hi + 1] @ qf) * scale
     p = np.exp(sc - sc.max())
     return (p[:, None] * V[lo:hi + 1]).sum(0) / p.sum()
@@ -60,6 +60,26 @@ def test_attention_matches_bruteforce(fmt, dtype, block_size):
     pool, bt, k, v, q, aq, ctx = make_case(fmt, block_size, seq_lens, q_lens, 100 + block_size, dtype)
     batch = oracle.HostBatch(aq, seq_lens, bt, context_lens_before=ctx)
     out = oracle.paged_attention(pool, batch, q, dtype, 8)
+    qf = oracle.bits_to_f32(q, dtype).astype(np.float64)
+    for r in range(3):
+        for h in range(2):
+            K = gather_rows(pool, "k", bt[r], h, seq_lens[r])
+            V = gather_rows(pool, "v", bt[r], h, seq_lens[r])
+            for t in range(q_lens[r]):
+                tok = aq[r] + t
+                for a in range(4):
+                    want = brute(qf[tok, 4 * h + a], K, V, 0, ctx[r] + t, 0.0625)
+                    assert np.max(np.abs(out[tok, 4 * h + a] - want)) < 2e-5 * max(1.0, np.max(np.abs(want)))
+
+
+@pytest.mark.parametrize("fmt,dtype", [(FMT_FP16, DT_F16), (FMT_BF16, DT_BF16)])
+def test_attention_matches_bruteforce_at_head_dim_128(fmt, dtype):
+    """16-bit pages at the reference's other head dimension (ops/op_kv_cache.cu:1227)."""
+    seq_lens, q_lens = [70, 33, 129], [1, 4, 3]
+    pool, bt, k, v, q, aq, ctx = make_case(fmt, 16, seq_lens, q_lens, 117, dtype, head_dim=128)
+    batch = oracle.HostBatch(aq, seq_lens, bt, context_lens_before=ctx)
+    out = oracle.paged_attention(pool, batch, q, dtype, 8)
+    assert out.shape == (8, 8, 128)
     qf = oracle.bits_to_f32(q, dtype).astype(np.float64)
     for r in range(3):
         for h in range(2):

@@ -125,13 +125,15 @@ struct AttnParams {
 // (the gated full-attention layers, model/forward.rs:1192-1211) the stored value is the attention
 // output rounded to its 16-bit type and then passed through the gate operator's arithmetic
 // (ops/op_norms_rope_act.cu:742-759), so it has the bits of the two calls in sequence.
-template <typename TQ>
+// HD: the head dimension (lanes beyond a 128-element row store nothing).
+template <typename TQ, int HD = kHeadDim>
 __device__ __forceinline__ void store_out_row(const AttnParams& P, size_t row, int lane, const float (&o)[4]) {
+    if (HD < 256 && 4 * lane >= HD) return;
     uint16_t h[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k) h[k] = TQ::from_f32(o[k]);
     if (P.gate != nullptr) {
-        const uint2 g = *reinterpret_cast<const uint2*>(P.gate + row * kHeadDim + 4 * lane);
+        const uint2 g = *reinterpret_cast<const uint2*>(P.gate + row * HD + 4 * lane);
         const uint16_t gb[4] = {(uint16_t)g.x, (uint16_t)(g.x >> 16), (uint16_t)g.y, (uint16_t)(g.y >> 16)};
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
@@ -141,7 +143,7 @@ __device__ __forceinline__ void store_out_row(const AttnParams& P, size_t row, i
     uint2 ob;
     ob.x = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
     ob.y = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
-    *reinterpret_cast<uint2*>(P.out + row * kHeadDim + 4 * lane) = ob;
+    *reinterpret_cast<uint2*>(P.out + row * HD + 4 * lane) = ob;
 }
 
 
@@ -1533,7 +1535,7 @@ __global__ __launch_bounds__(1024) void balanced_merge_kernel(const AttnParams P
 // Everything the row needs (validity, chunk records, accumulators) is requested in ONE memory
 // round trip: records and accumulators of all max_chunks slots are loaded speculatively and
 // the slots beyond the row's chunk count are discarded with selects.
-template <typename TQ, bool SP = false>
+template <typename TQ, bool SP = false, int HD = kHeadDim>
 __global__ __launch_bounds__(1024) void split_merge_kernel(const float* part_acc_in, const float* part_ml_in,
                                                            int max_chunks_in, const AttnParams P,
                                                            float out_scale, int rotate) {
@@ -1561,7 +1563,9 @@ __global__ __launch_bounds__(1024) void split_merge_kernel(const float* part_acc
     for (int k = 0; k < kMergeMaxPerGroup; ++k) {
         const int s = grp + k * kMergeGroups;
         a[k] = f4{0.f, 0.f, 0.f, 0.f};
-        if (s < max_chunks_in) a[k] = *reinterpret_cast<const f4*>(acc + (size_t)s * kHeadDim + 4 * lane);
+        // (records keep a 256-float stride at every head dimension; lanes beyond the row load nothing)
+        if (s < max_chunks_in && (HD == 256 || 4 * lane < HD))
+            a[k] = *reinterpret_cast<const f4*>(acc + (size_t)s * kHeadDim + 4 * lane);
     }
     // row validity (wave 0): token mask and owning request, first match wins
     if (grp == 0) {
@@ -1639,7 +1643,7 @@ __global__ __launch_bounds__(1024) void split_merge_kernel(const float* part_acc
 #pragma unroll
         for (int k = 0; k < 4; ++k) o[k] = apply_sign(o[k], 4 * lane + k);
     }
-    store_out_row<TQ>(P, (size_t)row, lane, o);
+    store_out_row<TQ, HD>(P, (size_t)row, lane, o);
 }
 
 }  // namespace w34
@@ -1982,7 +1986,7 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
 }
 
 // VRES: value rows stored rotated in an 8-bit format (residual operand, see rows_tile)
-template <typename TQ, int KVF, bool VRES = false>
+template <typename TQ, int KVF, bool VRES = false, int HD = kHeadDim>
 static int launch_rows(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
                        const warp34_attention_batch* batch, const void* q, void* out, int num_q_heads,
                        int force_single, const void* gate) {
@@ -2038,7 +2042,7 @@ static int launch_rows(const warp34_exec* ex, const warp34_kv_layer_layout* layo
     const dim3 grid((unsigned)grid_x, (unsigned)kv_subs, (unsigned)grid_z);
     hipStream_t stream = (hipStream_t)ex->stream;
     int rc;
-    if (balanced_decode_applicable(ex, batch, P.tiles_by_request, force_single)) {
+    if (HD == kHeadDim && balanced_decode_applicable(ex, batch, P.tiles_by_request, force_single)) {
         const int groups = balanced_groups(P.q_subgroups);
         const size_t prows = bal_partial_row(groups + batch->num_reqs, kv_subs, 0, 0);
         if (partial_bytes((long long)prows, 1) + (size_t)batch->total_tokens * 16 <= ex->scratch_size) {
@@ -2058,13 +2062,13 @@ static int launch_rows(const warp34_exec* ex, const warp34_kv_layer_layout* layo
             return (int)hipGetLastError();
         }
     }
-    rc = ensure_dynamic_lds(paged_attn_rows_kernel<TQ, 1, KVF, VRES>, kv16_smem_bytes(1));
+    rc = ensure_dynamic_lds(paged_attn_rows_kernel<TQ, 1, KVF, VRES, HD>, kv16_smem_bytes(1));
     if (rc) return rc;
-    hipLaunchKernelGGL((paged_attn_rows_kernel<TQ, 1, KVF, VRES>), grid, dim3(kKv16Waves * 64), kv16_smem_bytes(1), stream, P);
+    hipLaunchKernelGGL((paged_attn_rows_kernel<TQ, 1, KVF, VRES, HD>), grid, dim3(kKv16Waves * 64), kv16_smem_bytes(1), stream, P);
     rc = (int)hipGetLastError();
     if (rc) return rc;
     if (P.max_chunks > 1) {
-        hipLaunchKernelGGL((split_merge_kernel<TQ>), dim3((unsigned)rows), dim3(1024), 0, stream,
+        hipLaunchKernelGGL((split_merge_kernel<TQ, false, HD>), dim3((unsigned)rows), dim3(1024), 0, stream,
                            (const float*)P.part_acc, (const float*)P.part_ml, P.max_chunks, P, 1.0f, P.rot_out);
         rc = (int)hipGetLastError();
     }
@@ -2146,13 +2150,14 @@ static int launch_prefill_tq4(const warp34_exec* ex, const warp34_kv_layer_layou
 }
 
 static bool is_kv16(const warp34_kv_layer_layout* l, int format) {
-    return l->head_dim == 256 && l->k_format == format && l->v_format == format &&
+    return (l->head_dim == 256 || l->head_dim == 128) && l->k_format == format && l->v_format == format &&
            l->k_transform == WARP34_KV_TRANSFORM_IDENTITY && l->v_transform == WARP34_KV_TRANSFORM_IDENTITY;
 }
 
 static bool kv16_geometry_ok(const warp34_kv_layer_layout* l, const void* q, const void* out) {
-    return l->block_size > 0 && (l->block_size % 16) == 0 && l->k_token_stride_bytes == 512 &&
-           l->v_token_stride_bytes == 512 && (l->k_base & 15u) == 0 && (l->v_base & 15u) == 0 &&
+    const unsigned row_bytes = 2u * (unsigned)l->head_dim;
+    return l->block_size > 0 && (l->block_size % 16) == 0 && l->k_token_stride_bytes == row_bytes &&
+           l->v_token_stride_bytes == row_bytes && (l->k_base & 15u) == 0 && (l->v_base & 15u) == 0 &&
            (l->k_page_stride_bytes & 15u) == 0 && (l->k_head_stride_bytes & 15u) == 0 &&
            (l->v_page_stride_bytes & 15u) == 0 && (l->v_head_stride_bytes & 15u) == 0 &&
            (((uintptr_t)q) & 15u) == 0 && (((uintptr_t)out) & 7u) == 0;
@@ -2228,6 +2233,9 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
         // many query rows per request: the tile kernel (rows copied as stored)
         const bool many_rows = batch->max_q_len >= 32 &&
                                (long long)batch->total_tokens * num_q_heads >= 128ll * kPfRows;
+        // head dimension 128 (op_kv_cache.cu:1227): the decode / verify kernel serves every batch shape
+        if (layout->head_dim == 128)
+            return launch_rows<TQ, TQ::kStorageFormat, false, 128>(ex, layout, batch, q, out, num_q_heads, force_single, gate);
         if ((force_tile || (!force && many_rows)) && prefill_tq4_applicable(layout, batch, num_q_heads))
             return launch_prefill_tq4<TQ, TQ::kStorageFormat>(ex, layout, batch, q, out, num_q_heads, gate);
         return launch_rows<TQ, TQ::kStorageFormat>(ex, layout, batch, q, out, num_q_heads, force_single, gate);

@@ -102,18 +102,25 @@ __device__ __forceinline__ f4 mfma_x16(u2v a, u2v b, f4 c) {
 // of a rotated row with large entries holds few distinct codes, so part of the fp16 rounding of
 // d * code is common to the block, and the inverse rotation of the finished row would gather
 // that common part into a single channel.
-template <typename TQ, int NT, int KVF, bool BAL, bool VRES = false, bool STREAM = BAL>
+// HD: the head dimension, 256 or -- 16-bit rows only (op_kv_cache.cu:1227) -- 128.  At 128 a row is
+// one 128-element half: four QK operands instead of eight, eight value tiles instead of sixteen,
+// and lanes 0-31 carry a finished row.  The split-K partial records keep their 256-float stride.
+template <typename TQ, int NT, int KVF, bool BAL, bool VRES = false, bool STREAM = BAL, int HD = kHeadDim>
 __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, const BalItem& item) {
     static_assert(!VRES || KVF == WARP34_KV_FORMAT_FP8_E4M3 || KVF == WARP34_KV_FORMAT_Q8_0, "residual operand: 8-bit rows");
     constexpr bool K8 = KVF == WARP34_KV_FORMAT_FP8_E4M3 || KVF == WARP34_KV_FORMAT_Q8_0;
+    static_assert(HD == 256 || (HD == 128 && !K8), "head dimension 128: 16-bit rows only");
+    constexpr int kM = HD / 32;   // QK operands (32 elements each) per row
+    constexpr int kH = HD / 128;  // 128-element halves of a row
     constexpr bool FP8 = KVF == WARP34_KV_FORMAT_FP8_E4M3;
     static_assert(K8 || KVF == TQ::kStorageFormat, "16-bit pages are read in the query type");
     constexpr bool IS_BF16 = !K8 && TQ::kStorageFormat == WARP34_KV_FORMAT_BF16;
     constexpr bool Q_BF16 = TQ::kStorageFormat == WARP34_KV_FORMAT_BF16;
     constexpr int kWaves = kKv16Waves;
-    constexpr int kRowStride = K8 ? kKv8RowStride : kKv16RowStride;    // LDS row stride of the key rows
-    constexpr int kVRowStride = K8 ? kKv8RowStride : kKv16VRowStride;  // ... of the value rows
-    constexpr int kRowBytes = K8 ? (FP8 ? 264 : 272) : 512;          // row in memory
+    // LDS row strides (16-bit rows of 256 bytes: the row plus 32 / 64 bytes, the same bank pattern as 544 / 576)
+    constexpr int kRowStride = K8 ? kKv8RowStride : (HD == 256 ? kKv16RowStride : 2 * HD + 32);    // key rows
+    constexpr int kVRowStride = K8 ? kKv8RowStride : (HD == 256 ? kKv16VRowStride : 2 * HD + 64);  // value rows
+    constexpr int kRowBytes = K8 ? (FP8 ? 264 : 272) : 2 * HD;       // row in memory
 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
@@ -135,7 +142,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
     // corrected after it.
     const int tok_guess = BAL ? item.rq_start
                               : min(P.tiles_by_request ? tile_z : tile_z * P.tok_tile, B.total_tokens - 1);
-    u4 bq[NT][8];
+    u4 bq[NT][kM];
     auto load_q = [&](int tokbase) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
@@ -143,9 +150,9 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
             const int t = fast_div(col, P.q_group);
             const int a = col - t * P.q_group;
             const int tok = min(tokbase + t, B.total_tokens - 1);
-            const uint16_t* qrow = P.q + ((size_t)tok * P.num_q_heads + (size_t)(q_head_base + a)) * kHeadDim;
+            const uint16_t* qrow = P.q + ((size_t)tok * P.num_q_heads + (size_t)(q_head_base + a)) * HD;
 #pragma unroll
-            for (int m = 0; m < 8; ++m) bq[nt][m] = *reinterpret_cast<const u4*>(qrow + 32 * m + 8 * b);
+            for (int m = 0; m < kM; ++m) bq[nt][m] = *reinterpret_cast<const u4*>(qrow + 32 * m + 8 * b);
         }
     };
     // Rotated K rows: the query rows go through sign + WHT256 first (one row per wave at a time,
@@ -153,6 +160,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
     // back in MFMA layout.
     constexpr int kQStride = 264;  // halves
     auto load_q_rotated = [&](int tokbase) {
+        if constexpr (HD != 256) return;
         _Float16* qlds = reinterpret_cast<_Float16*>(smem);
         for (int col = wave; col < 16 * NT; col += kWaves) {
             const int t = fast_div(col, P.q_group);
@@ -174,7 +182,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-            for (int m = 0; m < 8; ++m)
+            for (int m = 0; m < kM; ++m)
                 bq[nt][m] = *reinterpret_cast<const u4*>(qlds + (nt * 16 + n) * kQStride + 32 * m + 8 * b);
         __syncthreads();  // the staging area is reused by the K/V rows
     };
@@ -214,7 +222,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                for (int m = 0; m < 8; ++m)
+                for (int m = 0; m < kM; ++m)
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
                         const uint32_t w = bq[nt][m][k];
@@ -274,7 +282,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
                 }
             } else {
 #pragma unroll
-                for (int m = 0; m < 8; ++m) bq[nt][m] = u4{0u, 0u, 0u, 0u};
+                for (int m = 0; m < kM; ++m) bq[nt][m] = u4{0u, 0u, 0u, 0u};
             }
             ok_mask[nt] = (uint32_t)(__ballot(ok) & 0xFFFFull);
         }
@@ -346,8 +354,8 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
     // A half = 16 consecutive tokens: 16 K rows and 16 V rows, each run contiguous inside one
     // page (8 KiB of 16-bit rows, 4224 B of FP8 rows, 4352 B of Q8_0 rows).  It is fetched as
     // 16-byte pieces c = lane + 64 i.
-    constexpr int kPieces = 16 * kRowBytes / 16;        // 512, 264 or 272
-    constexpr int kLoads = (kPieces + 63) / 64;         // 8 or 5
+    constexpr int kPieces = 16 * kRowBytes / 16;        // 512, 264 or 272 (256 at head dimension 128)
+    constexpr int kLoads = (kPieces + 63) / 64;         // 8 or 5 (4)
     u4 pf[2 * kLoads];
     auto issue_half = [&](int hidx) {  // hidx = 2 * unit + half
         const int pos = hidx * 16;
@@ -425,14 +433,14 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
         }
     };
 
-    f4 o_acc[NT][2][8];
+    f4 o_acc[NT][kH][8];
     float m_run[NT], l_run[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         m_run[nt] = kNegBig;
         l_run[nt] = 0.f;
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
+        for (int h = 0; h < kH; ++h)
 #pragma unroll
             for (int j = 0; j < 8; ++j) o_acc[nt][h][j] = f4{0.f, 0.f, 0.f, 0.f};
     }
@@ -446,9 +454,9 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) s_acc[nt] = f4{0.f, 0.f, 0.f, 0.f};
         // V operands of the 16 P V MFMAs: a_v[h][j] = element 128 h + 8 n + j of tokens 4b..4b+3
-        u2v a_v[2][8];
+        u2v a_v[kH][8];
         u2v a_vr[VRES ? 2 : 1][VRES ? 8 : 1];  // residuals of a_v
-        if constexpr (K8) {
+        if constexpr (K8 && HD == 256) {
             // Codes of row n, elements 32 m + 8 b .. + 7, widened to fp16; one partial score per
             // scale block (FP8: 2 blocks of 128 = m / 4; Q8_0: 4 blocks of 64 = m / 2), combined
             // with the fp32 scales of this lane's 4 tokens.
@@ -523,19 +531,19 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
                 }
             }
         } else {
-            u4 ka[8];
+            u4 ka[kM];
 #pragma unroll
-            for (int m = 0; m < 8; ++m)
+            for (int m = 0; m < kM; ++m)
                 ka[m] = *reinterpret_cast<const u4*>(k_rows + n * kRowStride + 64 * m + 16 * b);
 #pragma unroll
-            for (int m = 0; m < 8; ++m)
+            for (int m = 0; m < kM; ++m)
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) s_acc[nt] = mfma_x32<IS_BF16>(ka[m], bq[nt][m], s_acc[nt]);
 
             // V slices of this lane's 4 tokens (rows 4b..4b+3), both halves of the head dim; the
             // 4x8 block of 16-bit values is transposed in registers
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
+            for (int h = 0; h < kH; ++h) {
                 u4 vr[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
@@ -584,7 +592,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
             l_run[nt] = l_run[nt] * alpha + psum;
             if (__ballot(alpha != 1.0f) != 0ull) {
 #pragma unroll
-                for (int h = 0; h < 2; ++h)
+                for (int h = 0; h < kH; ++h)
 #pragma unroll
                     for (int j = 0; j < 8; ++j) o_acc[nt][h][j] *= alpha;
             }
@@ -605,7 +613,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
 
         // ---- O^T += V^T P^T: row r = n of MFMA (h, j) is head dimension 128 h + 8 n + j ----
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
+        for (int h = 0; h < kH; ++h) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const u2v a = a_v[h][j];
@@ -650,7 +658,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int m = 0; m < 8; ++m)
+        for (int m = 0; m < kM; ++m)
             asm volatile("" ::"v"(bq[nt][m][0]), "v"(bq[nt][m][1]), "v"(bq[nt][m][2]), "v"(bq[nt][m][3]));
     issue_half(hidx);
     if (simple) column_info(false);
@@ -690,7 +698,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
     int merge_slot[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        const int e = 4 * lane + k;
+        const int e = (4 * lane + k) & (HD - 1);  // (lanes beyond the row repeat its start and store nothing)
         const int h = e >> 7, r = (e >> 3) & 15, j = e & 7;
         merge_slot[k] = ((h * 8 + j) * 4 + (r >> 2)) * 4 + (r & 3);
     }
@@ -703,7 +711,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
             const size_t prow = BAL ? bal_partial_row(item.slot, (int)gridDim.y, kv_sub, col)
                                     : row * P.max_chunks + chunk;
             float* dst = P.part_acc + prow * kHeadDim;
-            *reinterpret_cast<f4*>(dst + 4 * lane) = f4{v[0], v[1], v[2], v[3]};
+            if (4 * lane < HD) *reinterpret_cast<f4*>(dst + 4 * lane) = f4{v[0], v[1], v[2], v[3]};
             if (lane == 0) {
                 *reinterpret_cast<f4*>(P.part_ml + prow * 4) = f4{m_col, l_col, (float)g.n_chunks, 0.f};
             }
@@ -716,7 +724,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
 #pragma unroll
                 for (int k = 0; k < 4; ++k) v[k] = apply_sign(v[k], 4 * lane + k);
             }
-            store_out_row<TQ>(P, row, lane, v);
+            store_out_row<TQ, HD>(P, row, lane, v);
         }
     };
     {
@@ -731,7 +739,7 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
         if (col_ok[0]) {
             float* c = region + n * kColStride;
 #pragma unroll
-            for (int h = 0; h < 2; ++h)
+            for (int h = 0; h < kH; ++h)
 #pragma unroll
                 for (int j = 0; j < 8; ++j) *reinterpret_cast<f4*>(c + ((h * 8 + j) * 4 + b) * 4) = o_acc[0][h][j];
         }
@@ -753,7 +761,8 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
             for (int w = 0; w < kWaves; ++w) {
                 const float wgt = __builtin_amdgcn_exp2f(mw[w] - m_col);
                 l_col += lw[w] * wgt;
-                tot += *reinterpret_cast<const f4*>(smem + w * kKv16Stage + (col * kColStride + 4 * lane) * 4) * wgt;
+                // (head dimension 128: the upper lanes read what the lower ones read and drop it)
+                tot += *reinterpret_cast<const f4*>(smem + w * kKv16Stage + (col * kColStride + ((4 * lane) & (HD - 1))) * 4) * wgt;
             }
             *reinterpret_cast<f4*>(tbuf + 4 * lane) = tot;
             float v[4];  // the reads follow the write of the same wave in LDS order
@@ -764,15 +773,15 @@ __device__ __forceinline__ void rows_tile(const AttnParams& P, uint8_t* smem, co
     }
 }
 
-template <typename TQ, int NT, int KVF, bool VRES>
+template <typename TQ, int NT, int KVF, bool VRES, int HD = kHeadDim>
 __global__ __launch_bounds__(kKv16Waves * 64, 1) void paged_attn_rows_kernel(const AttnParams P) {
     extern __shared__ __align__(16) uint8_t smem[];
     // (one body per kind of load: a branch around the loads themselves keeps the compiler from
     // scheduling them freely and loses what the hint gains)
     if (P.tiles_by_request != 0 && P.q_subgroups == 1) {  // uniform for the grid
-        rows_tile<TQ, NT, KVF, false, VRES, true>(P, smem, BalItem{});
+        rows_tile<TQ, NT, KVF, false, VRES, true, HD>(P, smem, BalItem{});
     } else {
-        rows_tile<TQ, NT, KVF, false, VRES, false>(P, smem, BalItem{});
+        rows_tile<TQ, NT, KVF, false, VRES, false, HD>(P, smem, BalItem{});
     }
 }
 
