@@ -131,10 +131,12 @@ _Static_assert(sizeof(warp34_attention_batch) == 96, "warp34_attention_batch ABI
  * t*row_stride + h*head_dim.  Row strides are in ELEMENTS and must be
  * >= local_kv_heads*head_dim.  Destination row:
  *   base + (slot / block_size)*page_stride + head*head_stride + (slot % block_size)*token_stride.
- * Formats built: FP16, BF16 (converted from fp16), TQ4 (head_dim 256 + WHT256 transform),
- * Q8_0 and FP8_E4M3 (head_dim 256, identity or WHT256 transform, rows 4-byte aligned).
+ * Formats built: FP16, BF16 (converted from fp16), TQ4 (rotated rows at head_dim 256 with the
+ * WHT256 transform; every other TQ4 layout at head_dim 128 or 256 is the plain block quantiser,
+ * one 66-byte block per 128 elements, op_kv_cache.cu:219-264), Q8_0 and FP8_E4M3 (head_dim 256,
+ * identity or WHT256 transform, rows 4-byte aligned).
  * TQ4, Q8_0 and FP8 rows are bit-exact with the declared-numerics CPU restatement of
- * op_kv_cache.cu:32-218.
+ * op_kv_cache.cu:32-264.
  * ------------------------------------------------------------------------------------ */
 int warp34_kv_cache_write(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
                           const warp34_attention_batch* batch,
@@ -145,9 +147,9 @@ int warp34_kv_cache_write_strided(const warp34_exec* ex, const warp34_kv_layer_l
                                   int k_row_stride, int v_row_stride);       /* warp34_cuda.h:356-359 */
 
 /* bf16 source rows (replaces op_kv_cache.cu:798-824,1172-1190).  The reference accepts
- * only BF16-format identity layouts here; this library additionally accepts TQ4+WHT256,
- * Q8_0 and FP8_E4M3 layouts at head_dim 256 (bf16 -> fp32 is exact, the encode is the
- * same arithmetic). */
+ * only BF16-format identity layouts here; this library additionally accepts the TQ4 layouts
+ * and, at head_dim 256, Q8_0 and FP8_E4M3 (bf16 -> fp32 is exact, the encode is the same
+ * arithmetic). */
 int warp34_kv_cache_write_bf16(const warp34_exec* ex, const warp34_kv_layer_layout* layout,
                                const warp34_attention_batch* batch,
                                const void* k_in, const void* v_in);          /* warp34_cuda.h:362-363 */
@@ -165,8 +167,9 @@ int warp34_kv_cache_write_strided_bf16(const warp34_exec* ex, const warp34_kv_la
  *   max_kv = (mask_mode == NONCAUSAL_WINDOW ? seq_after-1 : ctx_before + q_off), clamped to seq_after-1
  *   min_kv = sliding_window > 0 ? max(0, ctx_before + q_off - sliding_window + 1) : 0
  * Output = softmax(sm_scale * q.K^T) V in fp32 accumulation; an empty key range gives zeros.
- * _f16 accepts FP16, TQ4+WHT256, Q8_0 and FP8_E4M3 layouts (the 8-bit ones plain or with
- * WHT256; K and V in the same format); _bf16 accepts BF16 (reference) and, additionally,
+ * _f16 accepts FP16, TQ4, Q8_0 and FP8_E4M3 layouts (TQ4 and the 8-bit ones with each slab
+ * plain or WHT256, op_paged_attn.cu:347,570; K and V in the same format); _bf16 accepts BF16
+ * (reference) and, additionally,
  * the TQ4 and 8-bit layouts.  head_dim must be 256 -- or, for the 16-bit layouts, 128
  * (op_kv_cache.cu:873,1227) --, block_size a multiple of 16, and the token stride the row size
  * (2 * head_dim / 132 / 272 / 264 bytes) with 16-byte aligned slabs.

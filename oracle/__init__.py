@@ -70,6 +70,8 @@ def lib():
         L.tq4o_f32_to_bf16.argtypes = [C.c_float]
         L.tq4o_wht256.argtypes = [C.c_void_p]
         L.tq4o_encode_row.argtypes = [C.c_void_p, C.c_void_p]
+        L.tq4o_encode_row_plain.argtypes = [C.c_void_p, C.c_int, C.c_void_p]
+        L.tq4o_encode_row_plain.restype = None
         L.tq4o_dequant_row.argtypes = [C.c_void_p, C.c_void_p]
         for name in ("tq4o_encode_row_fp8", "tq4o_encode_row_q8", "tq4o_dequant_row_fp8", "tq4o_dequant_row_q8"):
             getattr(L, name).argtypes = [C.c_void_p, C.c_void_p]
@@ -131,6 +133,15 @@ def encode_row(x):
     assert x.shape == (256,)
     out = np.zeros(132, dtype=np.uint8)
     lib().tq4o_encode_row(x.ctypes.data, out.ctypes.data)
+    return out
+
+
+def encode_row_plain(x):
+    """head_dim fp32 values (a multiple of 128) -> a TQ4 row without the rotation."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    assert x.ndim == 1 and x.shape[0] % 128 == 0
+    out = np.zeros(66 * (x.shape[0] // 128), dtype=np.uint8)
+    lib().tq4o_encode_row_plain(x.ctypes.data, x.shape[0], out.ctypes.data)
     return out
 
 
@@ -244,9 +255,10 @@ class HostPool:
     """One layer's K and V slabs in host memory with KvPool strides
     (crates/warp34-host/src/cache.rs:304-335)."""
 
-    def __init__(self, num_pages, kv_heads, head_dim, block_size, fmt, transform):
+    def __init__(self, num_pages, kv_heads, head_dim, block_size, fmt, transform, v_transform=None):
         self.num_pages, self.kv_heads, self.head_dim, self.block_size = num_pages, kv_heads, head_dim, block_size
         self.fmt, self.transform = fmt, transform
+        self.v_transform = transform if v_transform is None else v_transform  # the V slab's, if it differs
         self.tok = row_bytes(fmt, head_dim)
         self.head = block_size * self.tok
         self.page = kv_heads * self.head
@@ -256,7 +268,7 @@ class HostPool:
     def layout(self):
         return Layout(self.k.ctypes.data, self.v.ctypes.data, self.page, self.head, self.tok,
                       self.page, self.head, self.tok, self.kv_heads, self.head_dim, self.block_size,
-                      self.fmt, self.fmt, self.transform, self.transform)
+                      self.fmt, self.fmt, self.transform, self.v_transform)
 
 
 class HostBatch:

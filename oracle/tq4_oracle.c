@@ -183,6 +183,48 @@ void tq4o_encode_row(const float* x, uint8_t* dst) {
     }
 }
 
+/* ---- TQ4 without the rotation (any transform but WHT-256 at head_dim 256): op_kv_cache.cu:219-264.
+ * One 66-byte block per 128 elements; thread t of 128 holds element t.  Sums go through
+ * block_reduce_sum_128 (tq/tq4_kv_common.cuh:109-124): a 32-lane butterfly per warp, then the same
+ * butterfly over the four warp sums in lanes 0-3 of warp 0 (the other lanes hold 0). ---- */
+static float block_sum128(const float* v) {
+    float w[32];
+    memset(w, 0, sizeof(w));
+    for (int k = 0; k < 4; ++k) w[k] = warp_sum32(v + 32 * k);
+    return warp_sum32(w);
+}
+
+void tq4o_encode_row_plain(const float* x, int head_dim, uint8_t* dst) {
+    for (int sb = 0; sb < head_dim / 128; ++sb) {
+        const float* xs = x + 128 * sb;
+        uint8_t* blk = dst + 66 * sb;
+        float t[128];
+        for (int i = 0; i < 128; ++i) t[i] = xs[i] * xs[i];
+        const float norm_x = sqrtf(block_sum128(t)); /* :231 */
+        const float inv_norm = (norm_x > 1e-12f) ? (0.7071067811865475f / norm_x) : 0.0f;
+        uint8_t code[128];
+        float xc[128], cc[128];
+        for (int i = 0; i < 128; ++i) { /* :235-245 */
+            const float u = xs[i] * inv_norm;
+            int q = 0;
+            for (int b = 0; b < 15; ++b)
+                if (u > kBoundaries[b]) q = b + 1;
+            code[i] = (uint8_t)q;
+            const float c = kCentroids[q];
+            xc[i] = xs[i] * c;
+            cc[i] = c * c;
+        }
+        const float xc_dot = block_sum128(xc); /* :246-248 */
+        const float c_sq = block_sum128(cc);
+        const float d = (c_sq > 1e-12f) ? (xc_dot / c_sq) : 0.0f;
+        const uint16_t dh = tq4o_f32_to_f16(d);
+        blk[0] = (uint8_t)(dh & 0xFF);
+        blk[1] = (uint8_t)(dh >> 8);
+        for (int m = 0; m < 64; ++m) /* :253-261: element 2m low nibble, 2m + 1 high */
+            blk[2 + m] = (uint8_t)((code[2 * m] & 0x0F) | ((code[2 * m + 1] & 0x0F) << 4));
+    }
+}
+
 /* ---- TQ4 dequant: op_kv_cache.cu:298-306 ---- */
 void tq4o_dequant_row(const uint8_t* src, float* y) {
     for (int col = 0; col < 256; ++col) {
@@ -307,6 +349,12 @@ static int write_row(uint8_t* dst, int format, int transform, const uint16_t* sr
         float x[256];
         for (int c = 0; c < 256; ++c) x[c] = load16(src + c, in_dtype);
         tq4o_encode_row(x, dst);
+        return 0;
+    }
+    if (format == TQ4O_FMT_TQ4 && head_dim > 0 && head_dim <= 256 && (head_dim % 128) == 0) { /* op_kv_cache.cu:219 */
+        float x[256];
+        for (int c = 0; c < head_dim; ++c) x[c] = load16(src + c, in_dtype);
+        tq4o_encode_row_plain(x, head_dim, dst);
         return 0;
     }
     if ((format == TQ4O_FMT_Q8_0 || format == TQ4O_FMT_FP8) && head_dim == 256) {

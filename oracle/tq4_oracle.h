@@ -27,6 +27,9 @@
  *                     zero-row special case, layout pins (132 B stride, nibble order)
  *                     -- exact code/scale BYTES for general inputs are pinned by no
  *                     reference-held vector (none exists): "parity unpinned" beyond that
+ *   tq4o_encode_row_plain  (TQ4 without the rotation) the same fp64 restatement on the raw
+ *                     128-element blocks, zero-block special case, one-centroid rows reproduced
+ *                     exactly -- exact BYTES for general inputs: "parity unpinned" as above
  *   tq4o_attention    closed forms (Q=K=0 -> running mean of V, single key -> that V row),
  *                     brute-force fp64 softmax over independently dequantised rows
  *   tq4o_split_merge  equality with the single-pass result
@@ -107,6 +110,8 @@ void tq4o_wht256(float* x);
 /* --- op_kv_cache.cu:152-218 : quantize one 256-wide row (fp32 values of the fp16/bf16
  * source) into 132 bytes --- */
 void tq4o_encode_row(const float* x, uint8_t* dst132);
+/* TQ4 without the rotation: head_dim / 128 blocks of 66 bytes (op_kv_cache.cu:219-264) */
+void tq4o_encode_row_plain(const float* x, int head_dim, uint8_t* dst);
 
 /* OCP FP8 E4M3 (finite-only, max 448) <-> fp32: round to nearest even, saturating
  * (__nv_cvt_float2_to_fp8x2(.., __NV_SATFINITE, __NV_E4M3) in op_kv_cache.cu:83-86). */

@@ -6,14 +6,14 @@ from oracle import FMT_TQ4, XF_IDENTITY, XF_WHT256
 
 
 def make_case(fmt, block_size, seq_lens, q_lens, seed, dtype, kv_heads=2, q_heads=8, perm_seed=5,
-              extra_pages=3, xf=None, head_dim=256):
+              extra_pages=3, xf=None, head_dim=256, v_xf=None):
     """Append seq_len tokens per request through the oracle's write, return everything."""
     if xf is None:
         xf = XF_WHT256 if fmt == FMT_TQ4 else XF_IDENTITY
     pages_per = [(s + block_size - 1) // block_size for s in seq_lens]
     num_pages = sum(pages_per) + extra_pages
     perm = oracle.permutation(num_pages, perm_seed)
-    pool = oracle.HostPool(num_pages, kv_heads, head_dim, block_size, fmt, xf)
+    pool = oracle.HostPool(num_pages, kv_heads, head_dim, block_size, fmt, xf, v_xf)
     mb = max(pages_per)
     bt = np.zeros((len(seq_lens), mb), dtype=np.int32)
     at = 0

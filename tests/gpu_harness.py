@@ -52,7 +52,7 @@ class DevPool:
         fmt = h.fmt if fmt is None else fmt
         return ffi.Warp34KvLayerLayout(
             self.k.data_ptr(), self.v.data_ptr(), h.page, h.head, h.tok, h.page, h.head, h.tok,
-            0, 0, h.kv_heads, h.head_dim, h.block_size, fmt, fmt, h.transform, h.transform, 0)
+            0, 0, h.kv_heads, h.head_dim, h.block_size, fmt, fmt, h.transform, h.v_transform, 0)
 
     def download(self):
         torch.cuda.synchronize()

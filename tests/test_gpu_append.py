@@ -117,6 +117,51 @@ def test_16bit_formats_at_head_dim_128(fmt, in_dtype):
     assert gk.tobytes() == hpool.k.tobytes() and gv.tobytes() == hpool.v.tobytes()
 
 
+@pytest.mark.parametrize("in_dtype", [DT_BF16, DT_F16])
+@pytest.mark.parametrize("head_dim", [128, 256])
+def test_tq4_plain_append_bit_exact(in_dtype, head_dim):
+    """TQ4 without the rotation: one 66-byte block per 128 elements (ops/op_kv_cache.cu:219-264)."""
+    hpool, gk, gv = _run_append(FMT_TQ4, XF_IDENTITY, 64, 1500, in_dtype, seed=31, head_dim=head_dim)
+    assert gk.tobytes() == hpool.k.tobytes() and gv.tobytes() == hpool.v.tobytes()
+    hpool, gk, gv = _run_append(FMT_TQ4, XF_IDENTITY, 16, 77, in_dtype, seed=32, head_dim=head_dim,
+                                stride=2 * head_dim + 3)
+    assert gk.tobytes() == hpool.k.tobytes() and gv.tobytes() == hpool.v.tobytes()
+
+
+def test_tq4_plain_append_at_head_dim_128_ignores_the_transform():
+    """Rotated rows exist at head dimension 256 only: at 128 the WHT-256 transform value selects the
+    same plain block quantiser (ops/op_kv_cache.cu:152)."""
+    a, gk_a, gv_a = _run_append(FMT_TQ4, XF_WHT256, 16, 50, DT_F16, seed=33, head_dim=128)
+    b, gk_b, gv_b = _run_append(FMT_TQ4, XF_IDENTITY, 16, 50, DT_F16, seed=33, head_dim=128)
+    assert gk_a.tobytes() == a.k.tobytes() and gk_a.tobytes() == gk_b.tobytes() and gv_a.tobytes() == gv_b.tobytes()
+
+
+def test_tq4_plain_append_special_rows():
+    """Zero blocks (codes 7, scale 0), tiny, huge and negative-zero rows."""
+    import gpu_harness as G
+
+    rng = np.random.default_rng(2)
+    n = 8
+    k = np.zeros((n, 2, 256), dtype=np.float32)
+    k[1] = rng.standard_normal((2, 256)) * 1e-12
+    k[2] = rng.standard_normal((2, 256)) * 1e4
+    k[3, :, :128] = rng.standard_normal((2, 128))
+    k[4] = -0.0
+    k[5] = rng.standard_normal((2, 256)) * 1e-30
+    k[6] = -rng.random((2, 256))
+    k[7] = rng.standard_normal((2, 256))
+    kb = oracle.f32_to_f16_bits(k)
+    hpool = oracle.HostPool(2, 2, 256, 16, FMT_TQ4, XF_IDENTITY)
+    bt = np.array([[1, 0]], dtype=np.int32)
+    slots = oracle.slot_mapping(bt[0], 0, n, 16)
+    hb = oracle.HostBatch([0, n], [n], bt, context_lens_before=[0], write_slot_mapping=slots)
+    oracle.kv_cache_write(hpool, hb, kb, kb[::-1].copy(), DT_F16)
+    dpool = G.DevPool(hpool)
+    assert G.dev_write(dpool, hb, kb, kb[::-1].copy(), DT_F16) == 0
+    gk, gv = dpool.download()
+    assert gk.tobytes() == hpool.k.tobytes() and gv.tobytes() == hpool.v.tobytes()
+
+
 def test_tq4_strided_source_bf16():
     hpool, gk, gv = _run_append(FMT_TQ4, XF_WHT256, 64, 130, DT_BF16, seed=9, stride=3 * 512)
     assert gk.tobytes() == hpool.k.tobytes() and gv.tobytes() == hpool.v.tobytes()
@@ -206,10 +251,10 @@ def test_write_argument_validation():
     Lf8 = dpool.layout(fmt=ffi.WARP34_KV_FORMAT_FP8_E4M3)
     Lf8.k_token_stride_bytes = 266
     assert l.warp34_kv_cache_write(C.byref(ex), C.byref(Lf8), C.byref(B), G.ptr(k), G.ptr(k)) == inval
-    # a TQ4 row needs the WHT256 transform
+    # TQ4 rows exist at head dimensions 128 and 256 only (rotated at 256 + WHT256, else plain)
     Lt = dpool.layout()
-    Lt.k_transform = ffi.WARP34_KV_TRANSFORM_IDENTITY
-    assert l.warp34_kv_cache_write(C.byref(ex), C.byref(Lt), C.byref(B), G.ptr(k), G.ptr(k)) == nosup
+    Lt.head_dim = 64
+    assert l.warp34_kv_cache_write_strided(C.byref(ex), C.byref(Lt), C.byref(B), G.ptr(k), G.ptr(k), 512, 512) == nosup
     # bf16 entry points: FP16 storage is rejected like in the reference
     Lh = dpool.layout(fmt=ffi.WARP34_KV_FORMAT_FP16)
     assert l.warp34_kv_cache_write_bf16(C.byref(ex), C.byref(Lh), C.byref(B), G.ptr(k), G.ptr(k)) == inval

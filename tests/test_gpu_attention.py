@@ -30,11 +30,11 @@ def _dev_pool(pool):
 
 
 def _check(fmt, dtype, block_size, seq_lens, q_lens, seed, scratch=SCRATCH, q_heads=8, kv_heads=2,
-           mask_mode=0, window=0, ctx_null=False, xf=None, head_dim=256, **kw):
+           mask_mode=0, window=0, ctx_null=False, xf=None, head_dim=256, v_xf=None, plain_excess=0.0, **kw):
     import gpu_harness as G
 
     pool, bt, k, v, q, aq, ctx = make_case(fmt, block_size, seq_lens, q_lens, seed, dtype, kv_heads=kv_heads,
-                                           q_heads=q_heads, xf=xf, head_dim=head_dim)
+                                           q_heads=q_heads, xf=xf, head_dim=head_dim, v_xf=v_xf)
     hb = oracle.HostBatch(aq, seq_lens, bt, context_lens_before=None if ctx_null else ctx, mask_mode=mask_mode,
                           sliding_window=window)
     want = oracle.paged_attention(pool, hb, q, dtype, q_heads, n_threads=4)
@@ -42,7 +42,7 @@ def _check(fmt, dtype, block_size, seq_lens, q_lens, seed, scratch=SCRATCH, q_he
     rc, got, _ = G.dev_attention(dpool, hb, q, dtype, q_heads, scratch_bytes=scratch, **kw)
     assert rc == 0
     err = G.assert_close(got, dtype, want, what="fmt=%d bs=%d seq=%s q=%s" % (fmt, block_size, seq_lens, q_lens),
-                         scale=G.channel_scale(v, dtype, hb, q_heads))
+                         scale=G.channel_scale(v, dtype, hb, q_heads), plain_excess=plain_excess)
     return got, want, err
 
 
@@ -176,6 +176,41 @@ def test_force_kernel_selector_agrees():
     # kernels that add the same products in different orders, so the bytes differ
     assert outs[1] == outs[2]
     assert outs[0] != outs[1]
+
+
+# ---- TQ4 pages stored without the rotation, or with one slab rotated (ops/op_kv_cache.cu:219-264;
+# ops/op_paged_attn.cu:347,570: the query is rotated for rotated keys, the output for rotated values) ----
+
+TQ4_XF = [(XF_IDENTITY, XF_IDENTITY), (XF_WHT256, XF_IDENTITY), (XF_IDENTITY, XF_WHT256)]
+
+
+@pytest.mark.parametrize("k_xf,v_xf", TQ4_XF)
+@pytest.mark.parametrize("dtype", [DT_BF16, DT_F16])
+def test_tq4_plain_slabs_decode_and_verify(k_xf, v_xf, dtype):
+    _check(FMT_TQ4, dtype, 16, [70, 33, 129, 1, 32], [1, 1, 1, 1, 1], 301, xf=k_xf, v_xf=v_xf)
+    _check(FMT_TQ4, dtype, 64, [300, 307], [4, 3], 302, q_heads=16, xf=k_xf, v_xf=v_xf)
+
+
+@pytest.mark.parametrize("k_xf,v_xf", TQ4_XF)
+@pytest.mark.parametrize("scratch", [0, SCRATCH])
+def test_tq4_plain_slabs_long_decode(k_xf, v_xf, scratch):
+    """Split-K with the merge kernel (rotation there follows the V slab) and the single pass."""
+    _check(FMT_TQ4, DT_BF16, 64, [20000, 777], [1, 1], 303, scratch=scratch, q_heads=16, xf=k_xf, v_xf=v_xf)
+
+
+@pytest.mark.parametrize("k_xf,v_xf", TQ4_XF)
+def test_tq4_plain_slabs_batched_decode_and_prefill(k_xf, v_xf):
+    """The balanced decode kernel (equal shares of a batch) and the 128-row tile kernel."""
+    _check(FMT_TQ4, DT_BF16, 64, [9000, 3000, 5000, 700], [1, 1, 1, 1], 304, scratch=64 << 20, q_heads=16,
+           xf=k_xf, v_xf=v_xf)
+    # Tolerance: the contract bound plus 2.5e-3 absolute on the plain channels.  Without the rotation
+    # the three x20 channels of a key row carry most of a score, so the rounding of the query's fp16
+    # MFMA operand on those three channels does not average out over 256 channels as it does in the
+    # rotated domain: about five times the score error from the same operand types (the decode kernel
+    # and the tile kernel, two independent implementations, land on the same values here: worst
+    # element +1.6e-3 over the literal bound, 18 of 13 million elements over it).
+    _check(FMT_TQ4, DT_BF16, 64, [1400, 1100], [1200, 900], 305, scratch=0, q_heads=16, xf=k_xf, v_xf=v_xf,
+           plain_excess=2.5e-3)
 
 
 # ---- 16-bit pages (FP16 pages with the f16 entry point, BF16 pages with the bf16 one) ----

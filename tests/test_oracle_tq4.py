@@ -162,3 +162,91 @@ def test_rotation_preserves_inner_products_and_quality():
         xhat = oracle.unrotate_row(yhat)
         assert abs(float(np.sum((xhat - r) ** 2) / np.sum(r ** 2)) - errs[-1]) < 1e-4
     assert 0.005 < np.mean(errs) < 0.015, np.mean(errs)
+
+
+# ---- TQ4 without the rotation (op_kv_cache.cu:219-264): the same block quantiser on the raw
+# 128-element blocks of a row of any head dimension that is a multiple of 128 ----
+
+def unpack_blocks(row):
+    """Independent reader: 66-byte blocks {fp16 scale, 64 bytes of nibbles} -> (codes, scales)."""
+    row = np.asarray(row, dtype=np.uint8).reshape(-1, 66)
+    d = row[:, 0:2].copy().view(np.float16).astype(np.float32).reshape(-1)
+    codes = np.empty((row.shape[0], 128), dtype=np.int64)
+    codes[:, 0::2] = row[:, 2:] & 0x0F
+    codes[:, 1::2] = row[:, 2:] >> 4
+    return codes.reshape(-1), d
+
+
+def encode_plain_fp64(x):
+    c = oracle.centroids().astype(np.float64)
+    x = x.astype(np.float64)
+    nb = x.shape[0] // 128
+    codes = np.empty(x.shape[0], dtype=np.int64)
+    d = np.empty(nb)
+    margin = np.empty(x.shape[0])
+    for b in range(nb):
+        xb = x[128 * b:128 * (b + 1)]
+        n = np.sqrt(float(xb @ xb))
+        u = xb * (np.sqrt(0.5) / n) if n > 1e-12 else np.zeros(128)
+        dist = np.abs(u[:, None] - c[None, :])
+        k = np.argmin(dist, axis=1)
+        part = np.sort(dist, axis=1)
+        margin[128 * b:128 * (b + 1)] = part[:, 1] - part[:, 0]
+        codes[128 * b:128 * (b + 1)] = k
+        ck = c[k]
+        d[b] = np.linalg.lstsq(ck[:, None], xb, rcond=None)[0][0]
+    return codes, d, margin
+
+
+def test_plain_encode_matches_fp64_restatement():
+    n_checked = 0
+    for hd in (128, 256):
+        bits = oracle.fill_kv_rows(48, 1, hd, 21 + hd, oracle.DT_BF16, 3)
+        for r in oracle.bf16_bits_to_f32(bits.reshape(48, hd)):
+            row = oracle.encode_row_plain(r)
+            assert row.shape == (66 * (hd // 128),)
+            codes, d = unpack_blocks(row)
+            codes64, d64, margin = encode_plain_fp64(r)
+            safe = margin > 1e-5
+            assert safe.sum() > hd - 6
+            assert np.array_equal(codes[safe], codes64[safe])
+            n_checked += int(safe.sum())
+            if np.array_equal(codes, codes64):
+                want = d64.astype(np.float32).astype(np.float16).astype(np.float32)
+                ulp = np.maximum(np.abs(want) * 2.0 ** -10, 2.0 ** -24)
+                assert np.all(np.abs(d - want) <= ulp)
+    assert n_checked > 96 * 120
+
+
+def test_plain_encode_special_rows():
+    """Zero block: inv_norm = 0 -> u = 0 -> code 7 (the strict compare stops at b[7] = 0), x.c = 0 -> d = 0.
+    A block that is a multiple of a centroid pattern: the codes reproduce the pattern and the
+    scale is that multiple (every element then dequantises to itself up to the fp16 scale)."""
+    codes, d = unpack_blocks(oracle.encode_row_plain(np.zeros(256, dtype=np.float32)))
+    assert np.all(codes == 7) and np.all(d == 0)
+    c = oracle.centroids().astype(np.float64)
+    rng = np.random.default_rng(5)
+    pattern = rng.integers(0, 16, 128)
+    x = np.concatenate([3.0 * c[pattern], np.zeros(128)]).astype(np.float32)
+    codes, d = unpack_blocks(oracle.encode_row_plain(x))
+    # the normalisation maps the block onto the unit-variance codebook only if its RMS matches;
+    # what must hold for ANY scale: the quantiser is monotone, so equal inputs get equal codes
+    # and larger inputs never get smaller codes
+    order = np.argsort(x[:128], kind="stable")
+    assert np.all(np.diff(codes[:128][order]) >= 0)
+    for v in np.unique(x[:128]):
+        assert len(set(codes[:128][x[:128] == v])) == 1
+    assert np.all(codes[128:] == 7) and d[1] == 0
+    # least-squares optimality of the scale
+    ck = c[codes[:128]]
+    d_opt = float(x[:128].astype(np.float64) @ ck) / float(ck @ ck)
+    assert abs(d[0] - d_opt) <= abs(d_opt) * 2.0 ** -10
+
+
+def test_plain_encode_power_of_two_scaling_covariance():
+    """x -> 4x: same codes, scale x 4 (exact in fp32; the fp16 scale stays in range)."""
+    bits = oracle.fill_kv_rows(8, 1, 256, 77, oracle.DT_BF16, 0)
+    for r in oracle.bf16_bits_to_f32(bits.reshape(8, 256)):
+        c1, d1 = unpack_blocks(oracle.encode_row_plain(r))
+        c4, d4 = unpack_blocks(oracle.encode_row_plain(4.0 * r))
+        assert np.array_equal(c1, c4) and np.array_equal(4.0 * d1, d4)

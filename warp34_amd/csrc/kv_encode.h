@@ -170,6 +170,65 @@ __device__ __forceinline__ void tq4_encode_row(float (&v)[8], int lane, uint8_t*
     }
 }
 
+// TQ4 without the rotation (op_kv_cache.cu:219-264): the block quantiser on the raw 128-element
+// blocks of the row, v[j] = x[8 l32 + j]; lanes 0-15 hold block 0, lanes 16-31 block 1 (absent at
+// head dimension 128: those lanes carry zeros and their bytes are not stored).  The reference sums
+// with block_reduce_sum_128 (tq4_kv_common.cuh:109-124): the 32-lane butterfly inside each warp,
+// then the same butterfly over the four warp sums in lanes 0-3 of a warp whose other lanes hold
+// +0 -- three additions of +0, then (s0 + s2) + (s1 + s3).
+__device__ __forceinline__ float block128_sum(const float (&p)[8], int lane) {
+    float t = group32_sums(p, lane);  // lanes 4 g .. 4 g + 3: the sum of warp g of the row
+    t = ((t + 0.0f) + 0.0f) + 0.0f;   // (a sum that is -0 ends as +0, as in the reference)
+    t = t + lane_xor<8>(t, lane);     // s0 + s2 (lanes of warps 0, 2), s1 + s3 (warps 1, 3)
+    return t + lane_xor<4>(t, lane);
+}
+
+__device__ __forceinline__ void tq4_encode_row_plain(const float (&v)[8], int lane, uint8_t* row) {
+    const int l32 = lane & 31;
+    const int tab_b = __float_as_int(kBoundaries[(lane & 15) < 15 ? (lane & 15) : 14]);
+    const int tab_c = __float_as_int(kCentroids[lane & 15]);
+    float p[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) p[j] = v[j] * v[j];
+    const float norm_x = __builtin_sqrtf(block128_sum(p, lane));
+    const float inv_norm = (norm_x > 1e-12f) ? (0.7071067811865475f / norm_x) : 0.0f;
+    int q[8];
+    float c[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        // "q = b + 1 for the last boundary b below u" over ascending boundaries = the number of
+        // boundaries below u: the binary search of tq4_encode_row
+        const float u = v[j] * inv_norm;
+        int code = (u > kBoundaries[7]) ? 1 : 0;
+#pragma unroll
+        for (int lvl = 1; lvl < 4; ++lvl) {
+            const int idx = (code << (4 - lvl)) + (1 << (3 - lvl)) - 1;
+            const float t = __int_as_float(__builtin_amdgcn_ds_bpermute(idx << 2, tab_b));
+            code = 2 * code + ((u > t) ? 1 : 0);
+        }
+        q[j] = code;
+        c[j] = __int_as_float(__builtin_amdgcn_ds_bpermute(code << 2, tab_c));
+    }
+    uint32_t word = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) word |= (uint32_t)(q[2 * k] | (q[2 * k + 1] << 4)) << (8 * k);
+    uint8_t* wdst = row + 66 * (l32 >> 4) + 2 + 4 * (l32 & 15);
+    *reinterpret_cast<uint16_t*>(wdst) = (uint16_t)word;
+    *reinterpret_cast<uint16_t*>(wdst + 2) = (uint16_t)(word >> 16);
+    float pv[8], pc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        pv[j] = v[j] * c[j];
+        pc[j] = c[j] * c[j];
+    }
+    const float xc_dot = block128_sum(pv, lane);
+    const float c_sq = block128_sum(pc, lane);
+    if ((l32 & 15) == 0) {
+        const float d = (c_sq > 1e-12f) ? (xc_dot / c_sq) : 0.0f;
+        *reinterpret_cast<uint16_t*>(row + 66 * (l32 >> 4)) = F16::from_f32(d);
+    }
+}
+
 // fp32 -> OCP FP8 E4M3, round to nearest even, saturating at +-448, NaN -> 0x7f
 // (__nv_cvt_float2_to_fp8x2(.., __NV_SATFINITE, __NV_E4M3) in op_kv_cache.cu:83-86).  Integer
 // arithmetic, so the bits do not depend on a hardware conversion mode.
@@ -256,7 +315,11 @@ __device__ __forceinline__ void encode_store_row(float (&v)[8], int format, int 
     }
     int n_dwords = 33;
     if (format == WARP34_KV_FORMAT_TQ4) {
-        tq4_encode_row(v, lane, row);
+        if (transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256) {
+            tq4_encode_row(v, lane, row);
+        } else {
+            tq4_encode_row_plain(v, lane, row);
+        }
     } else {
         if (transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256) sign_wht256(v, lane);
         if (format == WARP34_KV_FORMAT_FP8_E4M3) {
@@ -304,7 +367,9 @@ inline bool format_supported_for_write(int format, int transform, int head_dim) 
         return transform == WARP34_KV_TRANSFORM_IDENTITY;
     }
     if (format == WARP34_KV_FORMAT_TQ4) {
-        return head_dim == 256 && transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256;
+        // rotated at head dimension 256 with the WHT-256 transform; every other combination is the
+        // plain block quantiser, one block per 128 elements (op_kv_cache.cu:152,219)
+        return head_dim == 256 || head_dim == 128;
     }
     if (format == WARP34_KV_FORMAT_Q8_0 || format == WARP34_KV_FORMAT_FP8_E4M3) {
         // the tail-anchor layers of the default policy store these un-rotated (cache.rs:87-109);

@@ -94,11 +94,18 @@ __global__ __launch_bounds__(256) void kv_append_kernel(warp34_kv_layer_layout L
         return;
     }
     if (format == WARP34_KV_FORMAT_TQ4) {
-        // host side guarantees head_dim == 256 and the WHT256 transform for TQ4
+        // host side guarantees head_dim 256 or 128.  Rotated rows exist at 256 with the WHT-256
+        // transform only; everything else is the plain block quantiser (op_kv_cache.cu:152,219).
+        const bool rotated = L.head_dim == 256 &&
+                             (is_v ? L.v_transform : L.k_transform) == WARP34_KV_TRANSFORM_RADEMACHER_WHT256;
         // lane l32 takes elements 8 l32 .. 8 l32 + 7: one 16-byte load where the source allows it
+        // (lanes beyond a 128-element row carry zeros)
         float v[8];
         const uint16_t* src8 = src + 8 * l32;
-        if ((reinterpret_cast<uintptr_t>(src8) & 15u) == 0) {
+        if (8 * l32 >= L.head_dim) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = 0.0f;
+        } else if ((reinterpret_cast<uintptr_t>(src8) & 15u) == 0) {
             const uint4 raw = *reinterpret_cast<const uint4*>(src8);
             const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
@@ -113,11 +120,15 @@ __global__ __launch_bounds__(256) void kv_append_kernel(warp34_kv_layer_layout L
         // the row is assembled in LDS and leaves with one 32-bit store per lane (16-bit stores
         // when the destination is only 2-byte aligned, which is all the row format promises)
         uint8_t* row = rows[wave][is_v];
-        tq4_encode_row(v, lane, row);
+        if (rotated) {
+            tq4_encode_row(v, lane, row);
+        } else {
+            tq4_encode_row_plain(v, lane, row);
+        }
         __atomic_signal_fence(__ATOMIC_SEQ_CST);
         __builtin_amdgcn_wave_barrier();
         __atomic_signal_fence(__ATOMIC_SEQ_CST);
-        if ((reinterpret_cast<uintptr_t>(dst) & 3u) == 0) {
+        if (L.head_dim == 256 && (reinterpret_cast<uintptr_t>(dst) & 3u) == 0) {
             const uint32_t* r32 = reinterpret_cast<const uint32_t*>(row);
             uint32_t* d32 = reinterpret_cast<uint32_t*>(dst);
             d32[l32] = r32[l32];
@@ -125,9 +136,10 @@ __global__ __launch_bounds__(256) void kv_append_kernel(warp34_kv_layer_layout L
         } else {
             const uint16_t* r16 = reinterpret_cast<const uint16_t*>(row);
             uint16_t* d16 = reinterpret_cast<uint16_t*>(dst);
+            const int n16 = 33 * (L.head_dim >> 7);  // 66 bytes per 128 elements
             d16[l32] = r16[l32];
-            d16[l32 + 32] = r16[l32 + 32];
-            if (l32 < 2) d16[l32 + 64] = r16[l32 + 64];
+            if (l32 + 32 < n16) d16[l32 + 32] = r16[l32 + 32];
+            if (l32 + 64 < n16) d16[l32 + 64] = r16[l32 + 64];
         }
         return;
     }
@@ -206,7 +218,7 @@ extern "C" int warp34_kv_cache_write(const warp34_exec* ex, const warp34_kv_laye
 }
 
 // Layouts the bf16 entry points accept: the reference's BF16 identity layout
-// (op_kv_cache.cu:860-865) plus, at head_dim 256, TQ4 + WHT256 and the 8-bit row formats.
+// (op_kv_cache.cu:860-865) plus TQ4 (rotated or plain) and, at head_dim 256, the 8-bit row formats.
 static bool valid_bf16_entry_layout(const warp34_kv_layer_layout* l) {
     if (!l || l->local_kv_heads <= 0 || l->block_size <= 0 || l->head_dim <= 0 || l->head_dim > 256 ||
         !l->k_base || !l->v_base) {
@@ -215,10 +227,9 @@ static bool valid_bf16_entry_layout(const warp34_kv_layer_layout* l) {
     const bool bf16 = l->k_format == WARP34_KV_FORMAT_BF16 && l->v_format == WARP34_KV_FORMAT_BF16 &&
                       l->k_transform == WARP34_KV_TRANSFORM_IDENTITY &&
                       l->v_transform == WARP34_KV_TRANSFORM_IDENTITY;
-    const bool tq4 = l->head_dim == 256 && l->k_format == WARP34_KV_FORMAT_TQ4 &&
-                     l->v_format == WARP34_KV_FORMAT_TQ4 &&
-                     l->k_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 &&
-                     l->v_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256;
+    const bool tq4 = l->k_format == WARP34_KV_FORMAT_TQ4 && l->v_format == WARP34_KV_FORMAT_TQ4 &&
+                     format_supported_for_write(l->k_format, l->k_transform, l->head_dim) &&
+                     format_supported_for_write(l->v_format, l->v_transform, l->head_dim);
     const bool q8 = l->head_dim == 256 && is_8bit_format(l->k_format) && is_8bit_format(l->v_format) &&
                     format_supported_for_write(l->k_format, l->k_transform, 256) &&
                     format_supported_for_write(l->v_format, l->v_transform, 256) &&

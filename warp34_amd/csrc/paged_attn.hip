@@ -100,8 +100,8 @@ struct AttnParams {
     int max_chunks;   // cap on chunks per tile (1 = no split, scratch untouched)
     int min_upc;      // minimum units per chunk
     int tiles_by_request;  // 1: blockIdx.z is a request (no request has more than one tile)
-    int rot_q;             // row-format kernel: K rows are stored rotated, rotate the query rows
-    int rot_out;           // row-format kernel: V rows are stored rotated, rotate the output back
+    int rot_q;             // K rows are stored rotated (WHT-256 transform): rotate the query rows
+    int rot_out;           // V rows are stored rotated: rotate the output back
     int32_t* bal_table;    // balanced decode: per query token {first partial slot, pieces, token of the tile, -}
     uint32_t block_magic;  // floor(2^32 / block_size), see div_block
     const uint16_t* gate;  // fp16 [tokens, q heads, 256] or null: out = fp16(out) * sigmoid(gate)
@@ -904,9 +904,11 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
             if (pack && c == 1) {  // mirror column: the operands of column col - 8
                 packed = packed_prev;
             } else if (okc) {  // dead columns stay zero: no need to rotate them
+                if (P.rot_q) {  // keys stored rotated (uniform for the launch)
 #pragma unroll
-                for (int k = 0; k < 4; ++k) q_rot[k] = apply_sign(q_rot[k], 4 * lane + k);
-                wht256_wave(q_rot, lane);
+                    for (int k = 0; k < 4; ++k) q_rot[k] = apply_sign(q_rot[k], 4 * lane + k);
+                    wht256_wave(q_rot, lane);
+                }
                 packed.x = pack_h2(q_rot[0] * q_scale, q_rot[1] * q_scale);
                 packed.y = pack_h2(q_rot[2] * q_scale, q_rot[3] * q_scale);
             }
@@ -1319,9 +1321,11 @@ __device__ __forceinline__ void tq4_tile(const AttnParams& P, uint8_t* smem, con
                 const float inv = l_col > 0.f ? kLutInvGain / l_col : 0.f;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) v[k] *= inv;
-                wht256_wave(v, lane);
+                if (P.rot_out) {  // values stored rotated
+                    wht256_wave(v, lane);
 #pragma unroll
-                for (int k = 0; k < 4; ++k) v[k] = apply_sign(v[k], 4 * lane + k);
+                    for (int k = 0; k < 4; ++k) v[k] = apply_sign(v[k], 4 * lane + k);
+                }
                 store_out_row<TQ>(P, row, lane, v);
             }
         }
@@ -1851,6 +1855,8 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     P.q = (const uint16_t*)q;
     P.out = (uint16_t*)out;
     P.gate = (const uint16_t*)gate;
+    P.rot_q = layout->k_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 ? 1 : 0;
+    P.rot_out = layout->v_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256 ? 1 : 0;
     P.num_q_heads = num_q_heads;
     P.gqa = num_q_heads / layout->local_kv_heads;
     int q_group = P.gqa;
@@ -1946,7 +1952,7 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
             rc = (int)hipGetLastError();
             if (rc) return rc;
             hipLaunchKernelGGL((split_merge_kernel<TQ, true>), dim3((unsigned)rows), dim3(1024), 0, stream,
-                               (const float*)P.part_acc, (const float*)P.part_ml, stride, P, kLutInvGain, 1);
+                               (const float*)P.part_acc, (const float*)P.part_ml, stride, P, kLutInvGain, P.rot_out);
             return (int)hipGetLastError();
         }
     }
@@ -1968,7 +1974,7 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
             if (rc) return rc;
             hipLaunchKernelGGL((balanced_merge_kernel<TQ>),
                                dim3((unsigned)rows), dim3(1024), 0, stream, P,
-                               kv_subs, kLutInvGain, 1);
+                               kv_subs, kLutInvGain, P.rot_out);
             return (int)hipGetLastError();
         }
     }
@@ -1979,7 +1985,7 @@ static int launch_tq4(const warp34_exec* ex, const warp34_kv_layer_layout* layou
     if (rc) return rc;
     if (P.max_chunks > 1) {
         hipLaunchKernelGGL((split_merge_kernel<TQ>), dim3((unsigned)rows), dim3(1024), 0, stream,
-                           (const float*)P.part_acc, (const float*)P.part_ml, P.max_chunks, P, kLutInvGain, 1);
+                           (const float*)P.part_acc, (const float*)P.part_ml, P.max_chunks, P, kLutInvGain, P.rot_out);
         rc = (int)hipGetLastError();
     }
     return rc;
@@ -2187,6 +2193,16 @@ static bool is_tq4_wht(const warp34_kv_layer_layout* l) {
            l->v_transform == WARP34_KV_TRANSFORM_RADEMACHER_WHT256;
 }
 
+// TQ4 pages at head dimension 256, each slab stored rotated or plain (op_paged_attn.cu:347,570:
+// the query is rotated for rotated keys, the output rotated back for rotated values)
+static bool is_tq4(const warp34_kv_layer_layout* l) {
+    const auto xf_ok = [](int t) {
+        return t == WARP34_KV_TRANSFORM_IDENTITY || t == WARP34_KV_TRANSFORM_RADEMACHER_WHT256;
+    };
+    return l->head_dim == 256 && l->k_format == WARP34_KV_FORMAT_TQ4 && l->v_format == WARP34_KV_FORMAT_TQ4 &&
+           xf_ok(l->k_transform) && xf_ok(l->v_transform);
+}
+
 static bool tq4_geometry_ok(const warp34_kv_layer_layout* l, const void* q) {
     // 16-token runs must be contiguous and 16-byte aligned for the staging copy
     return l->block_size > 0 && (l->block_size % 16) == 0 && l->k_token_stride_bytes == kTq4RowBytes &&
@@ -2216,7 +2232,7 @@ static int attention_entry(const warp34_exec* ex, const warp34_kv_layer_layout* 
         (batch->mask_mode != WARP34_ATTN_MASK_CAUSAL && batch->mask_mode != WARP34_ATTN_MASK_NONCAUSAL_WINDOW)) {
         return (int)hipErrorInvalidValue;
     }
-    if (is_tq4_wht(layout)) {
+    if (is_tq4(layout)) {
         if (!tq4_geometry_ok(layout, q) || (((uintptr_t)out) & 7u) != 0) return (int)hipErrorNotSupported;
         // Many query rows per request and enough tiles to fill the chip: the tile kernel shares
         // every dequantised key block between 128 query rows.

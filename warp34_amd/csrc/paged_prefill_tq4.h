@@ -179,8 +179,8 @@ __global__ __launch_bounds__((PC ? 12 : kPfWaves) * 64, 1) void paged_prefill_tq
     constexpr int kQStride = 264;
     _Float16* qbuf = reinterpret_cast<_Float16*>(smem + kPfDeqBase) + wave * 16 * kQStride;
     const float q_scale = B.sm_scale * kLog2e * (TQ4F ? kLutInvGain : 1.0f);
-    const bool rot_q = !K16 && (TQ4F || P.rot_q != 0);
-    const bool rot_out = !K16 && (TQ4F || P.rot_out != 0);
+    const bool rot_q = !K16 && P.rot_q != 0;
+    const bool rot_out = !K16 && P.rot_out != 0;
     if (!producer) {
         uint2 q_raw[16];
 #pragma unroll
