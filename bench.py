@@ -66,20 +66,20 @@ WORKLOADS = {
 # be read from inside this process, so workloads without such a profile report null.
 PROFILED_TRAFFIC = {
     # workload: (HBM bytes per launch of the dominant kernel, the profile that holds the counter readings)
-    "tq4_decode_b1_ctx131072": (71_840_000, "profiles/paged_attn_tq4_decode_b1_ctx131072.txt"),
-    "tq4_decode_b8_ctx131072": (559_930_000, "profiles/paged_attn_tq4_decode_b8_ctx131072.txt"),
-    "tq4_decode_b32_ctx1k_64k": (587_130_000, "profiles/paged_attn_tq4_decode_b32_ctx1k_64k.txt"),
-    "bf16_decode_b1_ctx32768": (69_530_000, "profiles/paged_attn_rows_bf16_decode_b1_ctx32768.txt"),
-    "fp8_decode_b32_ctx1k_64k": (1_190_030_000, "profiles/paged_attn_rows_fp8_decode_b32_ctx1k_64k.txt"),
-    "fp8_decode_b1_ctx131072": (142_320_000, "profiles/paged_attn_rows_fp8_decode_b1_ctx131072.txt"),
-    "q8_0_decode_b1_ctx131072": (145_360_000, "profiles/paged_attn_rows_q8_0_decode_b1_ctx131072.txt"),
-    # (the four kernels of the shared-prefix path together: probe 0.27 + tile 144.84 + decode 534.73 + merge 39.06 MB)
-    "tq4_verify_16x4_ctx262144_shared200k": (718_900_000, "profiles/paged_attn_tq4_verify_16x4_ctx262144_shared200k.txt"),
-    "tq4_prefill_8x2048_ctx16384": (1_126_470_000, "profiles/paged_prefill_tq4_8x2048_ctx16384.txt"),
+    "tq4_decode_b1_ctx131072": (71_820_000, "profiles/paged_attn_tq4_decode_b1_ctx131072.txt"),
+    "tq4_decode_b8_ctx131072": (559_960_000, "profiles/paged_attn_tq4_decode_b8_ctx131072.txt"),
+    "tq4_decode_b32_ctx1k_64k": (587_160_000, "profiles/paged_attn_tq4_decode_b32_ctx1k_64k.txt"),
+    "bf16_decode_b1_ctx32768": (69_520_000, "profiles/paged_attn_rows_bf16_decode_b1_ctx32768.txt"),
+    "fp8_decode_b32_ctx1k_64k": (1_190_120_000, "profiles/paged_attn_rows_fp8_decode_b32_ctx1k_64k.txt"),
+    "fp8_decode_b1_ctx131072": (142_290_000, "profiles/paged_attn_rows_fp8_decode_b1_ctx131072.txt"),
+    "q8_0_decode_b1_ctx131072": (145_300_000, "profiles/paged_attn_rows_q8_0_decode_b1_ctx131072.txt"),
+    # (the four kernels of the shared-prefix path together: probe 0.27 + tile 144.84 + decode 534.98 + merge 39.06 MB)
+    "tq4_verify_16x4_ctx262144_shared200k": (719_150_000, "profiles/paged_attn_tq4_verify_16x4_ctx262144_shared200k.txt"),
+    "tq4_prefill_8x2048_ctx16384": (1_119_610_000, "profiles/paged_prefill_tq4_8x2048_ctx16384.txt"),
     "tq4_qsa_sparse_16x513_ctx131072": (23_400_000, "profiles/qsa_sparse_tq4_16x513_ctx131072.txt"),
-    "tq4_norm_rope_append_8192": (183_290_000, "profiles/qk_norm_rope_tq4_append_8192.txt"),
-    "tq4_fused_qk_gate_append_8192": (289_030_000, "profiles/fused_qk_norm_rope_gate_tq4_append_8192.txt"),
-    "tq4_append_4096": (10_870_000, "profiles/kv_append_tq4_4096.txt"),
+    "tq4_norm_rope_append_8192": (182_920_000, "profiles/qk_norm_rope_tq4_append_8192.txt"),
+    "tq4_fused_qk_gate_append_8192": (289_660_000, "profiles/fused_qk_norm_rope_gate_tq4_append_8192.txt"),
+    "tq4_append_4096": (10_880_000, "profiles/kv_append_tq4_4096.txt"),
 }
 SHARED_PREFIX = {"tq4_verify_16x4_ctx262144_shared200k": 200000}
 VERIFY_Q = {"tq4_verify_16x4_ctx262144_shared200k": 4}
