@@ -14,9 +14,9 @@
 //           scratch size -- never on max_seq_len, max_blocks_per_req, physical page numbers or
 //           local_kv_heads -- so outputs are bit-identical under page permutation, graph-bucket
 //           bounds and head sharding (tests/tq4_vision_and_moe.rs:1089-1663).
-//   unit  = 32 consecutive tokens handled by ONE wave start to finish: the wave copies the
-//           raw K and V rows of the unit into its private LDS area (coalesced 16-byte loads
-//           from a wave-uniform base, next unit prefetched into registers), forms
+//   unit  = 32 consecutive tokens handled by ONE wave start to finish: the raw K and V rows of
+//           the unit go straight from the pages into the wave's private LDS area (LDS-direct
+//           16-byte loads from a wave-uniform base, one unit ahead), the wave forms
 //           S^T = K Q'^T with MFMA, does the online softmax in registers and accumulates
 //           O^T += V^T P^T with MFMA.  Waves never synchronise inside the key loop; their
 //           (m, l, O) states are merged once at the end.
@@ -52,9 +52,9 @@ typedef float f2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u2v __attribute__((ext_vector_type(2)));
 
-// waves per workgroup of the TQ4 decode kernel: ten (SIMDs 0 and 1 run three, SIMDs 2 and 3 two),
-// which caps a wave at 168 registers and is what the LDS holds: table + 10 staging areas + the
-// query operand table = 159 232 of 163 840 bytes
+// waves per workgroup of the TQ4 decode kernel: eight, two per SIMD (up to 256 registers each); the
+// LDS holds the table, eight staging areas, the query operand table and the (m, l) tables:
+// 142 KB of 160 KB, one workgroup per CU
 constexpr int kTq4Waves = 8;
 __host__ __device__ constexpr int waves_for(int nt) { return nt == 1 ? kTq4Waves : 4; }
 constexpr int kUnit = 32;             // tokens per wave iteration
