@@ -127,7 +127,7 @@ def _dev_fused_write(dpool, qg, k, v, qw, kw, pos, slots, qh, kh, hd, rot, mask=
     return rc, [d[x].cpu().numpy().view(np.uint16) for x in ("q", "ko", "g")]
 
 
-@pytest.mark.parametrize("fmt,xf", [(FMT_TQ4, XF_WHT256), (FMT_FP8, XF_WHT256), (FMT_Q8_0, XF_WHT256),
+@pytest.mark.parametrize("fmt,xf", [(FMT_TQ4, XF_WHT256), (FMT_TQ4, XF_IDENTITY), (FMT_FP8, XF_WHT256), (FMT_Q8_0, XF_WHT256),
                                     (FMT_FP8, XF_IDENTITY), (FMT_Q8_0, XF_IDENTITY), (FMT_FP16, XF_IDENTITY)])
 @pytest.mark.parametrize("with_k_out", [True, False])
 def test_fused_append_equals_operator_then_append(fmt, xf, with_k_out):

@@ -85,7 +85,7 @@ def test_operator_q_out_bit_exact():
     assert (got[:, :q_heads * dim] == qkv[:, :q_heads * dim]).all()  # packed Q untouched
 
 
-@pytest.mark.parametrize("fmt,xf", [(FMT_BF16, XF_IDENTITY), (FMT_TQ4, XF_WHT256), (FMT_FP8, XF_IDENTITY),
+@pytest.mark.parametrize("fmt,xf", [(FMT_BF16, XF_IDENTITY), (FMT_TQ4, XF_WHT256), (FMT_TQ4, XF_IDENTITY), (FMT_FP8, XF_IDENTITY),
                                     (FMT_Q8_0, XF_IDENTITY), (FMT_FP8, XF_WHT256), (FMT_Q8_0, XF_WHT256)])
 def test_fused_kv_write_bit_exact_and_equal_to_operator_then_append(fmt, xf):
     import gpu_harness as G
